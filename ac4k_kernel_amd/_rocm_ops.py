@@ -1,0 +1,170 @@
+"""Tensor-level binding over the C ABI: the module the reference's package would import as
+`ac4k_kernel._rocm_ops` (python/ac4k_kernel/__init__.py:39-48), with the function names and
+positional arguments of `_cuda_ops` (lib/cuda_bindings.cc:64-85, include/ac4k_kernel/ops.h:27-48).
+
+All functions write into caller-provided tensors, return None, enqueue on the current
+torch stream and never synchronise.  Argument checks mirror the reference host launchers'
+TORCH_CHECKs and raise RuntimeError.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_L = _lib.load()
+
+__arch__ = _L.ac4k_arch().decode()
+__arch_description__ = _L.ac4k_arch_description().decode()
+__backend__ = _L.ac4k_backend().decode()
+__version__ = _L.ac4k_version().decode()
+
+_DTYPE_TAG = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _check_tensor(t, dtype, name: str) -> None:
+    _check(isinstance(t, torch.Tensor), f"{name} must be a tensor")
+    _check(t.is_cuda, f"{name} must be a CUDA tensor")
+    _check(t.is_contiguous(), f"{name} must be contiguous")
+    _check(t.dtype == dtype, f"Inconsistency of Tensor type: {name} must be {dtype}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _align_up(a: int, b: int) -> int:
+    return (a + b - 1) // b * b
+
+
+def _quant_geometry(inp: torch.Tensor, cross_dim: int, reduce_dim: int):
+    """Checks shared by the three quantizers (quantize_nvfp4.cu:171-190,226-241)."""
+    _check_tensor(inp, torch.bfloat16, "in")
+    _check(2 <= inp.dim() <= 4, "in must be 2-4D")
+    _check(0 <= cross_dim < inp.dim(), "cross_dim must be less than in.dim()")
+    _check(0 <= reduce_dim < inp.dim(), "reduce_dim must be less than in.dim()")
+    _check(cross_dim != reduce_dim, "cross_dim and reduce_dim must be different")
+    shape, stride = list(inp.shape), list(inp.stride())
+    lead = [i for i in range(inp.dim()) if i not in (cross_dim, reduce_dim)]
+    lead_shape = [shape[i] for i in lead]
+    ld = [(shape[i], stride[i]) for i in lead]
+    while len(ld) < 2:
+        ld.insert(0, (1, 0))
+    (d0, s0), (d1, s1) = ld
+    _check(inp.numel() > 0, "in must not be empty")
+    return lead_shape, (d0, d1, shape[cross_dim], shape[reduce_dim], s0, s1, stride[cross_dim], stride[reduce_dim])
+
+
+def global_scale(out: torch.Tensor, inp: torch.Tensor, max_scale: float) -> None:
+    """out (0-dim fp32) = amax(|inp|) / max_scale  (python/ac4k_kernel/ops/quant.py:33-59)."""
+    _check_tensor(inp, torch.bfloat16, "in")
+    _check_tensor(out, torch.float32, "global_scale")
+    _check(out.dim() == 0, "global_scale must be a scalar")
+    _lib.check(_L.ac4k_global_scale_bf16(out.data_ptr(), inp.data_ptr(), inp.numel(), float(max_scale), _stream()))
+
+
+def quantize_nvfp4(out, sf, inp, global_scale, cross_dim: int, reduce_dim: int, swizzle: bool) -> None:
+    lead_shape, geom = _quant_geometry(inp, cross_dim, reduce_dim)
+    R, K = geom[2], geom[3]
+    _check_tensor(global_scale, torch.float32, "global_scale")
+    _check(global_scale.dim() == 0, "global_scale must be a scalar")
+    _check_tensor(out, torch.uint8, "out")
+    _check(list(out.shape) == lead_shape + [R, _align_up(K, 64) // 2],
+           "out must have shape [.., cross, align_up(reduce, 64) / 2]")
+    _check_tensor(sf, torch.float8_e4m3fn, "sf")
+    _check(list(sf.shape) == lead_shape + [_align_up(K, 64) // 64, _align_up(R, 16), 4], "meet invalid sf shape")
+    _lib.check(_L.ac4k_quantize_nvfp4(out.data_ptr(), sf.data_ptr(), inp.data_ptr(), global_scale.data_ptr(),
+                                      *geom, int(bool(swizzle)), _stream()))
+
+
+def _quantize_rowwise(fn, out, out_dtype, sf, inp, scale_max, scale_dtype, cross_dim, reduce_dim, *extra):
+    lead_shape, geom = _quant_geometry(inp, cross_dim, reduce_dim)
+    R, K = geom[2], geom[3]
+    _check_tensor(scale_max, scale_dtype, "scale_max")
+    _check(scale_max.dim() == 0, "scale_max must be a scalar")
+    _check_tensor(out, out_dtype, "out")
+    _check(list(out.shape) == lead_shape + [R, _align_up(K, 16)], "out must have shape [.., cross, align_up(reduce, 16)]")
+    _check_tensor(sf, torch.float32, "sf")
+    _check(list(sf.shape) == lead_shape + [_align_up(R, 16)], "meet invalid sf shape")
+    _lib.check(fn(out.data_ptr(), sf.data_ptr(), inp.data_ptr(), scale_max.data_ptr(), *geom, *extra, _stream()))
+
+
+def quantize_fp8(out, sf, inp, scale_max, cross_dim: int, reduce_dim: int, swizzle: bool) -> None:
+    _quantize_rowwise(_L.ac4k_quantize_fp8, out, torch.float8_e4m3fn, sf, inp, scale_max, torch.float32,
+                      cross_dim, reduce_dim, int(bool(swizzle)))
+
+
+def quantize_int8(out, sf, inp, scale_max, cross_dim: int, reduce_dim: int) -> None:
+    _quantize_rowwise(_L.ac4k_quantize_int8, out, torch.int8, sf, inp, scale_max, torch.int32,
+                      cross_dim, reduce_dim)
+
+
+def _check_linear_operand(x, x_sf, x_gs, rows, name):
+    _check(x.dim() == 2, f"{name} must be a 2d matrix")
+    _check_tensor(x, torch.uint8, name)
+    K = x.size(1) * 2
+    _check(x_sf.dim() == 3, f"scale_{name} must be a 3d matrix")
+    _check_tensor(x_sf, torch.float8_e4m3fn, f"scale_{name}")
+    _check(list(x_sf.shape) == [(K + 63) // 64, _align_up(rows, 16), 4], f"scale_{name} has an invalid shape")
+    _check_tensor(x_gs, torch.float32, f"global_scale_{name}")
+    _check(x_gs.dim() == 0, f"{name}_global_scale must be a scalar")
+    return K
+
+
+def linear_nvfp4(D, A, A_sf, A_global_scale, B, B_sf, B_global_scale, bias=None) -> None:
+    """Checks of linear_nvfp4.cu:759-805."""
+    _check(isinstance(D, torch.Tensor) and D.dim() == 2, "d must be a 2d matrix")
+    _check(D.dtype in _DTYPE_TAG, "d must be bfloat16, half or float")
+    _check(D.is_cuda and D.is_contiguous(), "d must be contiguous")
+    M, N = D.shape
+    _check(A.dim() == 2 and A.size(0) == M, f"A size(0) must be {M}")
+    K = _check_linear_operand(A, A_sf, A_global_scale, M, "a")
+    _check(K % 16 == 0, f"A size(1)*2 must be multiple of 16 but see {K}")
+    _check(B.dim() == 2 and B.size(1) == A.size(1), "B size(1) must equal A size(1)")
+    _check(B.size(0) == N, f"B size(0) must be {N}")
+    _check_linear_operand(B, B_sf, B_global_scale, N, "b")
+    bias_ptr, bias_tag = None, 0
+    if bias is not None:
+        _check(bias.dtype in _DTYPE_TAG, "bias must be bfloat16, half or float")
+        _check(bias.is_cuda and bias.is_contiguous(), "bias must be contiguous")
+        _check(bias.dim() == 2, "bias must be a 2d matrix")
+        _check(bias.size(0) == 1, "bias shape[0] must be 1")
+        _check(bias.size(1) == N, f"bias shape[1] must be {N}")
+        bias_ptr, bias_tag = bias.data_ptr(), _DTYPE_TAG[bias.dtype]
+    if M == 0 or N == 0:
+        return
+    _lib.check(_L.ac4k_linear_nvfp4(D.data_ptr(), _DTYPE_TAG[D.dtype], A.data_ptr(), A_sf.data_ptr(),
+                                    A_global_scale.data_ptr(), B.data_ptr(), B_sf.data_ptr(),
+                                    B_global_scale.data_ptr(), bias_ptr, bias_tag, M, N, K, _stream()))
+
+
+def linear_nvfp4_fused(D, X, X_q, X_sf, X_global_scale, B, B_sf, B_global_scale, bias=None) -> None:
+    """quantize(X, 0, 1) + linear_nvfp4 in one call for 1 <= M <= 32; X_q / X_sf / X_global_scale
+    receive the quantized activation."""
+    _check(isinstance(D, torch.Tensor) and D.dim() == 2, "d must be a 2d matrix")
+    _check(D.dtype in _DTYPE_TAG, "d must be bfloat16, half or float")
+    _check(D.is_cuda and D.is_contiguous(), "d must be contiguous")
+    M, N = D.shape
+    _check_tensor(X, torch.bfloat16, "x")
+    _check(X.dim() == 2 and X.size(0) == M, f"x must be [{M}, K]")
+    K = X.size(1)
+    _check(K % 64 == 0, "K must be a multiple of 64")
+    _check_tensor(X_q, torch.uint8, "x_q")
+    _check(list(X_q.shape) == [M, K // 2], "x_q must be [M, K/2]")
+    _check_linear_operand(X_q, X_sf, X_global_scale, M, "x")
+    _check(B.dim() == 2 and B.size(0) == N and B.size(1) == K // 2, "weight must be [N, K/2]")
+    _check_linear_operand(B, B_sf, B_global_scale, N, "b")
+    bias_ptr, bias_tag = None, 0
+    if bias is not None:
+        _check(bias.dtype in _DTYPE_TAG, "bias must be bfloat16, half or float")
+        _check(bias.is_cuda and bias.is_contiguous() and list(bias.shape) == [1, N], f"bias must be [1, {N}]")
+        bias_ptr, bias_tag = bias.data_ptr(), _DTYPE_TAG[bias.dtype]
+    _lib.check(_L.ac4k_linear_nvfp4_fused_bf16(D.data_ptr(), _DTYPE_TAG[D.dtype], X.data_ptr(), X_q.data_ptr(),
+                                               X_sf.data_ptr(), X_global_scale.data_ptr(), B.data_ptr(),
+                                               B_sf.data_ptr(), B_global_scale.data_ptr(), bias_ptr, bias_tag,
+                                               M, N, K, _stream()))

@@ -1,0 +1,456 @@
+// BF16 -> NVFP4 / FP8E4M3 / INT8 quantizers and the global-scale reduction for gfx950.
+//
+// Arithmetic follows the reference kernels' operation order in IEEE round-to-nearest fp32:
+//   global scale  python/ac4k_kernel/ops/quant.py:33-59
+//   nvfp4         lib/cuda/sm120/quantize_nvfp4.cu:49-157
+//   fp8 per row   lib/cuda/sm120/quantize_fp8.cu:57-185
+//   int8 per row  lib/cuda/sm120/quantize_int8.cu:61-168
+// The reference's rcp.approx / fast-math divisions are replaced by correctly rounded
+// divisions, and the file is compiled with -ffp-contract=off so that the separate
+// multiplies of the spec stay separate.
+//
+// All kernels are bandwidth-bound: the row-major paths move 16 bytes per lane per load,
+// reduce amax inside the wavefront with DPP, and store packed words.
+#include "ac4k_common.h"
+
+namespace ac4k {
+
+// ===========================================================================
+// global scale:  *gs = fp32(max |x|) / max_scale
+// ===========================================================================
+
+__global__ void zero_u32_kernel(uint32_t *p) { *p = 0u; }
+
+constexpr int AMAX_THREADS = 256;
+constexpr int AMAX_UNROLL = 4;
+
+__global__ __launch_bounds__(AMAX_THREADS) void amax_scale_bf16_kernel(
+    uint32_t *__restrict__ gs_bits, const uint16_t *__restrict__ x, int64_t n, int64_t head,
+    int64_t nvec, float max_scale) {
+  // x[0..head) and the tail after the vectors are handled by scalar loads of block 0;
+  // the 16-byte aligned middle is streamed with grid-stride uint4 loads.
+  const uint4 *xv = reinterpret_cast<const uint4 *>(x + head);
+  uint32_t m = 0;
+  const int64_t stride = (int64_t)gridDim.x * AMAX_THREADS;
+  int64_t i = (int64_t)blockIdx.x * AMAX_THREADS + threadIdx.x;
+  for (; i + (AMAX_UNROLL - 1) * stride < nvec; i += AMAX_UNROLL * stride) {
+    uint4 v[AMAX_UNROLL];
+#pragma unroll
+    for (int u = 0; u < AMAX_UNROLL; ++u) v[u] = ld_stream_u4(xv + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < AMAX_UNROLL; ++u) m = umax32(m, absmax_bf16x8(v[u]));
+  }
+  for (; i < nvec; i += stride) m = umax32(m, absmax_bf16x8(xv[i]));
+  if (blockIdx.x == 0) {
+    for (int64_t j = threadIdx.x; j < head; j += AMAX_THREADS) m = umax32(m, x[j] & 0x7fffu);
+    for (int64_t j = head + nvec * 8 + threadIdx.x; j < n; j += AMAX_THREADS)
+      m = umax32(m, x[j] & 0x7fffu);
+  }
+  m = group_umax<64>(m);
+  __shared__ uint32_t part[AMAX_THREADS / 64];
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int w = 1; w < AMAX_THREADS / 64; ++w) m = umax32(m, part[w]);
+    // division is monotone, so the max of the per-block quotients is the quotient of the
+    // max; non-negative floats order like unsigned integers.
+    float q = bf16_bits_to_f32(m) / max_scale;
+    if (q > 0.0f || q != q) atomicMax(gs_bits, __float_as_uint(q));
+  }
+}
+
+// ===========================================================================
+// nvfp4
+// ===========================================================================
+
+struct QuantGeom {
+  int64_t d1, R, K, Kp, Rp;
+  int64_t s0, s1, sR, sK;
+};
+
+// One 16-block given 16 floats already in output order.  Returns the e4m3 code.
+__device__ __forceinline__ float nvfp4_block_scale(float amax, float alpha, uint32_t &code) {
+  float s32 = alpha * (amax * 0.16666666666666666f);
+  code = f32_to_ue4m3_satfinite(s32);
+  float s = e4m3_to_f32(code);
+  return (s != 0.0f) ? alpha * (1.0f / s) : 0.0f;
+}
+
+__device__ __forceinline__ uint32_t nvfp4_pack8(uint4 v, float o) {
+  float f[8] = {bf16_lo(v.x) * o, bf16_hi(v.x) * o, bf16_lo(v.y) * o, bf16_hi(v.y) * o,
+                bf16_lo(v.z) * o, bf16_hi(v.z) * o, bf16_lo(v.w) * o, bf16_hi(v.w) * o};
+  return f32x8_to_e2m1x8(f);
+}
+
+// Row-major fast path: reduce dim contiguous, no swizzle, K % 8 == 0, 16-byte aligned rows.
+// A lane owns 8 consecutive elements (half a 16-block); lane pairs share the block amax
+// through one DPP quad_perm; the four scale bytes of a 64-chunk are gathered into the
+// chunk's first lane with three DPP row shifts and stored as one dword.
+//   CPR  = 64-element chunks per wave row (8*CPR lanes per row, 8/CPR rows per wave pass)
+//   ITER = wave passes per workgroup (independent loads in flight per lane)
+template <int CPR, int ITER>
+__global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
+    uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in,
+    const float *__restrict__ global_scale, QuantGeom g) {
+  constexpr int LPR = 8 * CPR;   // lanes per row
+  constexpr int RW = 64 / LPR;   // rows per wave pass
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t lead = blockIdx.y;
+  const int64_t ngroups = ceil_div(g.Kp / 64, CPR);  // chunk groups along the reduce dim
+  const int64_t k = ((int64_t)(blockIdx.x % ngroups) * LPR + (lane % LPR)) * 8;
+  const int64_t row0 = (int64_t)(blockIdx.x / ngroups) * (4 * RW * ITER) + lane / LPR;
+  if (k >= g.Kp) return;
+  const float alpha = 1.0f / *global_scale;
+  const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + k;
+  const bool kvalid = k < g.K;
+
+  uint4 v[ITER];
+#pragma unroll
+  for (int it = 0; it < ITER; ++it) {
+    const int64_t r = row0 + (int64_t)(it * 4 + wave) * RW;
+    v[it] = make_uint4(0, 0, 0, 0);
+    if (kvalid && r < g.R)
+      v[it] = ld_stream_u4(src + r * g.sR);
+  }
+#pragma unroll
+  for (int it = 0; it < ITER; ++it) {
+    const int64_t r = row0 + (int64_t)(it * 4 + wave) * RW;
+    uint32_t m = absmax_bf16x8(v[it]);
+    m = umax32(m, dpp_u32<DPP_QUAD_XOR1>(m));
+    uint32_t code;
+    float o = nvfp4_block_scale(bf16_bits_to_f32(m), alpha, code);
+    if (r >= g.R) code = 0;  // pad rows carry zero scales
+    uint32_t packed = nvfp4_pack8(v[it], o);
+    uint32_t sfw = code | (dpp_u32<DPP_ROW_SHL(2)>(code) << 8) | (dpp_u32<DPP_ROW_SHL(4)>(code) << 16) |
+                   (dpp_u32<DPP_ROW_SHL(6)>(code) << 24);
+    if (r < g.R)
+      st_stream_u1(out + (lead * g.R + r) * (g.Kp / 2) + k / 2, packed);
+    if ((lane & 7) == 0 && r < g.Rp)
+      reinterpret_cast<uint32_t *>(sf)[(lead * (g.Kp / 64) + k / 64) * g.Rp + r] = sfw;
+  }
+}
+
+// Generic path: any strides, optional swizzle.  One lane owns one (row, 64-chunk): it reads
+// its 64 elements with scalar loads (coalesced across lanes when the cross dim is the
+// contiguous one), and writes 32 packed bytes and one scale dword.
+template <bool SWIZZLE>
+__global__ __launch_bounds__(256) void quantize_nvfp4_generic_kernel(
+    uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in,
+    const float *__restrict__ global_scale, QuantGeom g) {
+  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t chunk = blockIdx.y, lead = blockIdx.z;
+  if (r >= g.Rp) return;
+  uint32_t *sfp = reinterpret_cast<uint32_t *>(sf) + (lead * (g.Kp / 64) + chunk) * g.Rp + r;
+  if (r >= g.R) {
+    *sfp = 0u;
+    return;
+  }
+  const float alpha = 1.0f / *global_scale;
+  const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + r * g.sR;
+  uint32_t sfw = 0;
+  uint32_t *op = reinterpret_cast<uint32_t *>(out + (lead * g.R + r) * (g.Kp / 2) + chunk * 32);
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    uint32_t h[16];
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      int p = b * 16 + i;  // position inside the 64-chunk, output order
+      if (SWIZZLE) {
+        int q32 = p & 31;
+        p = (p & 32) + ((q32 & 7) >> 1) * 8 + (q32 >> 3) * 2 + (q32 & 1);
+      }
+      const int64_t kk = chunk * 64 + p;
+      h[i] = kk < g.K ? (uint32_t)src[kk * g.sK] : 0u;
+      m = umax32(m, h[i] & 0x7fffu);
+    }
+    uint32_t code;
+    float o = nvfp4_block_scale(bf16_bits_to_f32(m), alpha, code);
+    sfw |= code << (8 * b);
+    float f0[8], f1[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      f0[i] = bf16_bits_to_f32(h[i]) * o;
+      f1[i] = bf16_bits_to_f32(h[8 + i]) * o;
+    }
+    op[2 * b] = f32x8_to_e2m1x8(f0);
+    op[2 * b + 1] = f32x8_to_e2m1x8(f1);
+  }
+  *sfp = sfw;
+}
+
+// ===========================================================================
+// per-row fp8 / int8
+// ===========================================================================
+
+enum class RowFmt { FP8, INT8 };
+
+// scale_max is a device scalar: fp32 for fp8 (quantize_fp8.cu:205), int32 for int8
+// (quantize_int8.cu:189), converted to float where it is used (:127,135).
+template <RowFmt FMT>
+__device__ __forceinline__ float load_scale_max(const void *p) {
+  return FMT == RowFmt::FP8 ? *static_cast<const float *>(p) : (float)*static_cast<const int32_t *>(p);
+}
+
+// satfinite e4m3 of four floats -> four bytes, element 0 in the low byte.
+__device__ __forceinline__ uint32_t f32x4_to_e4m3x4(float a, float b, float c, float d) {
+  a = __builtin_amdgcn_fmed3f(a, -448.0f, 448.0f);
+  b = __builtin_amdgcn_fmed3f(b, -448.0f, 448.0f);
+  c = __builtin_amdgcn_fmed3f(c, -448.0f, 448.0f);
+  d = __builtin_amdgcn_fmed3f(d, -448.0f, 448.0f);
+  int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+  return (uint32_t)w;
+}
+
+__device__ __forceinline__ uint32_t f32_to_s8_sat(float x) {
+  // cvt.rni.sat.s8.f32: round half to even, clamp, NaN -> 0
+  int i = (int)__builtin_rintf(x);  // v_cvt_i32_f32 saturates and maps NaN to 0
+  i = i < -128 ? -128 : (i > 127 ? 127 : i);
+  return (uint32_t)i & 0xffu;
+}
+
+template <RowFmt FMT>
+__device__ __forceinline__ uint2 rowfmt_pack8(uint4 v, float recp, bool nan_row) {
+  float f[8] = {bf16_lo(v.x) * recp, bf16_hi(v.x) * recp, bf16_lo(v.y) * recp, bf16_hi(v.y) * recp,
+                bf16_lo(v.z) * recp, bf16_hi(v.z) * recp, bf16_lo(v.w) * recp, bf16_hi(v.w) * recp};
+  uint2 o;
+  if (FMT == RowFmt::FP8) {
+    o.x = f32x4_to_e4m3x4(f[0], f[1], f[2], f[3]);
+    o.y = f32x4_to_e4m3x4(f[4], f[5], f[6], f[7]);
+    if (nan_row) o.x = o.y = 0x7f7f7f7fu;  // amax == 0: 0 * inf = NaN in every position
+  } else {
+    o.x = f32_to_s8_sat(f[0]) | (f32_to_s8_sat(f[1]) << 8) | (f32_to_s8_sat(f[2]) << 16) |
+          (f32_to_s8_sat(f[3]) << 24);
+    o.y = f32_to_s8_sat(f[4]) | (f32_to_s8_sat(f[5]) << 8) | (f32_to_s8_sat(f[6]) << 16) |
+          (f32_to_s8_sat(f[7]) << 24);
+  }
+  return o;
+}
+
+// Row-major fast path: the whole row lives in registers between the amax pass and the
+// convert pass, so the input is read from memory once.  LPR lanes share a row (DPP / swizzle
+// reduction), each lane holds NV 16-byte vectors at a stride of LPR*8 elements.
+template <RowFmt FMT, int LPR, int NV>
+__global__ __launch_bounds__(256) void quantize_rowwise_rowmajor_kernel(
+    uint8_t *__restrict__ out, float *__restrict__ sf, const uint16_t *__restrict__ in,
+    const void *__restrict__ smax_p, QuantGeom g) {
+  const float smax = load_scale_max<FMT>(smax_p);
+  constexpr int RPB = 256 / LPR;  // rows per block
+  const int sub = threadIdx.x % LPR;
+  const int64_t r = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
+  const int64_t lead = blockIdx.y;
+  const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + r * g.sR;
+  uint4 v[NV];
+  uint32_t m = 0;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int64_t k = ((int64_t)j * LPR + sub) * 8;
+    v[j] = make_uint4(0, 0, 0, 0);
+    if (r < g.R && k < g.K) v[j] = ld_stream_u4(src + k);
+    m = umax32(m, absmax_bf16x8(v[j]));
+  }
+  m = group_umax<LPR>(m);
+  const float amax = bf16_bits_to_f32(m);
+  if (sub == 0 && r < g.Rp) sf[lead * g.Rp + r] = amax / smax;
+  if (r >= g.R) return;
+  const float recp = smax / amax;
+  const bool nan_row = (FMT == RowFmt::FP8) && (amax == 0.0f);
+  uint8_t *op = out + (lead * g.R + r) * g.Kp;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int64_t k = ((int64_t)j * LPR + sub) * 8;
+    if (k < g.Kp)
+      st_stream_u2(op + k, rowfmt_pack8<FMT>(v[j], recp, nan_row));
+  }
+}
+
+// Generic path: any strides / swizzle / K.  One lane per row, two passes over the row.
+template <RowFmt FMT, bool SWIZZLE>
+__global__ __launch_bounds__(256) void quantize_rowwise_generic_kernel(
+    uint8_t *__restrict__ out, float *__restrict__ sf, const uint16_t *__restrict__ in,
+    const void *__restrict__ smax_p, QuantGeom g) {
+  const float smax = load_scale_max<FMT>(smax_p);
+  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t lead = blockIdx.y;
+  if (r >= g.Rp) return;
+  if (r >= g.R) {
+    sf[lead * g.Rp + r] = 0.0f / smax;
+    return;
+  }
+  const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + r * g.sR;
+  uint32_t m = 0;
+  for (int64_t k = 0; k < g.K; ++k) m = umax32(m, src[k * g.sK] & 0x7fffu);
+  const float amax = bf16_bits_to_f32(m);
+  sf[lead * g.Rp + r] = amax / smax;
+  const float recp = smax / amax;
+  const bool nan_row = (FMT == RowFmt::FP8) && (amax == 0.0f);
+  uint32_t *op = reinterpret_cast<uint32_t *>(out + (lead * g.R + r) * g.Kp);
+  for (int64_t k4 = 0; k4 < g.Kp; k4 += 4) {
+    float f[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int64_t kk = k4 + i;
+      if (SWIZZLE) {
+        int p = (int)(kk & 15);
+        kk = (kk & ~(int64_t)15) + ((p & 3) >> 1) * 8 + (p >> 2) * 2 + (p & 1);
+      }
+      f[i] = (kk < g.K ? bf16_bits_to_f32(src[kk * g.sK]) : 0.0f) * recp;
+    }
+    uint32_t w;
+    if (FMT == RowFmt::FP8) {
+      w = nan_row ? 0x7f7f7f7fu : f32x4_to_e4m3x4(f[0], f[1], f[2], f[3]);
+    } else {
+      w = f32_to_s8_sat(f[0]) | (f32_to_s8_sat(f[1]) << 8) | (f32_to_s8_sat(f[2]) << 16) |
+          (f32_to_s8_sat(f[3]) << 24);
+    }
+    op[k4 / 4] = w;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host launchers
+// ---------------------------------------------------------------------------
+
+static int check_geom(const void *out, const void *sf, const void *in, const void *scalar, int64_t d0,
+                      int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR, int64_t sK) {
+  AC4K_REQUIRE(out && sf && in && scalar, "null pointer argument");
+  AC4K_REQUIRE(d0 >= 1 && d1 >= 1 && R >= 1 && K >= 1, "sizes must be positive (d0=%lld d1=%lld R=%lld K=%lld)",
+               (long long)d0, (long long)d1, (long long)R, (long long)K);
+  AC4K_REQUIRE(s0 >= 0 && s1 >= 0 && sR >= 1 && sK >= 1, "strides must be positive");
+  AC4K_REQUIRE(d0 * d1 <= 65535, "product of the leading dims must be <= 65535 (got %lld)", (long long)(d0 * d1));
+  return 0;
+}
+
+static bool rowmajor_ok(const void *in, int64_t K, int64_t s0, int64_t s1, int64_t sR, int64_t sK) {
+  return sK == 1 && K % 8 == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0 && sR % 8 == 0 &&
+         s0 % 8 == 0 && s1 % 8 == 0;
+}
+
+template <int CPR>
+static void launch_nvfp4_rowmajor(uint8_t *out, uint8_t *sf, const uint16_t *in, const float *gs,
+                                  const QuantGeom &g, int64_t lead, hipStream_t st) {
+  constexpr int ITER = 4;
+  constexpr int ROWS = 4 * (8 / CPR) * ITER;
+  dim3 grid((unsigned)(ceil_div(g.Kp / 64, CPR) * ceil_div(g.Rp, ROWS)), (unsigned)lead);
+  hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER>), grid, dim3(256), 0, st, out, sf, in, gs, g);
+}
+
+}  // namespace ac4k
+
+using namespace ac4k;
+
+extern "C" __attribute__((visibility("default"))) int ac4k_global_scale_bf16(float *gs, const void *x, int64_t n, float max_scale,
+                                      ac4k_stream_t stream) {
+  AC4K_REQUIRE(gs && (x || n == 0), "null pointer argument");
+  AC4K_REQUIRE(n >= 0, "n must be non-negative");
+  AC4K_REQUIRE((reinterpret_cast<uintptr_t>(x) & 1) == 0, "x must be 2-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(1), 0, st, reinterpret_cast<uint32_t *>(gs));
+  if (n > 0) {
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(x);
+    int64_t head = ((16 - (addr & 15)) & 15) / 2;
+    if (head > n) head = n;
+    const int64_t nvec = (n - head) / 8;
+    int64_t blocks = ceil_div(nvec, (int64_t)AMAX_THREADS * AMAX_UNROLL);
+    if (blocks < 1) blocks = 1;
+    if (blocks > 2048) blocks = 2048;
+    hipLaunchKernelGGL(amax_scale_bf16_kernel, dim3((unsigned)blocks), dim3(AMAX_THREADS), 0, st,
+                       reinterpret_cast<uint32_t *>(gs), static_cast<const uint16_t *>(x), n, head, nvec,
+                       max_scale);
+  }
+  return check_launch("ac4k_global_scale_bf16");
+}
+
+extern "C" __attribute__((visibility("default"))) int ac4k_quantize_nvfp4(void *out, void *sf, const void *in, const float *global_scale, int64_t d0,
+                                   int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
+                                   int64_t sK, int swizzle, ac4k_stream_t stream) {
+  if (int rc = check_geom(out, sf, in, global_scale, d0, d1, R, K, s0, s1, sR, sK)) return rc;
+  QuantGeom g{d1, R, K, align_up(K, 64), align_up(R, 16), s0, s1, sR, sK};
+  hipStream_t st = (hipStream_t)stream;
+  uint8_t *o = static_cast<uint8_t *>(out), *s = static_cast<uint8_t *>(sf);
+  const uint16_t *x = static_cast<const uint16_t *>(in);
+  const int64_t lead = d0 * d1;
+  if (!swizzle && rowmajor_ok(in, K, s0, s1, sR, sK) && ceil_div(g.Kp, 64) * ceil_div(g.Rp, 16) < (1ll << 31)) {
+    const int64_t chunks = g.Kp / 64;
+    if (chunks >= 8)
+      launch_nvfp4_rowmajor<8>(o, s, x, global_scale, g, lead, st);
+    else if (chunks >= 3)
+      launch_nvfp4_rowmajor<4>(o, s, x, global_scale, g, lead, st);
+    else if (chunks == 2)
+      launch_nvfp4_rowmajor<2>(o, s, x, global_scale, g, lead, st);
+    else
+      launch_nvfp4_rowmajor<1>(o, s, x, global_scale, g, lead, st);
+  } else {
+    AC4K_REQUIRE(g.Kp / 64 <= 65535, "reduce dim too large for the strided path (%lld)", (long long)K);
+    dim3 grid((unsigned)ceil_div(g.Rp, 256), (unsigned)(g.Kp / 64), (unsigned)lead);
+    if (swizzle)
+      hipLaunchKernelGGL(quantize_nvfp4_generic_kernel<true>, grid, dim3(256), 0, st, o, s, x, global_scale, g);
+    else
+      hipLaunchKernelGGL(quantize_nvfp4_generic_kernel<false>, grid, dim3(256), 0, st, o, s, x, global_scale, g);
+  }
+  return check_launch("ac4k_quantize_nvfp4");
+}
+
+namespace ac4k {
+
+template <RowFmt FMT, int LPR, int NV>
+static void launch_rowwise_rowmajor(uint8_t *out, float *sf, const uint16_t *in, const void *smax,
+                                    const QuantGeom &g, int64_t lead, hipStream_t st) {
+  dim3 grid((unsigned)ceil_div(g.Rp, 256 / LPR), (unsigned)lead);
+  hipLaunchKernelGGL((quantize_rowwise_rowmajor_kernel<FMT, LPR, NV>), grid, dim3(256), 0, st, out, sf, in,
+                     smax, g);
+}
+
+template <RowFmt FMT>
+static int quantize_rowwise(void *out, float *sf, const void *in, const void *smax, int64_t d0, int64_t d1,
+                            int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR, int64_t sK, int swizzle,
+                            hipStream_t st, const char *what) {
+  if (int rc = check_geom(out, sf, in, smax, d0, d1, R, K, s0, s1, sR, sK)) return rc;
+  QuantGeom g{d1, R, K, align_up(K, 16), align_up(R, 16), s0, s1, sR, sK};
+  uint8_t *o = static_cast<uint8_t *>(out);
+  const uint16_t *x = static_cast<const uint16_t *>(in);
+  const int64_t lead = d0 * d1;
+  if (!swizzle && rowmajor_ok(in, K, s0, s1, sR, sK) && K <= 8192) {
+    if (K <= 64)
+      launch_rowwise_rowmajor<FMT, 8, 1>(o, sf, x, smax, g, lead, st);
+    else if (K <= 128)
+      launch_rowwise_rowmajor<FMT, 16, 1>(o, sf, x, smax, g, lead, st);
+    else if (K <= 256)
+      launch_rowwise_rowmajor<FMT, 32, 1>(o, sf, x, smax, g, lead, st);
+    else if (K <= 512)
+      launch_rowwise_rowmajor<FMT, 64, 1>(o, sf, x, smax, g, lead, st);
+    else if (K <= 1024)
+      launch_rowwise_rowmajor<FMT, 64, 2>(o, sf, x, smax, g, lead, st);
+    else if (K <= 2048)
+      launch_rowwise_rowmajor<FMT, 64, 4>(o, sf, x, smax, g, lead, st);
+    else if (K <= 4096)
+      launch_rowwise_rowmajor<FMT, 64, 8>(o, sf, x, smax, g, lead, st);
+    else
+      launch_rowwise_rowmajor<FMT, 64, 16>(o, sf, x, smax, g, lead, st);
+  } else {
+    dim3 grid((unsigned)ceil_div(g.Rp, 256), (unsigned)lead);
+    if (swizzle)
+      hipLaunchKernelGGL((quantize_rowwise_generic_kernel<FMT, true>), grid, dim3(256), 0, st, o, sf, x, smax, g);
+    else
+      hipLaunchKernelGGL((quantize_rowwise_generic_kernel<FMT, false>), grid, dim3(256), 0, st, o, sf, x, smax, g);
+  }
+  return check_launch(what);
+}
+
+}  // namespace ac4k
+
+extern "C" __attribute__((visibility("default"))) int ac4k_quantize_fp8(void *out, float *sf, const void *in, const float *scale_max, int64_t d0,
+                                 int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
+                                 int64_t sK, int swizzle, ac4k_stream_t stream) {
+  return quantize_rowwise<RowFmt::FP8>(out, sf, in, scale_max, d0, d1, R, K, s0, s1, sR, sK, swizzle,
+                                       (hipStream_t)stream, "ac4k_quantize_fp8");
+}
+
+extern "C" __attribute__((visibility("default"))) int ac4k_quantize_int8(void *out, float *sf, const void *in, const int32_t *scale_max, int64_t d0,
+                                  int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
+                                  int64_t sK, ac4k_stream_t stream) {
+  return quantize_rowwise<RowFmt::INT8>(out, sf, in, scale_max, d0, d1, R, K, s0, s1, sR, sK, 0,
+                                        (hipStream_t)stream, "ac4k_quantize_int8");
+}

@@ -1,0 +1,92 @@
+"""`quantize` with the reference's signature, shapes and return tuples
+(python/ac4k_kernel/ops/quant.py:68-294), running on the gfx950 HIP kernels.
+
+The global-scale reduction that the reference does in Triton (quant.py:21-59) is a HIP
+kernel behind the same C ABI.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _rocm_ops
+from .utils import align_up
+
+quantize_nvfp4 = _rocm_ops.quantize_nvfp4
+quantize_fp8 = _rocm_ops.quantize_fp8
+quantize_int8 = _rocm_ops.quantize_int8
+
+
+def _global_scale(x: torch.Tensor, max_scale: float) -> torch.Tensor:
+    out = torch.empty((), dtype=torch.float32, device=x.device)
+    _rocm_ops.global_scale(out, x, max_scale)
+    return out
+
+
+def _lead_shape(shape, cross_dim, reduce_dim):
+    return [shape[i] for i in range(len(shape)) if i != cross_dim and i != reduce_dim]
+
+
+class Ac4kQuantizeOp(torch.nn.Module):
+
+    def forward(self, input: torch.Tensor, cross_dim, reduce_dim, max_scale=None, precision="nvfp4",
+                swizzle=False, output=None, sf=None):
+        assert input.ndim >= 2 and input.ndim <= 4, "input tensor must be 2D, 3D or 4D"
+        assert precision in ["nvfp4", "fp8e4m3", "int8"]
+        if cross_dim < 0:
+            cross_dim += input.ndim
+        if reduce_dim < 0:
+            reduce_dim += input.ndim
+        assert cross_dim != reduce_dim, "cross_dim and reduce_dim must be different"
+
+        shape = input.shape
+        lead = _lead_shape(shape, cross_dim, reduce_dim)
+        R, K = shape[cross_dim], shape[reduce_dim]
+        dev = input.device
+
+        if precision in ("fp8e4m3", "int8"):
+            fp8 = precision == "fp8e4m3"
+            out_dtype = torch.float8_e4m3fn if fp8 else torch.int8
+            # out [.., cross, align_up(reduce, 16)], sf [.., align_up(cross, 16)] fp32
+            if output is None:
+                output = torch.empty(lead + [R, align_up(K, 16)], dtype=out_dtype, device=dev)
+            if sf is None:
+                sf = torch.empty(lead + [align_up(R, 16)], dtype=torch.float32, device=dev)
+            if max_scale is None:
+                max_scale = 448 if fp8 else 127
+            if fp8:
+                smax = torch.full([], max_scale, dtype=torch.float32, device=dev)
+                quantize_fp8(output, sf, input, smax, cross_dim, reduce_dim, swizzle)
+            else:
+                smax = torch.full([], max_scale, dtype=torch.int32, device=dev)
+                quantize_int8(output, sf, input, smax, cross_dim, reduce_dim)
+            return output, sf
+
+        if max_scale is None:
+            max_scale = torch.finfo(torch.float8_e4m3fn).max * 6.0
+        global_scale = _global_scale(input, float(max_scale))
+        # out [.., cross, align_up(reduce, 64) / 2] u8, sf [.., align_up(reduce, 64) / 64, align_up(cross, 16), 4]
+        Kp = align_up(K, 64)
+        if output is None:
+            output = torch.empty(lead + [R, Kp // 2], dtype=torch.uint8, device=dev)
+        if sf is None:
+            sf = torch.empty(lead + [Kp // 64, align_up(R, 16), 4], dtype=torch.float8_e4m3fn, device=dev)
+        quantize_nvfp4(output, sf, input, global_scale, cross_dim, reduce_dim, swizzle)
+        return output, sf, global_scale
+
+
+def quantize(input, cross_dim, reduce_dim, max_scale=None, precision="nvfp4", swizzle=False, output=None,
+             sf=None):
+    """Quantize a bf16 tensor to nvfp4, fp8e4m3 or int8.
+
+    cross_dim is the M/N (parallel) dim, reduce_dim the K dim.  max_scale defaults to 6*448 for
+    nvfp4, 448 for fp8e4m3, 127 for int8.  swizzle permutes the reduce dim as
+    reshape(-1,4,4,2).permute(0,2,1,3) for nvfp4 and reshape(-1,2,4,2).permute(0,2,1,3) for fp8e4m3.
+
+    Returns (output, sf, global_scale) for nvfp4 and (output, sf) otherwise:
+      nvfp4   output [.., cross, align_up(reduce,64)/2] u8, sf [.., ceil(reduce/64), align_up(cross,16), 4] e4m3
+      fp8e4m3 output [.., cross, align_up(reduce,16)] e4m3, sf [.., align_up(cross,16)] fp32
+      int8    output [.., cross, align_up(reduce,16)] int8, sf [.., align_up(cross,16)] fp32
+    where `..` are the remaining input dims in their original order.
+    """
+    return Ac4kQuantizeOp()(input, cross_dim, reduce_dim, max_scale=max_scale, precision=precision,
+                            swizzle=swizzle, output=output, sf=sf)

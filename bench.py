@@ -1,0 +1,222 @@
+#!/usr/bin/env python3
+"""Benchmark of the NVFP4 path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+
+Prints ONE JSON line.  The headline `value` is the NVFP4 linear at M=N=K=8192 (the
+north-star GEMM, also the first shape of the reference's test/test_linear_tflops.py:189)
+in TFLOP/s = 2*M*N*K / t, with the operands already quantized and resident in HBM.  The
+same line carries, under "quantize", the BF16->NVFP4 / FP8 / INT8 quantizers on the
+8192x4096 outlier activations (GB/s = (in + out + sf bytes) / t as in
+test/test_quantize_bandwidth.py:32-33, whole quantize() call) and the 4096x4096 case.
+
+A "step" is one pass of the timed op over one batch of synthetic input.  Timing uses
+events recorded on the stream the kernels are launched on (torch's current stream, which
+is the stream handed to the C ABI).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16 MFMA (identical rates)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_input(shape, seed=0, outliers=False, std=1.0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    x = torch.randn(shape, generator=g, dtype=torch.float32) * std
+    if outliers:
+        x = torch.where(torch.rand(shape, generator=g) < 0.001, x * 20.0, x)
+    return x.to(torch.bfloat16)
+
+
+def time_gpu(fn, steps, warmup):
+    """-> (total ms over `steps` calls, ms per call); events on the launch stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    total = start.elapsed_time(end)
+    return total, total / steps
+
+
+# --------------------------------------------------------------------------- quantize
+def quant_bytes(shape_rk, precision):
+    R, K = shape_rk
+    if precision == "nvfp4":
+        Kp, Rp = (K + 63) // 64 * 64, (R + 15) // 16 * 16
+        return 2 * R * K + R * Kp // 2 + (Kp // 64) * Rp * 4 + 4
+    Kp, Rp = (K + 15) // 16 * 16, (R + 15) // 16 * 16
+    return 2 * R * K + R * Kp + 4 * Rp
+
+
+def bench_quantize(ops, shape, precision, steps, warmup, outliers, check=True, nbuf=3):
+    from oracle import nvfp4_oracle as T
+    xs_cpu = [make_input(shape, seed=s, outliers=outliers) for s in range(nbuf)]
+    xs = [x.cuda() for x in xs_cpu]
+    res = ops.quantize(xs[0], 0, 1, precision=precision)
+    outs = [[torch.empty_like(t) for t in res[:2]] for _ in range(nbuf)]
+    ok = None
+    if check:
+        if precision == "nvfp4":
+            e = T.quantize_nvfp4(xs_cpu[0], 0, 1)
+            ok = (torch.equal(res[0].cpu(), e[0]) and torch.equal(res[1].cpu().view(torch.uint8), e[1])
+                  and res[2].item() == e[2].item())
+        elif precision == "fp8e4m3":
+            e = T.quantize_fp8(xs_cpu[0], 0, 1)
+            ok = torch.equal(res[0].cpu().view(torch.uint8), e[0]) and torch.equal(res[1].cpu(), e[1])
+        else:
+            e = T.quantize_int8(xs_cpu[0], 0, 1)
+            ok = torch.equal(res[0].cpu(), e[0]) and torch.equal(res[1].cpu(), e[1])
+    i = [0]
+
+    def step():
+        j = i[0] % nbuf
+        i[0] += 1
+        ops.quantize(xs[j], 0, 1, precision=precision, output=outs[j][0], sf=outs[j][1])
+
+    _, ms = time_gpu(step, steps, warmup)
+    nbytes = quant_bytes(shape, precision)
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return {"workload": f"quantize {precision} {shape[0]}x{shape[1]} bf16" + (" outliers" if outliers else ""),
+            "ms": ms, "bytes": nbytes, "GB/s": gbs, "bit_exact_vs_oracle": ok,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": gbs / HBM_PEAK_GBS, "traffic": None},
+            "rotating_buffers": nbuf}
+
+
+def cpu_quantize_baseline(shape, outliers):
+    from oracle import nvfp4_oracle as T
+    x = make_input(shape, seed=0, outliers=outliers)
+    T.quantize_nvfp4(x[:256], 0, 1)
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        T.quantize_nvfp4(x, 0, 1)
+        ts.append(time.perf_counter() - t0)
+    t = sorted(ts)[1]
+    return {"value": quant_bytes(shape, "nvfp4") / t / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port", "sample": f"full nvfp4 quantize of one {shape[0]}x{shape[1]} bf16 tensor, median of 3"}
+
+
+# --------------------------------------------------------------------------- linear
+def gpu_dequant(q, rows):
+    from oracle import nvfp4_oracle as T
+    packed, sf, gs = q
+    lut = T.E2M1_LUT.cuda()
+    v = torch.stack((lut[(packed & 0xF).long()], lut[(packed >> 4).long()]), dim=-1).reshape(rows, -1, 16)
+    s = sf.permute(1, 0, 2).reshape(sf.shape[1], -1)[:rows].float() * gs
+    return (v * s.unsqueeze(-1)).reshape(rows, -1)
+
+
+def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True):
+    a, b = make_input((m, k), seed=0), make_input((n, k), seed=1, std=wstd)
+    aq, bq = ops.quantize(a.cuda(), 0, 1), ops.quantize(b.cuda(), 0, 1)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    ops.linear(*aq, *bq, out=out)
+    ok = None
+    if check:  # fp32 dequantize-matmul on a row sample, atol = rtol = 1e-2
+        rows = torch.arange(0, m, max(1, m // 128), device="cuda")
+        ref = (gpu_dequant(aq, m)[rows] @ gpu_dequant(bq, n).t()).to(torch.bfloat16)
+        got = out[rows]
+        ok = bool(torch.all((got.float() - ref.float()).abs() <= 1e-2 + 1e-2 * ref.float().abs()).item())
+        del ref
+    total, ms = time_gpu(lambda: ops.linear(*aq, *bq, out=out), steps, warmup)
+    tflops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
+    return {"workload": f"NVFP4 linear M={m} N={n} K={k}, bf16 out, operands pre-quantized", "ms": ms,
+            "total_ms": total, "TFLOP/s": tflops, "within_1e-2_of_fp32_dequant_matmul": ok,
+            "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": tflops / MFMA_PEAK_TFLOPS, "traffic": None}}
+
+
+def cpu_linear_baseline(n, k, rows=256):
+    """fp32 dequantize-then-matmul of the oracle on `rows` rows of the 8192^3 problem."""
+    from oracle import nvfp4_oracle as T
+    a, b = make_input((rows, k), seed=0), make_input((n, k), seed=1)
+    aq, bq = T.quantize_nvfp4(a, 0, 1), T.quantize_nvfp4(b, 0, 1)
+    t0 = time.perf_counter()
+    T.linear_nvfp4(*aq, *bq)
+    t = time.perf_counter() - t0
+    return {"value": 2.0 * rows * n * k / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"oracle fp32 dequantize + torch.matmul of M={rows} rows of the N={n} K={k} problem, 1 run"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="all", choices=["all", "linear", "quantize"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1")
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    torch.set_num_threads(min(16, os.cpu_count() or 1))
+    from ac4k_kernel_amd import ops
+
+    check = not args.no_check
+    line = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "data": "synthetic (seed 0, generated on CPU, cast to bf16)"}
+    quant = None
+    if args.workload in ("all", "quantize"):
+        quant = {
+            "cfg2_nvfp4": bench_quantize(ops, (8192, 4096), "nvfp4", args.steps, args.warmup, True, check),
+            "cfg2_fp8e4m3": bench_quantize(ops, (8192, 4096), "fp8e4m3", args.steps, args.warmup, True, check),
+            "cfg2_int8": bench_quantize(ops, (8192, 4096), "int8", args.steps, args.warmup, True, check),
+            "cfg1_nvfp4": bench_quantize(ops, (4096, 4096), "nvfp4", args.steps, args.warmup, False, check),
+        }
+        for k_, v in quant.items():
+            log(f"[bench] {k_}: {v['ms'] * 1e3:.1f} us  {v['GB/s']:.0f} GB/s  "
+                f"({100 * v['roofline']['frac']:.1f}% of HBM peak)  bit-exact={v['bit_exact_vs_oracle']}")
+        if not args.no_cpu_baseline:
+            quant["cpu_baseline"] = cpu_quantize_baseline((4096, 4096), False)
+            log(f"[bench] cpu quantize oracle: {quant['cpu_baseline']['value']:.2f} GB/s on "
+                f"{quant['cpu_baseline']['cores']} threads")
+    if args.workload in ("all", "linear"):
+        lin = bench_linear(ops, 8192, 8192, 8192, args.steps, args.warmup, check=check)
+        log(f"[bench] {lin['workload']}: {lin['ms']:.3f} ms  {lin['TFLOP/s']:.1f} TFLOP/s "
+            f"({100 * lin['roofline']['frac']:.1f}% of MFMA peak)  ok={lin['within_1e-2_of_fp32_dequant_matmul']}")
+        line.update({"metric": "nvfp4_linear_tflops", "value": lin["TFLOP/s"], "unit": "TFLOP/s",
+                     "ms_per_step": lin["ms"], "dtype": "fp4 x e4m3 decoded exactly to fp16, fp32 accumulate",
+                     "config": {"workload": lin["workload"]}, "roofline": lin["roofline"],
+                     "parity": lin["within_1e-2_of_fp32_dequant_matmul"]})
+        if not args.no_cpu_baseline:
+            line["cpu_baseline"] = cpu_linear_baseline(8192, 8192)
+            log(f"[bench] cpu linear oracle: {line['cpu_baseline']['value']:.3f} TFLOP/s")
+        if quant is not None:
+            line["quantize"] = quant
+    else:
+        q = quant["cfg2_nvfp4"]
+        line.update({"metric": "nvfp4_quantize_gbs", "value": q["GB/s"], "unit": "GB/s", "ms_per_step": q["ms"],
+                     "dtype": "bf16 -> e2m1 + e4m3 scales (fp32 arithmetic)", "config": {"workload": q["workload"]},
+                     "roofline": q["roofline"], "parity": q["bit_exact_vs_oracle"], "quantize": quant})
+        if "cpu_baseline" in quant:
+            line["cpu_baseline"] = quant["cpu_baseline"]
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,101 @@
+/*
+ * ac4k_nvfp4.h — C ABI of the MI355X (gfx950) NVFP4 path.
+ *
+ * One shared library, plain pointers and sizes, no torch / pybind types.  It
+ * takes the place of the reference's pybind11 module `ac4k_kernel._cuda_ops`
+ * (lib/cuda_bindings.cc:37-97, declarations in include/ac4k_kernel/ops.h:27-48)
+ * for the quantize and linear entry points, and of the Triton global-scale
+ * helper (python/ac4k_kernel/ops/quant.py:33-59).
+ *
+ * Conventions (identical to the reference binding):
+ *   - every pointer is DEVICE memory owned by the caller; the library never
+ *     allocates, frees or synchronises; work is enqueued on `stream`
+ *     (a hipStream_t; NULL = the default stream) and returns immediately;
+ *   - scalars that the reference passes as 0-dim device tensors
+ *     (global_scale, scale_max) are device pointers here too;
+ *   - return value 0 = launched; non-zero = rejected, nothing was launched and
+ *     ac4k_last_error() (thread-local) says why.  The conditions are the
+ *     reference's TORCH_CHECKs that can be stated on raw pointers and sizes.
+ *
+ * Quantizer geometry.  The reference host code left-pads the input to 4-D and
+ * passes the sizes/strides of the two dims that are neither cross nor reduce
+ * (quantize_nvfp4.cu:226-241,257-260); the same is passed here:
+ *   d0,d1 : sizes of the two leading (batch-like) dims, 1 when absent
+ *   R, K  : cross (row) and reduce sizes
+ *   s0,s1,sR,sK : element strides of those four dims in `in`
+ * Outputs are dense: out [d0,d1,R,*], sf as documented per function.
+ */
+#ifndef AC4K_NVFP4_H_
+#define AC4K_NVFP4_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *ac4k_stream_t; /* hipStream_t */
+
+/* dtype tags for D and bias of ac4k_linear_nvfp4 */
+enum { AC4K_DTYPE_BF16 = 0, AC4K_DTYPE_FP16 = 1, AC4K_DTYPE_FP32 = 2 };
+
+/* Module attributes of lib/cuda_bindings.cc:41-44 (__arch__, __backend__, __version__,
+ * __arch_description__). */
+const char *ac4k_arch(void);             /* "gfx950" */
+const char *ac4k_arch_description(void); /* "AMD Instinct MI355X (CDNA4)" */
+const char *ac4k_backend(void);          /* "rocm" */
+const char *ac4k_version(void);          /* "0.1.0" */
+const char *ac4k_last_error(void);
+
+/* Replaces _global_scale / _triton_global_scale_kernel
+ * (python/ac4k_kernel/ops/quant.py:33-59):  *gs = fp32(max|x|) / max_scale over n
+ * contiguous bf16 values.  *gs needs no initialisation by the caller. */
+int ac4k_global_scale_bf16(float *gs, const void *x, int64_t n, float max_scale,
+                           ac4k_stream_t stream);
+
+/* Replaces ac4k::quantize_nvfp4 (lib/cuda/sm120/quantize_nvfp4.cu:164-271).
+ * out: uint8 [d0,d1,R,align_up(K,64)/2], low nibble = even element.
+ * sf : e4m3   [d0,d1,align_up(K,64)/64,align_up(R,16),4].
+ * Every byte of both is written (pad nibbles and pad-row scales are 0).
+ * swizzle != 0: reduce dim permuted as reshape(-1,4,4,2).permute(0,2,1,3). */
+int ac4k_quantize_nvfp4(void *out, void *sf, const void *in, const float *global_scale, int64_t d0,
+                        int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
+                        int64_t sK, int swizzle, ac4k_stream_t stream);
+
+/* Replaces ac4k::quantize_fp8 (lib/cuda/sm120/quantize_fp8.cu:192-290).
+ * out: e4m3 [d0,d1,R,align_up(K,16)];  sf: fp32 [d0,d1,align_up(R,16)] = amax/scale_max.
+ * swizzle != 0: reduce dim permuted as reshape(-1,2,4,2).permute(0,2,1,3). */
+int ac4k_quantize_fp8(void *out, float *sf, const void *in, const float *scale_max, int64_t d0,
+                      int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
+                      int64_t sK, int swizzle, ac4k_stream_t stream);
+
+/* Replaces ac4k::quantize_int8 (lib/cuda/sm120/quantize_int8.cu:175-262).
+ * scale_max is an int32 device scalar, as in the reference (:189). */
+int ac4k_quantize_int8(void *out, float *sf, const void *in, const int32_t *scale_max, int64_t d0,
+                       int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
+                       int64_t sK, ac4k_stream_t stream);
+
+/* Replaces ac4k::linear_nvfp4 (lib/cuda/sm120/linear_nvfp4.cu:753-901).
+ * D [M,N] (d_dtype) = (A . B^T) * (*A_gs * *B_gs) + bias.
+ * A [M,K/2], B [N,K/2] packed e2m1 (uint8); A_sf [ceil(K/64),align_up(M,16),4],
+ * B_sf [ceil(K/64),align_up(N,16),4] e4m3; bias [1,N] of bias_dtype or NULL.
+ * K = 2 * (bytes per packed row), K % 16 == 0. */
+int ac4k_linear_nvfp4(void *D, int d_dtype, const void *A, const void *A_sf, const float *A_gs,
+                      const void *B, const void *B_sf, const float *B_gs, const void *bias,
+                      int bias_dtype, int64_t M, int64_t N, int64_t K, ac4k_stream_t stream);
+
+/* Fused skinny linear: quantize(X,0,1) followed by linear(...) in one call, for decode-sized
+ * M (1..32).  No single reference function: it equals the composition the reference's tests
+ * make (test/test_linear_bench.py:128-137) — the activation bytes, scales and global scale
+ * it produces are those of ac4k_global_scale_bf16 + ac4k_quantize_nvfp4.
+ * X bf16 [M,K] contiguous, K % 64 == 0.  The quantized activation is also returned:
+ * X_q [M,K/2], X_sf [K/64,align_up(M,16),4], X_gs (1 float). */
+int ac4k_linear_nvfp4_fused_bf16(void *D, int d_dtype, const void *X, void *X_q, void *X_sf,
+                                 float *X_gs, const void *B, const void *B_sf, const float *B_gs,
+                                 const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K,
+                                 ac4k_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AC4K_NVFP4_H_ */

@@ -1,0 +1,77 @@
+"""The C-ABI library: loads, exports every function include/ac4k_nvfp4.h declares, reports
+attributes, and rejects bad arguments before touching the GPU (no compute calls here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "ac4k_nvfp4.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ac4k_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_loader_agree():
+    from ac4k_kernel_amd import _lib
+    names = declared_functions()
+    assert len(names) >= 11
+    assert sorted(_lib.SIGNATURES) == names
+    lib = _lib.load()
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_attributes():
+    import ac4k_kernel_amd as pkg
+    assert pkg.get_backend() == "rocm" and pkg.get_arch() == "gfx950"
+    assert pkg.get_info() == {"version": "0.1.0", "backend": "rocm", "arch": "gfx950"}
+    from ac4k_kernel_amd import ops
+    for name in ["quantize", "linear", "quantize_nvfp4", "quantize_fp8", "quantize_int8", "linear_nvfp4"]:
+        assert callable(getattr(ops, name))
+
+
+def test_product_does_not_import_oracle():
+    # the shipped package must not reach into oracle/ (it is the checker, not the product)
+    pkg = os.path.join(ROOT, "ac4k_kernel_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                src = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in src, os.path.join(dirpath, f)
+
+
+def test_argument_rejection_without_gpu():
+    from ac4k_kernel_amd import _lib
+    lib = _lib.load()
+    one = ctypes.c_void_p(16)  # never dereferenced: every call below is rejected during validation
+    rc = lib.ac4k_quantize_nvfp4(None, one, one, one, 1, 1, 4, 64, 0, 0, 64, 1, 0, None)
+    assert rc != 0 and b"null" in lib.ac4k_last_error()
+    rc = lib.ac4k_quantize_nvfp4(one, one, one, one, 1, 1, 0, 64, 0, 0, 64, 1, 0, None)
+    assert rc != 0 and b"positive" in lib.ac4k_last_error()
+    rc = lib.ac4k_linear_nvfp4(one, 0, one, one, one, one, one, one, None, 0, 4, 4, 24, None)
+    assert rc != 0 and b"multiple of 16" in lib.ac4k_last_error()
+    rc = lib.ac4k_linear_nvfp4(one, 7, one, one, one, one, one, one, None, 0, 4, 4, 64, None)
+    assert rc != 0 and b"bfloat16, half or float" in lib.ac4k_last_error()
+    rc = lib.ac4k_linear_nvfp4_fused_bf16(one, 0, one, one, one, one, one, one, one, None, 0, 64, 4, 64, None)
+    assert rc != 0 and b"1 <= M <= 32" in lib.ac4k_last_error()
+    with pytest.raises(RuntimeError):
+        _lib.check(rc)
+
+
+def test_python_checks_without_gpu():
+    import torch
+    from ac4k_kernel_amd import ops
+    x = torch.zeros((4, 64), dtype=torch.bfloat16)
+    with pytest.raises(AssertionError):
+        ops.quantize(x, 0, 0)
+    with pytest.raises(AssertionError):
+        ops.quantize(x, 0, 1, precision="fp4")
+    with pytest.raises(AssertionError):
+        ops.quantize(torch.zeros(8, dtype=torch.bfloat16), 0, 1)
+    with pytest.raises(RuntimeError):  # CPU tensor: "must be a CUDA tensor"
+        ops.quantize_fp8(torch.empty((4, 64), dtype=torch.float8_e4m3fn), torch.empty(16), x,
+                         torch.tensor(448.0), 0, 1, False)

@@ -1,0 +1,139 @@
+"""GPU parity of the NVFP4 linear: HIP kernel (through the C ABI) against the fp32
+dequantize-then-matmul oracle at atol = rtol = 1e-2 (test/test_linear_bench.py:152)."""
+import random
+
+import pytest
+import torch
+
+from conftest import make_input
+from oracle import c_oracle as C
+from oracle import nvfp4_oracle as T
+
+pytestmark = pytest.mark.gpu
+ATOL = RTOL = 1e-2
+
+
+def ops():
+    from ac4k_kernel_amd import ops as o
+    return o
+
+
+def gpu_quant(x):
+    out, sf, gs = ops().quantize(x.cuda(), 0, 1)
+    return out, sf, gs
+
+
+def cpu(q):
+    return q[0].cpu(), q[1].cpu().view(torch.uint8), q[2].cpu()
+
+
+def run_case(m, n, k, bias_dtype=None, o_dtype=None, seed=0, wstd=1.0):
+    a, b = make_input((m, k), seed=seed), make_input((n, k), seed=seed + 1, std=wstd)
+    aq, bq = gpu_quant(a), gpu_quant(b)
+    bias = None if bias_dtype is None else make_input((1, n), seed=seed + 2).to(bias_dtype)
+    out = None if o_dtype is None else torch.full((m, n), 7.0, dtype=o_dtype, device="cuda")
+    d = ops().linear(*aq, *bq, bias=None if bias is None else bias.cuda(), out=out)
+    assert d.shape == (m, n) and d.dtype == (o_dtype or torch.bfloat16)
+    ref = T.linear_nvfp4(*cpu(aq), *cpu(bq), bias=bias, out_dtype=o_dtype or torch.bfloat16)
+    torch.testing.assert_close(d.cpu(), ref, atol=ATOL, rtol=RTOL)
+    return d
+
+
+REF_SHAPES = [(128, 128, 128), (10, 512, 512), (1024, 1024, 384), (130, 384, 256), (666, 768, 512), (123, 321, 256),
+              (10, 15, 512), (1, 4, 256), (64, 64, 128), (12, 23, 55), (12, 23, 5), (256, 256, 2048), (129, 257, 192)]
+
+
+@pytest.mark.parametrize("m,n,k", REF_SHAPES)
+def test_reference_shapes(m, n, k):
+    run_case(m, n, k, seed=m + n)
+
+
+DT = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
+
+
+@pytest.mark.parametrize("o", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("b", ["bf16", "fp16", "fp32"])
+def test_dtype_matrix(o, b):
+    run_case(5, 33, 51, bias_dtype=DT[b], o_dtype=DT[o], seed=5)
+    run_case(130, 140, 128, bias_dtype=DT[b], o_dtype=DT[o], seed=6)
+
+
+def test_bias_1d_and_out_default():
+    a, b = make_input((7, 128), seed=1), make_input((9, 128), seed=2)
+    aq, bq = gpu_quant(a), gpu_quant(b)
+    bias = make_input((9,), seed=3)
+    d = ops().linear(*aq, *bq, bias=bias.cuda())
+    ref = T.linear_nvfp4(*cpu(aq), *cpu(bq), bias=bias)
+    torch.testing.assert_close(d.cpu(), ref, atol=ATOL, rtol=RTOL)
+
+
+def test_random_shapes():
+    rnd = random.Random(9567)
+    for t in range(20):
+        run_case(rnd.randint(2, 555), rnd.randint(2, 555), rnd.randint(2, 555), seed=t)
+
+
+def test_c_oracle_and_contract():
+    a, b = make_input((96, 320), seed=11), make_input((80, 320), seed=12, std=0.02)
+    aq, bq = gpu_quant(a), gpu_quant(b)
+    d = ops().linear(*aq, *bq, out=torch.empty((96, 80), dtype=torch.float32, device="cuda")).cpu()
+    torch.testing.assert_close(d, C.linear_nvfp4(*cpu(aq), *cpu(bq)), atol=1e-5, rtol=1e-4)
+    torch.testing.assert_close(d, T.linear_nvfp4_contract(*cpu(aq), *cpu(bq), out_dtype=torch.float32), atol=1e-5,
+                               rtol=1e-4)
+
+
+def gpu_dequant(q, rows):
+    """fp32 dequantize on the GPU with torch ops (for sizes the CPU oracle would take minutes on)."""
+    packed, sf, gs = q
+    lut = T.E2M1_LUT.cuda()
+    v = torch.stack((lut[(packed & 0xF).long()], lut[(packed >> 4).long()]), dim=-1).reshape(rows, -1, 16)
+    s = sf.permute(1, 0, 2).reshape(sf.shape[1], -1)[:rows].float() * gs
+    return (v * s.unsqueeze(-1)).reshape(rows, -1)
+
+
+@pytest.mark.parametrize("m,n,k,wstd", [(4096, 4096, 4096, 1.0), (2048, 14336, 4096, 0.02), (16, 4096, 14336, 0.02),
+                                        (8192, 8192, 8192, 1.0)])
+def test_large_shapes(m, n, k, wstd):
+    a, b = make_input((m, k), seed=0), make_input((n, k), seed=1, std=wstd)
+    aq, bq = gpu_quant(a), gpu_quant(b)
+    d = ops().linear(*aq, *bq)
+    # (1) CPU oracle on a sample of rows and columns
+    rows = torch.tensor([0, 1, m // 2, m - 1] if m >= 4 else list(range(m)))
+    cols = torch.arange(0, n, max(1, n // 64))
+    ca, cb = cpu(aq), cpu(bq)
+    fa = T.dequantize_nvfp4(ca[0][rows], ca[1][:, rows].contiguous(), ca[2])
+    fb = T.dequantize_nvfp4(cb[0][cols], cb[1][:, cols].contiguous(), cb[2])
+    ref = (fa @ fb.t()).to(torch.bfloat16)
+    torch.testing.assert_close(d.cpu()[rows][:, cols], ref, atol=ATOL, rtol=RTOL)
+    # (2) the whole matrix against a torch fp32 dequantize-matmul on the GPU
+    full = (gpu_dequant(aq, m) @ gpu_dequant(bq, n).t()).to(torch.bfloat16)
+    torch.testing.assert_close(d, full, atol=ATOL, rtol=RTOL)
+
+
+@pytest.mark.parametrize("m", [1, 8, 32])
+def test_fused_skinny_equals_composition(m):
+    n, k = 1024, 2048
+    x = make_input((m, k), seed=m, outliers=True).cuda()
+    wq = gpu_quant(make_input((n, k), seed=50, std=0.02))
+    d, (xq, xsf, xgs) = ops().fused_linear(x, *wq, return_quantized=True)
+    eq, esf, egs = T.quantize_nvfp4(x.cpu(), 0, 1)
+    assert torch.equal(xq.cpu(), eq) and torch.equal(xsf.cpu().view(torch.uint8), esf) and xgs.item() == egs.item()
+    ref = T.linear_nvfp4(eq, esf, egs, *cpu(wq))
+    torch.testing.assert_close(d.cpu(), ref, atol=ATOL, rtol=RTOL)
+    comp = ops().linear(*ops().quantize(x, 0, 1), *wq)
+    torch.testing.assert_close(d, comp, atol=ATOL, rtol=RTOL)
+
+
+def test_error_behaviour():
+    o = ops()
+    aq, bq = gpu_quant(make_input((8, 128), seed=1)), gpu_quant(make_input((16, 128), seed=2))
+    with pytest.raises(RuntimeError):
+        o.linear(*aq, *bq, out=torch.empty((8, 16), dtype=torch.float64, device="cuda"))
+    with pytest.raises(RuntimeError):
+        o.linear(*aq, *bq, bias=torch.zeros((1, 15), device="cuda"))
+    with pytest.raises(RuntimeError):
+        o.linear(aq[0], aq[1][:, :8], aq[2], *bq)        # scale tensor with the wrong row padding
+    with pytest.raises(RuntimeError):
+        o.linear(aq[0][:, :60], aq[1], aq[2], *bq)       # non-contiguous / K mismatch
+    with pytest.raises(RuntimeError):
+        o.linear(aq[0], aq[1], aq[2].reshape(1), *bq)    # global scale must be 0-dim

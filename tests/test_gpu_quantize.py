@@ -1,0 +1,166 @@
+"""GPU parity of the quantizers: HIP kernels (through the C ABI) against the CPU oracle,
+bit for bit, on the same seeded inputs."""
+import random
+
+import pytest
+import torch
+
+from conftest import make_input
+from oracle import c_oracle as C
+from oracle import nvfp4_oracle as T
+
+pytestmark = pytest.mark.gpu
+
+
+def ops():
+    from ac4k_kernel_amd import ops as o
+    return o
+
+
+def check_nvfp4(x, cross, red, swz=False, oracle=T, **kw):
+    out, sf, gs = ops().quantize(x.cuda(), cross, red, swizzle=swz, **kw)
+    eo, es, eg = oracle.quantize_nvfp4(x, cross, red, swz, **({"max_scale": kw["max_scale"]} if "max_scale" in kw else {}))
+    assert gs.dtype == torch.float32 and gs.dim() == 0 and gs.item() == eg.item(), (gs.item(), eg.item())
+    assert out.dtype == torch.uint8 and sf.dtype == torch.float8_e4m3fn
+    assert list(out.shape) == list(eo.shape) and list(sf.shape) == list(es.shape)
+    sfb = sf.cpu().view(torch.uint8)
+    nb = (out.cpu() != eo).sum().item()
+    ns = (sfb != es).sum().item()
+    assert nb == 0 and ns == 0, f"shape {tuple(x.shape)} cross {cross} reduce {red} swz {swz}: {nb} bytes, {ns} scales differ"
+
+
+NVFP4_SHAPES = [((128, 512), 0, 1), ((4096, 4096), 0, 1), ((1024, 1024), 1, 0), ((777, 879), 0, 1),
+                ((12, 5), 0, 1), ((1, 64), 0, 1), ((17, 8), 0, 1), ((33, 200), 0, 1), ((100, 1000), 0, 1),
+                ((3, 50, 72), 1, 2), ((3, 50, 72), 2, 1), ((2, 3, 40, 128), 2, 3), ((2, 300, 5, 128), 1, 3),
+                ((2, 300, 5, 128), 3, 1), ((5, 7, 96), 0, 2), ((257, 520), 0, 1), ((64, 136), 0, 1)]
+
+
+@pytest.mark.parametrize("shape,cross,red", NVFP4_SHAPES)
+@pytest.mark.parametrize("swz", [False, True])
+def test_nvfp4_gaussian(shape, cross, red, swz):
+    check_nvfp4(make_input(shape, seed=len(shape) + shape[-1], outliers=True), cross, red, swz)
+
+
+def test_nvfp4_value_set_and_c_oracle():
+    g = torch.Generator().manual_seed(9567)
+    vals = torch.tensor([1, 2, 4, 6, -1, -2, -4, -6], dtype=torch.bfloat16)
+    for shape, c, r, s in [((1024, 1024), 1, 0, False), ((128, 512), 0, 1, False), ((300, 77), 0, 1, True)]:
+        x = vals[torch.randint(0, 8, shape, generator=g)]
+        check_nvfp4(x, c, r, s, oracle=C)
+
+
+def test_nvfp4_random_shapes():
+    rnd = random.Random(9527)
+    for t in range(25):
+        shape = [rnd.randint(1, 512) for _ in range(2)]
+        c = rnd.randint(0, 1)
+        check_nvfp4(make_input(shape, seed=t), c, 1 - c, rnd.choice([False, True]))
+
+
+def test_nvfp4_config2_outliers_and_max_scale():
+    x = make_input((8192, 4096), seed=0, outliers=True)
+    check_nvfp4(x, 0, 1)
+    check_nvfp4(make_input((64, 256), seed=1), 0, 1, max_scale=1000.0)
+
+
+def test_nvfp4_edges():
+    x = torch.zeros((20, 100), dtype=torch.bfloat16)
+    x[3, 5], x[7, 70], x[9, 20] = 3.0, -0.5, -0.0
+    check_nvfp4(x, 0, 1)
+    check_nvfp4(torch.zeros((16, 64), dtype=torch.bfloat16), 0, 1)           # all-zero tensor: gs = 0
+    tiny = torch.full((4, 64), 1.0, dtype=torch.bfloat16)
+    tiny[:, 16:32] = 1e-6                                                    # block scale underflow
+    check_nvfp4(tiny, 0, 1)
+    big = make_input((32, 128), seed=2).float() * 1e30                       # large magnitudes
+    check_nvfp4(big.to(torch.bfloat16), 0, 1)
+
+
+def test_nvfp4_caller_buffers_and_negative_dims():
+    x = make_input((40, 192), seed=3).cuda()
+    out = torch.full((40, 96), 0xAA, dtype=torch.uint8, device="cuda")
+    sf = torch.full((3, 48, 4), 0.5, device="cuda").to(torch.float8_e4m3fn)
+    o2, s2, gs = ops().quantize(x, -2, -1, output=out, sf=sf)
+    assert o2 is out and s2 is sf
+    eo, es, eg = T.quantize_nvfp4(x.cpu(), 0, 1)
+    assert torch.equal(out.cpu(), eo) and torch.equal(sf.cpu().view(torch.uint8), es)
+
+
+def test_global_scale_unaligned_and_sizes():
+    from ac4k_kernel_amd import _rocm_ops
+    base = make_input((1 << 20) + 37, seed=4).cuda()
+    for off, n in [(0, 1), (1, 7), (3, 1000), (5, 65536 + 3), (0, (1 << 20) + 37), (7, 1 << 20)]:
+        x = base[off:off + n]
+        gs = torch.full((), 123.0, device="cuda")
+        _rocm_ops.global_scale(gs, x, 2688.0)
+        assert gs.item() == T.global_scale(x.cpu()).item(), (off, n)
+
+
+ROW_SHAPES = [((1024, 1024), 0, 1), ((8192, 4096), 0, 1), ((1024, 10), 0, 1), ((16, 16), 0, 1), ((777, 879), 0, 1),
+              ((2, 300, 5, 128), 3, 1), ((2, 300, 5, 128), 1, 3), ((50, 70), 1, 0), ((33, 8200), 0, 1),
+              ((9, 20000), 0, 1), ((65, 264), 0, 1), ((3, 50, 72), 1, 2), ((100, 2056), 0, 1)]
+
+
+@pytest.mark.parametrize("shape,cross,red", ROW_SHAPES)
+def test_fp8_gaussian(shape, cross, red):
+    x = make_input(shape, seed=shape[0], outliers=True)
+    for swz in (False, True):
+        out, sf = ops().quantize(x.cuda(), cross, red, precision="fp8e4m3", swizzle=swz)
+        eo, es = T.quantize_fp8(x, cross, red, None, swz)
+        assert out.dtype == torch.float8_e4m3fn and list(out.shape) == list(eo.shape)
+        assert torch.equal(sf.cpu(), es), (shape, swz)
+        n = (out.cpu().view(torch.uint8) != eo).sum().item()
+        assert n == 0, f"{shape} swz={swz}: {n} bytes differ"
+
+
+@pytest.mark.parametrize("shape,cross,red", ROW_SHAPES)
+def test_int8_gaussian(shape, cross, red):
+    x = make_input(shape, seed=shape[0] + 1, outliers=True)
+    out, sf = ops().quantize(x.cuda(), cross, red, precision="int8")
+    eo, es = T.quantize_int8(x, cross, red)
+    assert out.dtype == torch.int8 and list(out.shape) == list(eo.shape)
+    assert torch.equal(sf.cpu(), es)
+    n = (out.cpu() != eo).sum().item()
+    assert n == 0, f"{shape}: {n} bytes differ"
+
+
+def test_fp8_value_set_bit_exact():
+    g = torch.Generator().manual_seed(9567)
+    vals = torch.tensor([-8, -6, -5, -4, 1, 2, 3, 4, 5, 6, 8, 9], dtype=torch.bfloat16)
+    for shape, c, r, s in [((1024, 1024), 0, 1, False), ((1, 500, 40, 128), 3, 1, True), ((1024, 10), 0, 1, False),
+                           ((16, 16), 0, 1, True), ((777, 879), 0, 1, True)]:
+        x = vals[torch.randint(0, len(vals), shape, generator=g)]
+        out, sf = ops().quantize(x.cuda(), c, r, max_scale=2.25, swizzle=s, precision="fp8e4m3")
+        eo, es = C.quantize_fp8(x, c, r, 2.25, s)
+        assert torch.equal(sf.cpu(), es) and torch.equal(out.cpu().view(torch.uint8), eo), shape
+
+
+def test_rowwise_edges_and_max_scale():
+    x = make_input((40, 96), seed=6)
+    x[5] = 0                                   # zero row: fp8 bytes 0x7F, int8 bytes 0, scale 0
+    x[6, :] = 1e-38                            # amax so small that scale_max / amax overflows
+    for prec, orc, kw in [("fp8e4m3", T.quantize_fp8, {}), ("int8", T.quantize_int8, {}),
+                          ("fp8e4m3", T.quantize_fp8, {"max_scale": 1000.0}), ("int8", T.quantize_int8, {"max_scale": 7})]:
+        out, sf = ops().quantize(x.cuda(), 0, 1, precision=prec, **kw)
+        eo, es = orc(x, 0, 1, *( [kw["max_scale"]] if kw else []))
+        raw = out.cpu().view(torch.uint8) if prec == "fp8e4m3" else out.cpu()
+        assert torch.equal(sf.cpu(), es), (prec, kw)
+        assert torch.equal(raw, eo), (prec, kw, (raw != eo).nonzero()[:4])
+
+
+def test_error_behaviour():
+    o = ops()
+    x = make_input((8, 64), seed=7).cuda()
+    with pytest.raises(AssertionError):
+        o.quantize(x, 1, 1)
+    with pytest.raises(RuntimeError):
+        o.quantize(x.float(), 0, 1)                      # not bf16
+    with pytest.raises(RuntimeError):
+        o.quantize(x.t(), 0, 1)                          # not contiguous
+    with pytest.raises(RuntimeError):
+        o.quantize(x, 0, 1, output=torch.empty((8, 16), dtype=torch.uint8, device="cuda"))
+    with pytest.raises(RuntimeError):
+        o.quantize(x, 0, 1, sf=torch.empty((1, 8, 4), dtype=torch.float8_e4m3fn, device="cuda"))
+    gs = torch.ones((1,), device="cuda")
+    with pytest.raises(RuntimeError):                    # global scale must be 0-dim
+        o.quantize_nvfp4(torch.empty((8, 32), dtype=torch.uint8, device="cuda"),
+                         torch.empty((1, 16, 4), dtype=torch.float8_e4m3fn, device="cuda"), x, gs, 0, 1, False)
