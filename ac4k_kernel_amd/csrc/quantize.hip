@@ -80,7 +80,9 @@ __device__ __forceinline__ float nvfp4_block_scale(float amax, float alpha, uint
 __device__ __forceinline__ uint32_t nvfp4_pack8(uint4 v, float o) {
   float f[8] = {bf16_lo(v.x) * o, bf16_hi(v.x) * o, bf16_lo(v.y) * o, bf16_hi(v.y) * o,
                 bf16_lo(v.z) * o, bf16_hi(v.z) * o, bf16_lo(v.w) * o, bf16_hi(v.w) * o};
-  return f32x8_to_e2m1x8(f);
+  // A NaN multiplier (global scale 0: inf * 0) makes every product NaN; cvt.satfinite maps NaN
+  // to +6 whatever its sign, the gfx950 converter keeps the sign, so this case is spelled out.
+  return (o != o) ? 0x77777777u : f32x8_to_e2m1x8(f);
 }
 
 // Row-major fast path: reduce dim contiguous, no swizzle, K % 8 == 0, 16-byte aligned rows.
@@ -174,8 +176,8 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_generic_kernel(
       f0[i] = bf16_bits_to_f32(h[i]) * o;
       f1[i] = bf16_bits_to_f32(h[8 + i]) * o;
     }
-    op[2 * b] = f32x8_to_e2m1x8(f0);
-    op[2 * b + 1] = f32x8_to_e2m1x8(f1);
+    op[2 * b] = (o != o) ? 0x77777777u : f32x8_to_e2m1x8(f0);
+    op[2 * b + 1] = (o != o) ? 0x77777777u : f32x8_to_e2m1x8(f1);
   }
   *sfp = sfw;
 }
