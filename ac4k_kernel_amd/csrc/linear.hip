@@ -10,6 +10,9 @@
 // fp16 values and one v_pk_mul_f16 applies the E4M3 block scale.  e2m1 * e4m3 has at most
 // 5 significant bits and lies in [2^-10, 2688], so the fp16 product is exact; the MFMA
 // (v_mfma_f32_32x32x16_f16, same rate as bf16) accumulates in fp32.
+#include <stdlib.h>
+#include <string.h>
+
 #include "ac4k_common.h"
 
 namespace ac4k {
@@ -215,22 +218,221 @@ __global__ __launch_bounds__(256) void linear_nvfp4_tile128_kernel(LinearArgs a)
   }
 }
 
+// ===========================================================================
+// 256x256x64 tile kernel for large problems: 4 waves (2x2), each wave 128x128 = 4x4 MFMA
+// 32x32x16 tiles (256 fp32 accumulators per lane).  A wave tile this large halves the LDS
+// fragment traffic per flop against 64x64 wave tiles.  LDS is double buffered (2 x 64 KiB):
+// while the MFMAs consume K-step kt from one buffer, the packed slice of step kt+1 (already
+// in registers) is decoded into the other and the packed slice of step kt+2 is fetched.
+// Thread t owns row t of the A tile and row t of the B tile: 32 packed bytes + one scale
+// dword per K-step each.  Requires K % 64 == 0.
+// ===========================================================================
+constexpr int L_BM = 256, L_BN = 256, L_BK = 64;
+constexpr int L_TILE_HALVES = L_BM * L_BK;  // fp16 elements per operand tile
+
+struct PackedRow {
+  uint4 lo, hi;  // 64 nibbles: four 16-blocks
+  uint32_t sf;   // their four scale bytes
+};
+
+// `row` is clamped by the caller: rows past the matrix read the last valid row and feed
+// accumulators whose outputs are never stored, so the load needs no predicate.
+__device__ __forceinline__ PackedRow load_row(const uint8_t *base, const uint32_t *sf, int64_t rows_p,
+                                              int64_t K, int64_t row, int64_t kt) {
+  PackedRow r;
+  const uint4 *p = reinterpret_cast<const uint4 *>(base + row * (K >> 1) + kt * 32);
+  r.lo = p[0];
+  r.hi = p[1];
+  r.sf = sf[kt * rows_p + row];
+  return r;
+}
+
+// decode 16-block `q` (0..3) of a packed row into its two 16-byte LDS chunks
+__device__ __forceinline__ void decode_block_to_lds(_Float16 *tile, int row, int q, uint32_t w0, uint32_t w1,
+                                                    uint32_t sfw) {
+  f16x2 sp = scale_pattern(sfw >> (8 * q));
+  f16x2 lo[4], hi[4];
+  decode8(w0, sp, lo);
+  decode8(w1, sp, hi);
+  uint4 v0 = make_uint4(__builtin_bit_cast(uint32_t, lo[0]), __builtin_bit_cast(uint32_t, lo[1]),
+                        __builtin_bit_cast(uint32_t, lo[2]), __builtin_bit_cast(uint32_t, lo[3]));
+  uint4 v1 = make_uint4(__builtin_bit_cast(uint32_t, hi[0]), __builtin_bit_cast(uint32_t, hi[1]),
+                        __builtin_bit_cast(uint32_t, hi[2]), __builtin_bit_cast(uint32_t, hi[3]));
+  *reinterpret_cast<uint4 *>(tile + row * 64 + (((2 * q) ^ (row & 7)) << 3)) = v0;
+  *reinterpret_cast<uint4 *>(tile + row * 64 + (((2 * q + 1) ^ (row & 7)) << 3)) = v1;
+}
+
+__device__ __forceinline__ void decode_row_quarter(_Float16 *tile, int row, int q, const PackedRow &r) {
+  const uint32_t w[8] = {r.lo.x, r.lo.y, r.lo.z, r.lo.w, r.hi.x, r.hi.y, r.hi.z, r.hi.w};
+  decode_block_to_lds(tile, row, q, w[2 * q], w[2 * q + 1], r.sf);
+}
+
+struct Frags {
+  f16x8 a[4], b[4];
+};
+
+__device__ __forceinline__ void load_frags(Frags &f, const _Float16 *cA, const _Float16 *cB, int arow, int brow,
+                                           int chunk) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f.a[i] = lds_frag(cA, arow + i * 32, chunk);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) f.b[j] = lds_frag(cB, brow + j * 32, chunk);
+}
+
 template <int D_DT, int BIAS_DT>
-static void launch_tile128(const LinearArgs &a, hipStream_t st) {
+__global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256_kernel(LinearArgs a) {
+  extern __shared__ __attribute__((aligned(16))) _Float16 lds[];  // [2 buffers][A tile | B tile]
+
+  const int64_t tiles_m = ceil_div(a.M, L_BM), tiles_n = ceil_div(a.N, L_BN);
+  const int64_t ntiles = tiles_m * tiles_n;
+  int64_t pid = blockIdx.x;
+  {  // contiguous run of tiles per XCD (workgroups are dealt round-robin to the 8 XCDs)
+    const int64_t per = ntiles / 8, rem = ntiles % 8;
+    const int64_t xcd = pid % 8, idx = pid / 8;
+    pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
+  }
+  constexpr int GROUP_M = 4;
+  const int64_t group = pid / (GROUP_M * tiles_n);
+  const int64_t first_m = group * GROUP_M;
+  const int64_t gsize = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+  const int64_t tm = first_m + (pid % (GROUP_M * tiles_n)) % gsize;
+  const int64_t tn = (pid % (GROUP_M * tiles_n)) / gsize;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  int64_t arow = tm * L_BM + tid, brow = tn * L_BN + tid;
+  arow = arow < a.M ? arow : a.M - 1;
+  brow = brow < a.N ? brow : a.N - 1;
+  const int nk = (int)(a.K / L_BK);
+  const int fa_row = wm * 128 + (lane & 31), fb_row = wn * 128 + (lane & 31), half = lane >> 5;
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  PackedRow ra = load_row(a.A, a.A_sf, a.Mp, a.K, arow, 0);
+  PackedRow rb = load_row(a.B, a.B_sf, a.Np, a.K, brow, 0);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    decode_row_quarter(lds, tid, q, ra);
+    decode_row_quarter(lds + L_TILE_HALVES, tid, q, rb);
+  }
+  ra = load_row(a.A, a.A_sf, a.Mp, a.K, arow, nk > 1 ? 1 : 0);
+  rb = load_row(a.B, a.B_sf, a.Np, a.K, brow, nk > 1 ? 1 : 0);
+  __syncthreads();
+
+  Frags f[2];
+  for (int kt = 0; kt < nk; ++kt) {
+    const _Float16 *cA = lds + (kt & 1) * (2 * L_TILE_HALVES);
+    const _Float16 *cB = cA + L_TILE_HALVES;
+    _Float16 *nA = lds + ((kt + 1) & 1) * (2 * L_TILE_HALVES);
+    _Float16 *nB = nA + L_TILE_HALVES;
+    load_frags(f[0], cA, cB, fa_row, fb_row, half);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      // fragments of the next sub-step and a quarter of the next K-step's decode are issued
+      // in the shadow of this sub-step's 16 MFMAs (the last step decodes a stale slice into
+      // the buffer nobody reads again)
+      if (ks < 3) load_frags(f[(ks + 1) & 1], cA, cB, fa_row, fb_row, (ks + 1) * 2 + half);
+      decode_row_quarter(nA, tid, ks, ra);
+      decode_row_quarter(nB, tid, ks, rb);
+      const Frags &c = f[ks & 1];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(c.a[i], c.b[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+      for (int g = 0; g < 16; ++g) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                   // 1 MFMA
+        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);                   // 3 VALU
+        if (g < 8 && ks < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
+        if (g >= 12) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);          // 1 LDS write
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keep the sub-steps apart
+    }
+    const int kn = kt + 2 < nk ? kt + 2 : nk - 1;
+    ra = load_row(a.A, a.A_sf, a.Mp, a.K, arow, kn);
+    rb = load_row(a.B, a.B_sf, a.Np, a.K, brow, kn);
+    __syncthreads();
+  }
+
+  const float scale = (*a.A_gs) * (*a.B_gs);
+  using DE = Elem<D_DT>;
+  typename DE::T *D = static_cast<typename DE::T *>(a.D);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int64_t n = tn * L_BN + wn * 128 + j * 32 + (lane & 31);
+    float bv = 0.0f;
+    if constexpr (BIAS_DT != BIAS_NONE) {
+      if (n < a.N) bv = Elem<BIAS_DT>::load(a.bias, n);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int64_t m = tm * L_BM + wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (m < a.M && n < a.N) {
+          float v = acc[i][j][e] * scale;
+          if constexpr (BIAS_DT != BIAS_NONE) v += bv;
+          D[m * a.N + n] = DE::cvt(v);
+        }
+      }
+    }
+  }
+}
+
+constexpr int L_LDS_BYTES = 2 * 2 * L_TILE_HALVES * (int)sizeof(_Float16);  // 128 KiB
+
+enum class LinearKernel { AUTO, TILE128, TILE256 };
+
+static LinearKernel forced_kernel() {  // benchmarking aid: AC4K_LINEAR_KERNEL=tile128|tile256
+  static const LinearKernel k = [] {
+    const char *e = getenv("AC4K_LINEAR_KERNEL");
+    if (e && !strcmp(e, "tile128")) return LinearKernel::TILE128;
+    if (e && !strcmp(e, "tile256")) return LinearKernel::TILE256;
+    return LinearKernel::AUTO;
+  }();
+  return k;
+}
+
+template <int D_DT, int BIAS_DT>
+static int launch_tile256(const LinearArgs &a, hipStream_t st) {
+  auto *kern = linear_nvfp4_tile256_kernel<D_DT, BIAS_DT>;
+  static bool attr_set = false;  // per instantiation; the attribute is idempotent
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, L_LDS_BYTES);
+    if (e != hipSuccess) return set_error("hipFuncSetAttribute(LDS=%d): %s", L_LDS_BYTES, hipGetErrorString(e));
+    attr_set = true;
+  }
+  const int64_t ntiles = ceil_div(a.M, L_BM) * ceil_div(a.N, L_BN);
+  hipLaunchKernelGGL(kern, dim3((unsigned)ntiles), dim3(256), L_LDS_BYTES, st, a);
+  return 0;
+}
+
+template <int D_DT, int BIAS_DT>
+static int launch_linear(const LinearArgs &a, hipStream_t st) {
+  LinearKernel k = forced_kernel();
+  const bool big_ok = a.K % L_BK == 0 && (((uintptr_t)a.A | (uintptr_t)a.B) & 15) == 0;
+  if (k == LinearKernel::AUTO) k = (big_ok && a.M > 128 && a.N > 128) ? LinearKernel::TILE256 : LinearKernel::TILE128;
+  if (k == LinearKernel::TILE256 && big_ok) return launch_tile256<D_DT, BIAS_DT>(a, st);
   const int64_t ntiles = ceil_div(a.M, T_BM) * ceil_div(a.N, T_BN);
   hipLaunchKernelGGL((linear_nvfp4_tile128_kernel<D_DT, BIAS_DT>), dim3((unsigned)ntiles), dim3(256), 0, st, a);
+  return 0;
 }
 
 template <int D_DT>
 static int dispatch_bias(const LinearArgs &a, int bias_dtype, hipStream_t st) {
-  if (!a.bias) {
-    launch_tile128<D_DT, BIAS_NONE>(a, st);
-    return 0;
-  }
+  if (!a.bias) return launch_linear<D_DT, BIAS_NONE>(a, st);
   switch (bias_dtype) {
-    case AC4K_DTYPE_BF16: launch_tile128<D_DT, AC4K_DTYPE_BF16>(a, st); return 0;
-    case AC4K_DTYPE_FP16: launch_tile128<D_DT, AC4K_DTYPE_FP16>(a, st); return 0;
-    case AC4K_DTYPE_FP32: launch_tile128<D_DT, AC4K_DTYPE_FP32>(a, st); return 0;
+    case AC4K_DTYPE_BF16: return launch_linear<D_DT, AC4K_DTYPE_BF16>(a, st);
+    case AC4K_DTYPE_FP16: return launch_linear<D_DT, AC4K_DTYPE_FP16>(a, st);
+    case AC4K_DTYPE_FP32: return launch_linear<D_DT, AC4K_DTYPE_FP32>(a, st);
   }
   return set_error("bias must be bfloat16, half or float (dtype tag %d)", bias_dtype);
 }
