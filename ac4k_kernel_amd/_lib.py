@@ -34,9 +34,11 @@ _lib = None
 def load() -> ctypes.CDLL:
     global _lib
     if _lib is None:
-        path = _build.LIB_PATH
-        if not os.path.exists(path):
-            _build.build()
+        path = os.environ.get("AC4K_NVFP4_LIB")  # a prebuilt library elsewhere (kernel experiments)
+        if not path:
+            path = _build.LIB_PATH
+            if not os.path.exists(path):
+                _build.build()
         lib = ctypes.CDLL(path)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol

@@ -36,19 +36,19 @@ def needs_build() -> bool:
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def build(force: bool = False, verbose: bool = True) -> str:
-    if not force and not needs_build():
+def build(force: bool = False, verbose: bool = True, extra_flags=(), out: str = LIB_PATH) -> str:
+    if not force and out == LIB_PATH and not needs_build():
         return LIB_PATH
-    cmd = [HIPCC] + FLAGS + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", LIB_PATH]
+    cmd = [HIPCC] + FLAGS + list(extra_flags) + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", out]
     if verbose:
         print("[ac4k build]", " ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in res.stdout.splitlines() if "is not a recognized feature for this target" not in l)
+    log = "\n".join(l for l in res.stdout.splitlines() if "is not a recognized feature for this target" not in l)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
-    if verbose and out.strip():
-        print(out)
-    return LIB_PATH
+        raise RuntimeError("hipcc failed:\n" + log)
+    if verbose and log.strip():
+        print(log)
+    return out
 
 
 if __name__ == "__main__":

@@ -263,6 +263,9 @@ __device__ __forceinline__ void decode_block_to_lds(_Float16 *tile, int row, int
 }
 
 __device__ __forceinline__ void decode_row_quarter(_Float16 *tile, int row, int q, const PackedRow &r) {
+#ifdef EXP_NO_DECODE
+  return;
+#endif
   const uint32_t w[8] = {r.lo.x, r.lo.y, r.lo.z, r.lo.w, r.hi.x, r.hi.y, r.hi.z, r.hi.w};
   decode_block_to_lds(tile, row, q, w[2 * q], w[2 * q + 1], r.sf);
 }
@@ -273,6 +276,9 @@ struct Frags {
 
 __device__ __forceinline__ void load_frags(Frags &f, const _Float16 *cA, const _Float16 *cB, int arow, int brow,
                                            int chunk) {
+#ifdef EXP_NO_LDSREAD
+  if (chunk >= 0) return;
+#endif
 #pragma unroll
   for (int i = 0; i < 4; ++i) f.a[i] = lds_frag(cA, arow + i * 32, chunk);
 #pragma unroll
@@ -314,51 +320,103 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256_kernel(LinearArgs
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  PackedRow ra = load_row(a.A, a.A_sf, a.Mp, a.K, arow, 0);
-  PackedRow rb = load_row(a.B, a.B_sf, a.Np, a.K, brow, 0);
+  // Software pipeline.  Step kt multiplies LDS buffer kt&1 while it decodes the packed slice of
+  // step kt+1 (held in registers since the previous step) into the other buffer; the packed
+  // slices of steps kt+2 / kt+3 are in flight in the second register set.  The decode is done
+  // in sub-steps 0..2, the workgroup barrier sits before sub-step 3, and sub-step 3's MFMAs
+  // cover the barrier skew, the first fragment loads of step kt+1 and the next global loads.
+  PackedRow ra0 = load_row(a.A, a.A_sf, a.Mp, a.K, arow, 0);
+  PackedRow rb0 = load_row(a.B, a.B_sf, a.Np, a.K, brow, 0);
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
-    decode_row_quarter(lds, tid, q, ra);
-    decode_row_quarter(lds + L_TILE_HALVES, tid, q, rb);
+    decode_row_quarter(lds, tid, q, ra0);
+    decode_row_quarter(lds + L_TILE_HALVES, tid, q, rb0);
   }
-  ra = load_row(a.A, a.A_sf, a.Mp, a.K, arow, nk > 1 ? 1 : 0);
-  rb = load_row(a.B, a.B_sf, a.Np, a.K, brow, nk > 1 ? 1 : 0);
+  const int klast = nk - 1;
+  ra0 = load_row(a.A, a.A_sf, a.Mp, a.K, arow, 1 < klast ? 1 : klast);
+  rb0 = load_row(a.B, a.B_sf, a.Np, a.K, brow, 1 < klast ? 1 : klast);
+  PackedRow ra1 = load_row(a.A, a.A_sf, a.Mp, a.K, arow, 2 < klast ? 2 : klast);
+  PackedRow rb1 = load_row(a.B, a.B_sf, a.Np, a.K, brow, 2 < klast ? 2 : klast);
   __syncthreads();
 
   Frags f[2];
-  for (int kt = 0; kt < nk; ++kt) {
+  load_frags(f[0], lds, lds + L_TILE_HALVES, fa_row, fb_row, half);
+
+  auto mfma16 = [&](const Frags &c) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(c.a[i], c.b[j], acc[i][j], 0, 0, 0);
+  };
+  // one K-step; da/db hold the packed slice of step kt+1 and are refilled with step kt+3
+  auto kstep = [&](int kt, PackedRow &da, PackedRow &db) {
     const _Float16 *cA = lds + (kt & 1) * (2 * L_TILE_HALVES);
     const _Float16 *cB = cA + L_TILE_HALVES;
     _Float16 *nA = lds + ((kt + 1) & 1) * (2 * L_TILE_HALVES);
     _Float16 *nB = nA + L_TILE_HALVES;
-    load_frags(f[0], cA, cB, fa_row, fb_row, half);
+    // sub-step 0
+    load_frags(f[1], cA, cB, fa_row, fb_row, 2 + half);
+    decode_row_quarter(nA, tid, 0, da);
+    decode_row_quarter(nA, tid, 1, da);
+    decode_row_quarter(nA, tid, 2, da);
+    mfma16(f[0]);
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      // fragments of the next sub-step and a quarter of the next K-step's decode are issued
-      // in the shadow of this sub-step's 16 MFMAs (the last step decodes a stale slice into
-      // the buffer nobody reads again)
-      if (ks < 3) load_frags(f[(ks + 1) & 1], cA, cB, fa_row, fb_row, (ks + 1) * 2 + half);
-      decode_row_quarter(nA, tid, ks, ra);
-      decode_row_quarter(nB, tid, ks, rb);
-      const Frags &c = f[ks & 1];
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(c.a[i], c.b[j], acc[i][j], 0, 0, 0);
-#pragma unroll
-      for (int g = 0; g < 16; ++g) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                   // 1 MFMA
-        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);                   // 3 VALU
-        if (g < 8 && ks < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
-        if (g >= 12) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);          // 1 LDS write
-      }
-      __builtin_amdgcn_sched_barrier(0);  // keep the sub-steps apart
+    for (int g = 0; g < 16; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      if (g < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if (g >= 10) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
     }
-    const int kn = kt + 2 < nk ? kt + 2 : nk - 1;
-    ra = load_row(a.A, a.A_sf, a.Mp, a.K, arow, kn);
-    rb = load_row(a.B, a.B_sf, a.Np, a.K, brow, kn);
-    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    // sub-step 1
+    load_frags(f[0], cA, cB, fa_row, fb_row, 4 + half);
+    decode_row_quarter(nA, tid, 3, da);
+    decode_row_quarter(nB, tid, 0, db);
+    decode_row_quarter(nB, tid, 1, db);
+    mfma16(f[1]);
+#pragma unroll
+    for (int g = 0; g < 16; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      if (g < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if (g >= 10) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // sub-step 2
+    load_frags(f[1], cA, cB, fa_row, fb_row, 6 + half);
+    decode_row_quarter(nB, tid, 2, db);
+    decode_row_quarter(nB, tid, 3, db);
+    mfma16(f[0]);
+#pragma unroll
+    for (int g = 0; g < 16; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+      if (g < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if (g >= 12) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();  // buffer (kt+1)&1 is complete, buffer kt&1 has been read by everyone
+    // sub-step 3
+    load_frags(f[0], nA, nB, fa_row, fb_row, half);
+    const int kn = kt + 3 < klast ? kt + 3 : klast;
+    da = load_row(a.A, a.A_sf, a.Mp, a.K, arow, kn);
+    db = load_row(a.B, a.B_sf, a.Np, a.K, brow, kn);
+    mfma16(f[1]);
+#pragma unroll
+    for (int g = 0; g < 16; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+      if (g < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if (g >= 8 && g < 14) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  for (int kt = 0; kt < nk; ++kt) {
+    PackedRow na = ra1, nb = rb1;
+    kstep(kt, ra0, rb0);   // consumes ra0/rb0 (step kt+1), refills them with step kt+3
+    ra1 = ra0; rb1 = rb0;  // rotate: next step decodes the old ra1/rb1 (step kt+2)
+    ra0 = na; rb0 = nb;
   }
 
   const float scale = (*a.A_gs) * (*a.B_gs);
