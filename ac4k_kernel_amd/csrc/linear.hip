@@ -13,6 +13,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <type_traits>
+
 #include "ac4k_common.h"
 
 namespace ac4k {
@@ -79,9 +81,12 @@ __device__ __forceinline__ void decode8(uint32_t w, f16x2 sp, f16x2 (&h)[4]) {
 // ===========================================================================
 // 128x128x64 tile kernel, 4 waves (2x2), each wave 64x64 = 2x2 MFMA 32x32x16 tiles.
 // LDS holds the decoded fp16 tiles: row pitch 128 B (64 k), 16-byte chunk index XORed with
-// (row & 7) so that both the decode stores and the MFMA fragment loads are conflict-free.
+// LDS_SWZ(row) so that both the decode stores and the MFMA fragment loads are conflict-free.
 // ===========================================================================
 constexpr int T_BM = 128, T_BN = 128, T_BK = 64;
+#ifndef LDS_SWZ
+#define LDS_SWZ(row) ((row) & 7)
+#endif
 
 struct PackedRegs {
   uint2 d[2];    // two 16-blocks (8 bytes each) of this thread's row
@@ -120,13 +125,13 @@ __device__ __forceinline__ void decode_to_lds(_Float16 *tile, int row, int half,
                           __builtin_bit_cast(uint32_t, lo[2]), __builtin_bit_cast(uint32_t, lo[3]));
     uint4 v1 = make_uint4(__builtin_bit_cast(uint32_t, hi[0]), __builtin_bit_cast(uint32_t, hi[1]),
                           __builtin_bit_cast(uint32_t, hi[2]), __builtin_bit_cast(uint32_t, hi[3]));
-    *reinterpret_cast<uint4 *>(tile + row * 64 + ((c0 ^ (row & 7)) << 3)) = v0;
-    *reinterpret_cast<uint4 *>(tile + row * 64 + (((c0 + 1) ^ (row & 7)) << 3)) = v1;
+    *reinterpret_cast<uint4 *>(tile + row * 64 + ((c0 ^ LDS_SWZ(row)) << 3)) = v0;
+    *reinterpret_cast<uint4 *>(tile + row * 64 + (((c0 + 1) ^ LDS_SWZ(row)) << 3)) = v1;
   }
 }
 
 __device__ __forceinline__ f16x8 lds_frag(const _Float16 *tile, int row, int chunk) {
-  return *reinterpret_cast<const f16x8 *>(tile + row * 64 + ((chunk ^ (row & 7)) << 3));
+  return *reinterpret_cast<const f16x8 *>(tile + row * 64 + ((chunk ^ LDS_SWZ(row)) << 3));
 }
 
 template <int D_DT, int BIAS_DT>
@@ -250,22 +255,31 @@ __device__ __forceinline__ PackedRow load_row(const uint8_t *base, const uint32_
 // decode 16-block `q` (0..3) of a packed row into its two 16-byte LDS chunks
 __device__ __forceinline__ void decode_block_to_lds(_Float16 *tile, int row, int q, uint32_t w0, uint32_t w1,
                                                     uint32_t sfw) {
+#ifdef EXP_NO_DECODE
+  return;
+#endif
   f16x2 sp = scale_pattern(sfw >> (8 * q));
   f16x2 lo[4], hi[4];
+#ifdef EXP_NO_VALU
+  for (int i = 0; i < 4; ++i) { lo[i] = __builtin_bit_cast(f16x2, w0); hi[i] = __builtin_bit_cast(f16x2, w1 + sfw); }
+#else
   decode8(w0, sp, lo);
   decode8(w1, sp, hi);
+#endif
+#ifdef EXP_NO_WRITE
+  if (__builtin_bit_cast(uint32_t, lo[0]) != 0x12345678u || __builtin_bit_cast(uint32_t, hi[3]) != 0x9abcdef0u ||
+      __builtin_bit_cast(uint32_t, lo[1]) + __builtin_bit_cast(uint32_t, lo[2]) + __builtin_bit_cast(uint32_t, lo[3]) +
+      __builtin_bit_cast(uint32_t, hi[0]) + __builtin_bit_cast(uint32_t, hi[1]) + __builtin_bit_cast(uint32_t, hi[2]) != 0x1111u) return;
+#endif
   uint4 v0 = make_uint4(__builtin_bit_cast(uint32_t, lo[0]), __builtin_bit_cast(uint32_t, lo[1]),
                         __builtin_bit_cast(uint32_t, lo[2]), __builtin_bit_cast(uint32_t, lo[3]));
   uint4 v1 = make_uint4(__builtin_bit_cast(uint32_t, hi[0]), __builtin_bit_cast(uint32_t, hi[1]),
                         __builtin_bit_cast(uint32_t, hi[2]), __builtin_bit_cast(uint32_t, hi[3]));
-  *reinterpret_cast<uint4 *>(tile + row * 64 + (((2 * q) ^ (row & 7)) << 3)) = v0;
-  *reinterpret_cast<uint4 *>(tile + row * 64 + (((2 * q + 1) ^ (row & 7)) << 3)) = v1;
+  *reinterpret_cast<uint4 *>(tile + row * 64 + (((2 * q) ^ LDS_SWZ(row)) << 3)) = v0;
+  *reinterpret_cast<uint4 *>(tile + row * 64 + (((2 * q + 1) ^ LDS_SWZ(row)) << 3)) = v1;
 }
 
 __device__ __forceinline__ void decode_row_quarter(_Float16 *tile, int row, int q, const PackedRow &r) {
-#ifdef EXP_NO_DECODE
-  return;
-#endif
   const uint32_t w[8] = {r.lo.x, r.lo.y, r.lo.z, r.lo.w, r.hi.x, r.hi.y, r.hi.z, r.hi.w};
   decode_block_to_lds(tile, row, q, w[2 * q], w[2 * q + 1], r.sf);
 }
@@ -444,18 +458,540 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256_kernel(LinearArgs
   }
 }
 
+// ===========================================================================
+// 256x256x64 tile, 8 waves (2 x 4), each wave 128x64 = 4x2 MFMA tiles (128 accumulators).
+// Two waves share every SIMD, so one wave's decode VALU work, LDS stores and fragment loads
+// issue while the other wave's MFMAs run; a single wave per SIMD cannot overlap them because
+// it issues in order and an LDS store alone holds its issue port for ~32 cycles.
+// Thread t owns half a row (32 nibbles = two 16-blocks) of the A tile and of the B tile.
+// ===========================================================================
+struct PackedHalfRow {
+  uint4 d;      // 32 nibbles: two 16-blocks
+  uint32_t sf;  // scale dword of the row's 64-chunk (this thread uses two of its bytes)
+};
+
+__device__ __forceinline__ PackedHalfRow load_half_row(const uint8_t *base, const uint32_t *sf, int64_t rows_p,
+                                                       int64_t K, int64_t row, int half, int kt) {
+  PackedHalfRow r;
+  r.d = *reinterpret_cast<const uint4 *>(base + row * (K >> 1) + (int64_t)kt * 32 + half * 16);
+  r.sf = sf[(int64_t)kt * rows_p + row];
+  return r;
+}
+
+// block b (0/1) of a thread's half row -> its two 16-byte LDS chunks
+__device__ __forceinline__ void decode_half_block(_Float16 *tile, int row, int half, int b, const PackedHalfRow &r) {
+  const uint32_t w0 = b ? r.d.z : r.d.x, w1 = b ? r.d.w : r.d.y;
+  decode_block_to_lds(tile, row, half * 2 + b, w0, w1, r.sf);
+}
+
+template <int D_DT, int BIAS_DT>
+__global__ __launch_bounds__(512) void linear_nvfp4_tile256w8_kernel(LinearArgs a) {
+  extern __shared__ __attribute__((aligned(16))) _Float16 lds[];  // [2 buffers][A tile | B tile]
+
+  const int64_t tiles_m = ceil_div(a.M, L_BM), tiles_n = ceil_div(a.N, L_BN);
+  const int64_t ntiles = tiles_m * tiles_n;
+  int64_t pid = blockIdx.x;
+  {  // contiguous run of tiles per XCD (workgroups are dealt round-robin to the 8 XCDs)
+    const int64_t per = ntiles / 8, rem = ntiles % 8;
+    const int64_t xcd = pid % 8, idx = pid / 8;
+    pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
+  }
+  constexpr int GROUP_M = 4;
+  const int64_t group = pid / (GROUP_M * tiles_n);
+  const int64_t first_m = group * GROUP_M;
+  const int64_t gsize = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+  const int64_t tm = first_m + (pid % (GROUP_M * tiles_n)) % gsize;
+  const int64_t tn = (pid % (GROUP_M * tiles_n)) / gsize;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 2, wn = wave & 3;
+  const int ld_row = tid >> 1, ld_half = tid & 1;
+  int64_t arow = tm * L_BM + ld_row, brow = tn * L_BN + ld_row;
+  arow = arow < a.M ? arow : a.M - 1;  // rows past the matrix feed accumulators that are never stored
+  brow = brow < a.N ? brow : a.N - 1;
+  const int nk = (int)(a.K / L_BK), klast = nk - 1;
+  const int fa_row = wm * 128 + (lane & 31), fb_row = wn * 64 + (lane & 31), half = lane >> 5;
+
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  PackedHalfRow ra0 = load_half_row(a.A, a.A_sf, a.Mp, a.K, arow, ld_half, 0);
+  PackedHalfRow rb0 = load_half_row(a.B, a.B_sf, a.Np, a.K, brow, ld_half, 0);
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    decode_half_block(lds, ld_row, ld_half, b, ra0);
+    decode_half_block(lds + L_TILE_HALVES, ld_row, ld_half, b, rb0);
+  }
+  ra0 = load_half_row(a.A, a.A_sf, a.Mp, a.K, arow, ld_half, 1 < klast ? 1 : klast);
+  rb0 = load_half_row(a.B, a.B_sf, a.Np, a.K, brow, ld_half, 1 < klast ? 1 : klast);
+  PackedHalfRow ra1 = load_half_row(a.A, a.A_sf, a.Mp, a.K, arow, ld_half, 2 < klast ? 2 : klast);
+  PackedHalfRow rb1 = load_half_row(a.B, a.B_sf, a.Np, a.K, brow, ld_half, 2 < klast ? 2 : klast);
+  __syncthreads();
+
+  f16x8 fa[4], fb[2];
+  auto frags = [&](const _Float16 *cA, const _Float16 *cB, int ks) {
+#ifdef EXP_NO_LDSREAD
+    if (ks >= 0) return;
+#endif
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fa[i] = lds_frag(cA, fa_row + i * 32, ks * 2 + half);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) fb[j] = lds_frag(cB, fb_row + j * 32, ks * 2 + half);
+  };
+  auto mfma8 = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+  };
+
+  for (int kt = 0; kt < nk; ++kt) {
+    const _Float16 *cA = lds + (kt & 1) * (2 * L_TILE_HALVES);
+    const _Float16 *cB = cA + L_TILE_HALVES;
+    _Float16 *nA = lds + ((kt + 1) & 1) * (2 * L_TILE_HALVES);
+    _Float16 *nB = nA + L_TILE_HALVES;
+    // ra0/rb0 hold step kt+1 (decoded now), ra1/rb1 hold step kt+2 (possibly still in flight)
+    frags(cA, cB, 0);
+    decode_half_block(nA, ld_row, ld_half, 0, ra0);
+    decode_half_block(nA, ld_row, ld_half, 1, ra0);
+    mfma8();
+    frags(cA, cB, 1);
+    decode_half_block(nB, ld_row, ld_half, 0, rb0);
+    mfma8();
+    frags(cA, cB, 2);
+    decode_half_block(nB, ld_row, ld_half, 1, rb0);
+    mfma8();
+    frags(cA, cB, 3);
+    __syncthreads();  // next buffer complete; nobody reads the current buffer any more
+    const int kn = kt + 3 < klast ? kt + 3 : klast;
+    ra0 = ra1;
+    rb0 = rb1;
+    ra1 = load_half_row(a.A, a.A_sf, a.Mp, a.K, arow, ld_half, kn);
+    rb1 = load_half_row(a.B, a.B_sf, a.Np, a.K, brow, ld_half, kn);
+    mfma8();
+  }
+
+  const float scale = (*a.A_gs) * (*a.B_gs);
+  using DE = Elem<D_DT>;
+  typename DE::T *D = static_cast<typename DE::T *>(a.D);
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int64_t n = tn * L_BN + wn * 64 + j * 32 + (lane & 31);
+    float bv = 0.0f;
+    if constexpr (BIAS_DT != BIAS_NONE) {
+      if (n < a.N) bv = Elem<BIAS_DT>::load(a.bias, n);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int64_t m = tm * L_BM + wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (m < a.M && n < a.N) {
+          float v = acc[i][j][e] * scale;
+          if constexpr (BIAS_DT != BIAS_NONE) v += bv;
+          D[m * a.N + n] = DE::cvt(v);
+        }
+      }
+    }
+  }
+}
+
+// ===========================================================================
+// 256x256 tile, packed operands in LDS, decode after the fragment load.
+//
+// The packed A/B slices and their scale dwords go from global memory straight into LDS with
+// LDS-DMA loads (global_load_lds: no VGPR staging, no LDS store instruction), three stages of
+// 128 k each.  A wave (4 waves, 2x2, 128x128 each) reads for every 32-row fragment ONE 16-byte
+// word per lane per 64-chunk: lane (row r, half h) owns elements [32h, 32h+32) of the chunk;
+// dword s of that word feeds MFMA sub-step s.  The same k-slot assignment is used for A and
+// B, so the permutation of k inside a chunk cancels in the dot product.  Decode per dword:
+// 4 x v_cvt_scalef32_pk_f16_fp4 + 4 x v_pk_mul_f16 by the block scale (E4M3 -> fp16 with
+// v_cvt_scalef32_pk_f16_fp8, splat through op_sel), i.e. 4 VALU per MFMA, which issue in the
+// shadow of the previous MFMA.  There is one workgroup barrier per 128 k, placed in the
+// middle of the step so that the next stage is readable before the current one ends.
+// Requires K % 128 == 0 and 16-byte aligned operands.
+// ===========================================================================
+constexpr int P_BK = 128;                       // k per stage (two 64-chunks)
+constexpr int P_STAGES = 3;
+constexpr int P_ROW = 64;                       // packed bytes per row per stage: [chunk][half] x 16 B
+constexpr int P_OFF_B = 256 * P_ROW;            // B rows follow the 256 A rows
+constexpr int P_OFF_SFA = 2 * 256 * P_ROW;      // scale dwords: [chunk][256 rows]
+constexpr int P_OFF_SFB = P_OFF_SFA + 2 * 1024;
+constexpr int P_STAGE_BYTES = P_OFF_SFB + 2 * 1024;  // 36864
+constexpr int P_LDS_BYTES = P_STAGES * P_STAGE_BYTES;
+
+// LDS-DMA: global_load_lds with a scalar 64-bit base, a 32-bit lane offset and the LDS
+// destination of lane 0 in M0 (lane l lands at M0 + size * l).  Issued through inline asm so
+// that the compiler's wait-count insertion does not see these loads: with the builtin it puts
+// s_waitcnt vmcnt(0) in front of every later LDS read, which serialises the prefetch.  The
+// kernel waits with explicit s_waitcnt vmcnt(..) before the barrier that publishes a stage.
+__device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :: "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+__device__ __forceinline__ void dma4(const void *sbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :: "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+
+struct DecFrags {
+  f16x8 a[4], b[4];
+};
+
+// dword `w` (8 nibbles) times block scale `sc` (both halves of `sc2` hold candidates, HI picks)
+template <bool HI>
+__device__ __forceinline__ f16x8 decode_dword(uint32_t w, f16x2 sc2) {
+  const f16x2 sc = HI ? (f16x2){sc2.y, sc2.y} : (f16x2){sc2.x, sc2.x};
+  f16x2 d0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 0) * sc;
+  f16x2 d1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 1) * sc;
+  f16x2 d2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 2) * sc;
+  f16x2 d3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 3) * sc;
+  return (f16x8){d0.x, d0.y, d1.x, d1.y, d2.x, d2.y, d3.x, d3.y};
+}
+
+template <int S>
+__device__ __forceinline__ uint32_t dword_of(const uint4 &v) {
+  return S == 0 ? v.x : S == 1 ? v.y : S == 2 ? v.z : v.w;
+}
+
+template <int D_DT, int BIAS_DT>
+__global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char plds[];
+
+  const int64_t tiles_m = ceil_div(a.M, L_BM), tiles_n = ceil_div(a.N, L_BN);
+  const int64_t ntiles = tiles_m * tiles_n;
+  int64_t pid = blockIdx.x;
+  {  // contiguous run of tiles per XCD (workgroups are dealt round-robin to the 8 XCDs)
+    const int64_t per = ntiles / 8, rem = ntiles % 8;
+    const int64_t xcd = pid % 8, idx = pid / 8;
+    pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
+  }
+  constexpr int GROUP_M = 4;
+  const int64_t group = pid / (GROUP_M * tiles_n);
+  const int64_t first_m = group * GROUP_M;
+  const int64_t gsize = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+  const int64_t tm = first_m + (pid % (GROUP_M * tiles_n)) % gsize;
+  const int64_t tn = (pid % (GROUP_M * tiles_n)) / gsize;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int half = lane >> 5;
+  const int nkt = (int)(a.K / P_BK);
+
+  // LDS-DMA.  One transfer moves 16 rows x 64 B: lane l reads piece l%4 of row l/4, so four
+  // adjacent lanes cover one 64-byte sector, and lands at LDS base + 16*l, i.e. row-major 64-byte
+  // rows.  Per operand a wave moves its 64 rows in 4 transfers; the 32-bit lane offset is loop
+  // invariant and the 64-bit part is a scalar base that advances by 64 bytes per stage.
+  const int swave = __builtin_amdgcn_readfirstlane(wave);
+  const int64_t kb = a.K >> 1;
+  uint32_t offA[4], offB[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    int64_t ra = (swave * 4 + q) * 16 + (lane >> 2), rb = ra;
+    ra = tm * L_BM + ra < a.M ? ra : a.M - 1 - tm * L_BM;  // rows past the matrix read the last valid row
+    rb = tn * L_BN + rb < a.N ? rb : a.N - 1 - tn * L_BN;
+    offA[q] = (uint32_t)(ra * kb + (lane & 3) * 16);
+    offB[q] = (uint32_t)(rb * kb + (lane & 3) * 16);
+  }
+  auto uniform_ptr = [](const void *p) {  // pin a wave-uniform pointer to scalar registers
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
+  };
+  const uint8_t *baseA = uniform_ptr(a.A + tm * L_BM * kb), *baseB = uniform_ptr(a.B + tn * L_BN * kb);
+  int64_t sra = tm * L_BM + swave * 64 + lane, srb = tn * L_BN + swave * 64 + lane;
+  sra = sra < a.Mp ? sra : a.Mp - 1;
+  srb = srb < a.Np ? srb : a.Np - 1;
+  const uint32_t offSA = (uint32_t)sra * 4u, offSB = (uint32_t)srb * 4u;  // byte offsets inside a scale plane
+  const uint8_t *sfA8 = uniform_ptr(a.A_sf), *sfB8 = uniform_ptr(a.B_sf);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)plds;
+  // `kt` may run past the last stage: the source is clamped (re-reading the last slice) and the
+  // destination is a stage buffer nobody reads again, which keeps the main loop free of branches
+  auto issue_piece = [&](int kt_dst, int q) {
+    const uint32_t st = lds_base + (kt_dst % P_STAGES) * P_STAGE_BYTES;
+    const int kt = kt_dst < nkt ? kt_dst : nkt - 1;
+    if (q < 8) {
+      const int r = q >> 1;
+      if (q & 1)
+        dma16(baseB + (int64_t)kt * P_ROW, offB[r], st + P_OFF_B + (swave * 4 + r) * 1024);
+      else
+        dma16(baseA + (int64_t)kt * P_ROW, offA[r], st + (swave * 4 + r) * 1024);
+    } else {
+      const int c = (q - 8) >> 1;
+      if (q & 1)
+        dma4(sfB8 + ((int64_t)kt * 2 + c) * a.Np * 4, offSB, st + P_OFF_SFB + c * 1024 + swave * 256);
+      else
+        dma4(sfA8 + ((int64_t)kt * 2 + c) * a.Mp * 4, offSA, st + P_OFF_SFA + c * 1024 + swave * 256);
+    }
+  };
+  auto issue_stage = [&](int kt) {
+#pragma unroll
+    for (int q = 0; q < 12; ++q) issue_piece(kt, q);
+  };
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  // fragment addresses inside a stage (bytes)
+  const int fa_off = (wm * 128 + (lane & 31)) * P_ROW + half * 16;
+  const int fb_off = P_OFF_B + (wn * 128 + (lane & 31)) * P_ROW + half * 16;
+  const int sa_off = P_OFF_SFA + (wm * 128 + (lane & 31)) * 4;
+  const int sb_off = P_OFF_SFB + (wn * 128 + (lane & 31)) * 4;
+  const int sh = half * 16;
+
+  uint4 PA[2][4], PB[2][4];  // packed fragments of a 64-chunk, double buffered by chunk parity
+  f16x2 SA[2][4], SB[2][4];  // their two block scales (blocks 2*half, 2*half+1) as fp16
+  auto load_chunk = [&](int kt, int c) {
+    const char *st = plds + (kt % P_STAGES) * P_STAGE_BYTES;
+#ifdef EXP_NO_LDSREAD
+    if (kt > 0) return;
+#endif
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      PA[c][i] = *reinterpret_cast<const uint4 *>(st + fa_off + c * 32 + i * 32 * P_ROW);
+      PB[c][i] = *reinterpret_cast<const uint4 *>(st + fb_off + c * 32 + i * 32 * P_ROW);
+      uint32_t wa = *reinterpret_cast<const uint32_t *>(st + sa_off + c * 1024 + i * 128);
+      uint32_t wb = *reinterpret_cast<const uint32_t *>(st + sb_off + c * 1024 + i * 128);
+      SA[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((wa >> sh) & 0x7f7fu, 1.0f, false);
+      SB[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((wb >> sh) & 0x7f7fu, 1.0f, false);
+    }
+  };
+
+  DecFrags D[2];
+  auto decode = [&](DecFrags &d, int c, auto S) {
+    constexpr int s = decltype(S)::value;
+#ifdef EXP_NO_DEC
+    if (c >= 0) return;
+#endif
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      d.a[i] = decode_dword<(s >= 2)>(dword_of<s>(PA[c][i]), SA[c][i]);
+      d.b[i] = decode_dword<(s >= 2)>(dword_of<s>(PB[c][i]), SB[c][i]);
+    }
+  };
+  auto mfma16 = [&](const DecFrags &d) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(d.b[j], d.a[i], acc[i][j], 0, 0, 0);  // D^T block
+  };
+  auto interleave = [&]() {  // 16 x (1 MFMA, 4 VALU): the decode rides in the MFMA shadow
+#pragma unroll
+    for (int g = 0; g < 16; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+
+  // prologue: stages 0 and 1 in flight, stage 0 visible, chunk 0 fragments and first decode
+  issue_stage(0);
+  if (nkt > 1) issue_stage(1);
+  if (nkt > 1) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  load_chunk(0, 0);
+  decode(D[0], 0, I0{});
+
+#ifdef EXP_TIMING
+  long long tA = 0, tB = 0, tC = 0, tprev = __builtin_readcyclecounter(), tstart = tprev;
+  const long long rt0 = wall_clock64();
+#define TPOINT(acc_) { long long tn_ = __builtin_readcyclecounter(); acc_ += tn_ - tprev; tprev = tn_; }
+#else
+#define TPOINT(acc_)
+#endif
+  for (int kt = 0; kt < nkt; ++kt) {
+    // chunk 0: sub-steps 0..3 (fragments of chunk 1 are fetched meanwhile)
+    load_chunk(kt, 1);
+    decode(D[1], 0, I1{});
+    mfma16(D[0]);
+    interleave();
+    decode(D[0], 0, I2{});
+    mfma16(D[1]);
+    interleave();
+    decode(D[1], 0, I3{});
+    mfma16(D[0]);
+    interleave();
+    decode(D[0], 1, I0{});
+    mfma16(D[1]);
+    interleave();
+    // stage kt+1 must be complete (own DMA done, then everybody's); stage kt-1 is free after this
+    TPOINT(tA)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    TPOINT(tB)
+    // chunk 1: sub-steps 4..7 (chunk 0 of the next stage is fetched meanwhile); the DMA of stage
+    // kt+2 is spread over these sub-steps
+    decode(D[1], 1, I1{});
+#ifndef EXP_NO_DMA
+    issue_piece(kt + 2, 0); issue_piece(kt + 2, 1); issue_piece(kt + 2, 8);
+#endif
+    mfma16(D[0]);
+    interleave();
+    load_chunk(kt + 1, 0);  // past the end this reads a stale stage; the result is never used
+    decode(D[0], 1, I2{});
+#ifndef EXP_NO_DMA
+    issue_piece(kt + 2, 2); issue_piece(kt + 2, 3); issue_piece(kt + 2, 9);
+#endif
+    mfma16(D[1]);
+    interleave();
+    decode(D[1], 1, I3{});
+#ifndef EXP_NO_DMA
+    issue_piece(kt + 2, 4); issue_piece(kt + 2, 5); issue_piece(kt + 2, 10);
+#endif
+    mfma16(D[0]);
+    interleave();
+    decode(D[0], 0, I0{});  // first sub-step of the next stage (unused after the last step)
+#ifndef EXP_NO_DMA
+    issue_piece(kt + 2, 6); issue_piece(kt + 2, 7); issue_piece(kt + 2, 11);
+#endif
+    mfma16(D[1]);
+    interleave();
+    TPOINT(tC)
+  }
+#ifdef EXP_TIMING
+  long long tloop = __builtin_readcyclecounter() - tstart;
+#endif
+
+  // ---- epilogue.  The MFMAs were issued with the operands swapped, so acc[i][j] holds the
+  // TRANSPOSED 32x32 block: lane l, element e <-> n = j*32 + (e>>2)*8 + (l>>5)*4 + (e&3),
+  // m = i*32 + (l&31): four consecutive n per lane.  2-byte outputs are staged through LDS (free
+  // now) so that every lane stores 16 bytes and a wave store covers whole 256-byte row segments.
+  const float scale = (*a.A_gs) * (*a.B_gs);
+  using DE = Elem<D_DT>;
+  typename DE::T *Dp = static_cast<typename DE::T *>(a.D);
+  const int64_t m0 = tm * L_BM + wm * 128, n0 = tn * L_BN + wn * 128;
+  float bias4[4][4][4];  // [j][g][e&3]
+  if constexpr (BIAS_DT != BIAS_NONE) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int64_t n = n0 + j * 32 + g * 8 + half * 4 + q;
+          bias4[j][g][q] = n < a.N ? Elem<BIAS_DT>::load(a.bias, n) : 0.0f;
+        }
+  }
+  auto value = [&](int i, int j, int e) {
+    float v = acc[i][j][e] * scale;
+    if constexpr (BIAS_DT != BIAS_NONE) v += bias4[j][e >> 2][e & 3];
+    return v;
+  };
+  const bool vec_ok = sizeof(typename DE::T) == 2 && (a.N % 8 == 0) && ((uintptr_t)a.D % 16 == 0);
+  if (vec_ok) {
+    constexpr int PITCH = 272;  // bytes per staged row: 128 outputs + 16 bytes of padding
+    __syncthreads();            // every wave is done reading the operand stages
+    char *stg = plds + wave * (64 * PITCH);
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii) {
+        const int i = 2 * p + ii;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            typename DE::T h[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) h[q] = DE::cvt(value(i, j, g * 4 + q));
+            uint2 w;
+            __builtin_memcpy(&w, h, 8);
+            *reinterpret_cast<uint2 *>(stg + (ii * 32 + (lane & 31)) * PITCH + (j * 32 + g * 8 + half * 4) * 2) = w;
+          }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the staging region is private to the wave
+#pragma unroll
+      for (int it = 0; it < 16; ++it) {
+        const int id = it * 64 + lane, row = id >> 4, q = id & 15;
+        const uint4 v = *reinterpret_cast<const uint4 *>(stg + row * PITCH + q * 16);
+        const int64_t m = m0 + p * 64 + row, n = n0 + q * 8;
+        if (m < a.M && n < a.N) *reinterpret_cast<uint4 *>(Dp + m * a.N + n) = v;
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t m = m0 + i * 32 + (lane & 31);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int64_t n = n0 + j * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+          if (m < a.M && n < a.N) Dp[m * a.N + n] = DE::cvt(value(i, j, e));
+        }
+    }
+  }
+#ifdef EXP_TIMING
+  if (blockIdx.x == 0 && tid == 0) {
+    long long tend = __builtin_readcyclecounter();
+    Dp[0] = DE::cvt((float)tA); Dp[1] = DE::cvt((float)tB); Dp[2] = DE::cvt((float)tC);
+    Dp[3] = DE::cvt((float)tloop); Dp[4] = DE::cvt((float)(tend - tstart)); Dp[5] = DE::cvt((float)(wall_clock64() - rt0));
+  }
+#endif
+}
+
+template <int D_DT, int BIAS_DT>
+static int launch_tile256p(const LinearArgs &a, hipStream_t st) {
+  auto *kern = linear_nvfp4_tile256p_kernel<D_DT, BIAS_DT>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, P_LDS_BYTES);
+    if (e != hipSuccess) return set_error("hipFuncSetAttribute(LDS=%d): %s", P_LDS_BYTES, hipGetErrorString(e));
+    attr_set = true;
+  }
+  const int64_t ntiles = ceil_div(a.M, L_BM) * ceil_div(a.N, L_BN);
+  hipLaunchKernelGGL(kern, dim3((unsigned)ntiles), dim3(256), P_LDS_BYTES, st, a);
+  return 0;
+}
+
 constexpr int L_LDS_BYTES = 2 * 2 * L_TILE_HALVES * (int)sizeof(_Float16);  // 128 KiB
 
-enum class LinearKernel { AUTO, TILE128, TILE256 };
+enum class LinearKernel { AUTO, TILE128, TILE256, TILE256W8, TILE256P };
 
 static LinearKernel forced_kernel() {  // benchmarking aid: AC4K_LINEAR_KERNEL=tile128|tile256
   static const LinearKernel k = [] {
     const char *e = getenv("AC4K_LINEAR_KERNEL");
     if (e && !strcmp(e, "tile128")) return LinearKernel::TILE128;
     if (e && !strcmp(e, "tile256")) return LinearKernel::TILE256;
+    if (e && !strcmp(e, "tile256w8")) return LinearKernel::TILE256W8;
+    if (e && !strcmp(e, "tile256p")) return LinearKernel::TILE256P;
     return LinearKernel::AUTO;
   }();
   return k;
+}
+
+template <int D_DT, int BIAS_DT>
+static int launch_tile256w8(const LinearArgs &a, hipStream_t st) {
+  auto *kern = linear_nvfp4_tile256w8_kernel<D_DT, BIAS_DT>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, L_LDS_BYTES);
+    if (e != hipSuccess) return set_error("hipFuncSetAttribute(LDS=%d): %s", L_LDS_BYTES, hipGetErrorString(e));
+    attr_set = true;
+  }
+  const int64_t ntiles = ceil_div(a.M, L_BM) * ceil_div(a.N, L_BN);
+  hipLaunchKernelGGL(kern, dim3((unsigned)ntiles), dim3(512), L_LDS_BYTES, st, a);
+  return 0;
 }
 
 template <int D_DT, int BIAS_DT>
@@ -477,8 +1013,18 @@ template <int D_DT, int BIAS_DT>
 static int launch_linear(const LinearArgs &a, hipStream_t st) {
   LinearKernel k = forced_kernel();
   const bool big_ok = a.K % L_BK == 0 && (((uintptr_t)a.A | (uintptr_t)a.B) & 15) == 0;
-  if (k == LinearKernel::AUTO) k = (big_ok && a.M > 128 && a.N > 128) ? LinearKernel::TILE256 : LinearKernel::TILE128;
+  const bool packed_ok = big_ok && a.K % P_BK == 0 && (a.K >> 1) * 256 < (1ll << 31);
+  if (k == LinearKernel::AUTO) {
+    if (a.M > 128 && a.N > 128 && packed_ok)
+      k = LinearKernel::TILE256P;
+    else if (a.M > 128 && a.N > 128 && big_ok)
+      k = LinearKernel::TILE256;
+    else
+      k = LinearKernel::TILE128;
+  }
+  if (k == LinearKernel::TILE256P && packed_ok) return launch_tile256p<D_DT, BIAS_DT>(a, st);
   if (k == LinearKernel::TILE256 && big_ok) return launch_tile256<D_DT, BIAS_DT>(a, st);
+  if (k == LinearKernel::TILE256W8 && big_ok) return launch_tile256w8<D_DT, BIAS_DT>(a, st);
   const int64_t ntiles = ceil_div(a.M, T_BM) * ceil_div(a.N, T_BN);
   hipLaunchKernelGGL((linear_nvfp4_tile128_kernel<D_DT, BIAS_DT>), dim3((unsigned)ntiles), dim3(256), 0, st, a);
   return 0;
