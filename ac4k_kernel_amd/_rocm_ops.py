@@ -82,6 +82,23 @@ def quantize_nvfp4(out, sf, inp, global_scale, cross_dim: int, reduce_dim: int, 
                                       *geom, int(bool(swizzle)), _stream()))
 
 
+def quantize_nvfp4_with_global_scale(out, sf, global_scale, inp, cross_dim: int, reduce_dim: int, swizzle: bool,
+                                     max_scale: float) -> None:
+    """global_scale (written) = amax(|inp|) / max_scale, then quantize_nvfp4 with it: the nvfp4 branch
+    of the reference's Ac4kQuantizeOp.forward (quant.py:187-242) behind one C call."""
+    lead_shape, geom = _quant_geometry(inp, cross_dim, reduce_dim)
+    R, K = geom[2], geom[3]
+    _check_tensor(global_scale, torch.float32, "global_scale")
+    _check(global_scale.dim() == 0, "global_scale must be a scalar")
+    _check_tensor(out, torch.uint8, "out")
+    _check(list(out.shape) == lead_shape + [R, _align_up(K, 64) // 2],
+           "out must have shape [.., cross, align_up(reduce, 64) / 2]")
+    _check_tensor(sf, torch.float8_e4m3fn, "sf")
+    _check(list(sf.shape) == lead_shape + [_align_up(K, 64) // 64, _align_up(R, 16), 4], "meet invalid sf shape")
+    _lib.check(_L.ac4k_quantize_nvfp4_bf16(out.data_ptr(), sf.data_ptr(), global_scale.data_ptr(), inp.data_ptr(),
+                                           *geom, int(bool(swizzle)), float(max_scale), _stream()))
+
+
 def _quantize_rowwise(fn, out, out_dtype, sf, inp, scale_max, scale_dtype, cross_dim, reduce_dim, *extra):
     lead_shape, geom = _quant_geometry(inp, cross_dim, reduce_dim)
     R, K = geom[2], geom[3]

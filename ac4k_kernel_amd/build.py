@@ -1,7 +1,10 @@
 """Builds libac4k_nvfp4.so (the C-ABI library) for gfx950 with hipcc, in-tree.
 
-    python -m ac4k_kernel_amd.build            # build if sources are newer
-    python -m ac4k_kernel_amd.build --force
+    python ac4k_kernel_amd/build.py            # build if sources are newer
+    python ac4k_kernel_amd/build.py --force
+
+(run it as a script: `python -m ac4k_kernel_amd.build` would import the package, which loads
+the library that is about to be rebuilt)
 """
 from __future__ import annotations
 

@@ -11,6 +11,8 @@
 //
 // All kernels are bandwidth-bound: the row-major paths move 16 bytes per lane per load,
 // reduce amax inside the wavefront with DPP, and store packed words.
+#include <mutex>
+
 #include "ac4k_common.h"
 
 namespace ac4k {
@@ -23,12 +25,24 @@ __global__ void zero_u32_kernel(uint32_t *p) { *p = 0u; }
 
 constexpr int AMAX_THREADS = 256;
 constexpr int AMAX_UNROLL = 4;
+constexpr int AMAX_MAX_BLOCKS = 1024;  // four workgroups per CU
+constexpr int AMAX_SLOTS = 32;        // concurrent (device, stream) pairs served by the one-launch path
 
-__global__ __launch_bounds__(AMAX_THREADS) void amax_scale_bf16_kernel(
-    uint32_t *__restrict__ gs_bits, const uint16_t *__restrict__ x, int64_t n, int64_t head,
-    int64_t nvec, float max_scale) {
-  // x[0..head) and the tail after the vectors are handled by scalar loads of block 0;
-  // the 16-byte aligned middle is streamed with grid-stride uint4 loads.
+// Per-slot scratch of the two-kernel reduction: pass 1 deposits one maximum per block, the
+// consumer (the quantize kernel, or a one-block finalize kernel) reduces the deposits.  A slot
+// belongs to one (device, stream) pair, whose calls the stream serialises, so a slot is never
+// used by two reductions at once.
+struct AmaxScratch {
+  uint32_t partial[AMAX_SLOTS][AMAX_MAX_BLOCKS];
+};
+__device__ AmaxScratch g_amax_scratch;
+
+// |x| maximum of this block's share of x[0..n) as a bf16 bit pattern (valid in thread 0).
+__device__ __forceinline__ uint32_t block_absmax_bf16(const uint16_t *__restrict__ x, int64_t n, int64_t head,
+                                                     int64_t nvec) {
+  // x[0..head) and the tail after the vectors are handled by scalar loads of block 0; the
+  // 16-byte aligned middle is streamed with grid-stride uint4 loads.  Plain (cached) loads: the
+  // quantize pass that follows reads the same data again.
   const uint4 *xv = reinterpret_cast<const uint4 *>(x + head);
   uint32_t m = 0;
   const int64_t stride = (int64_t)gridDim.x * AMAX_THREADS;
@@ -36,7 +50,7 @@ __global__ __launch_bounds__(AMAX_THREADS) void amax_scale_bf16_kernel(
   for (; i + (AMAX_UNROLL - 1) * stride < nvec; i += AMAX_UNROLL * stride) {
     uint4 v[AMAX_UNROLL];
 #pragma unroll
-    for (int u = 0; u < AMAX_UNROLL; ++u) v[u] = ld_stream_u4(xv + i + u * stride);
+    for (int u = 0; u < AMAX_UNROLL; ++u) v[u] = xv[i + u * stride];
 #pragma unroll
     for (int u = 0; u < AMAX_UNROLL; ++u) m = umax32(m, absmax_bf16x8(v[u]));
   }
@@ -53,10 +67,49 @@ __global__ __launch_bounds__(AMAX_THREADS) void amax_scale_bf16_kernel(
   if (threadIdx.x == 0) {
 #pragma unroll
     for (int w = 1; w < AMAX_THREADS / 64; ++w) m = umax32(m, part[w]);
-    // division is monotone, so the max of the per-block quotients is the quotient of the
-    // max; non-negative floats order like unsigned integers.
-    float q = bf16_bits_to_f32(m) / max_scale;
-    if (q > 0.0f || q != q) atomicMax(gs_bits, __float_as_uint(q));
+  }
+  return m;
+}
+
+// Pass 1 of the two-kernel reduction: every block deposits its maximum (no atomics: atomics of
+// many blocks on one address serialise at about 25-50 ns each across the 8 XCDs).
+__global__ __launch_bounds__(AMAX_THREADS) void amax_partials_bf16_kernel(const uint16_t *__restrict__ x, int64_t n,
+                                                                          int64_t head, int64_t nvec, int slot) {
+  const uint32_t m = block_absmax_bf16(x, n, head, nvec);
+  if (threadIdx.x == 0) g_amax_scratch.partial[slot][blockIdx.x] = m;
+}
+
+// max over the deposits of a slot, by every thread of the calling block (all must call it)
+__device__ __forceinline__ uint32_t reduce_amax_partials(int slot, int npart) {
+  uint32_t r = 0;
+  for (int b = threadIdx.x; b < npart; b += blockDim.x) r = umax32(r, g_amax_scratch.partial[slot][b]);
+  r = group_umax<64>(r);
+  __shared__ uint32_t red[16];
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = r;
+  __syncthreads();
+  r = 0;
+  for (int w = 0; w < (int)(blockDim.x >> 6); ++w) r = umax32(r, red[w]);
+  return r;
+}
+
+// Pass 2 when only the scale is wanted: one block.
+__global__ __launch_bounds__(AMAX_THREADS) void amax_finalize_kernel(float *__restrict__ gs, int slot, int npart,
+                                                                     float max_scale) {
+  const uint32_t r = reduce_amax_partials(slot, npart);
+  if (threadIdx.x == 0) *gs = bf16_bits_to_f32(r) / max_scale;
+}
+
+// Fallback when every slot is taken: *gs zeroed by a fill kernel, then an atomic max per block.
+// Division is monotone, so the max of the per-block quotients is the quotient of the max;
+// non-negative floats order like unsigned integers.
+__global__ __launch_bounds__(AMAX_THREADS) void amax_scale_bf16_atomic_kernel(
+    uint32_t *__restrict__ gs_bits, const uint16_t *__restrict__ x, int64_t n, int64_t head, int64_t nvec,
+    float max_scale) {
+  const uint32_t m = block_absmax_bf16(x, n, head, nvec);
+  if (threadIdx.x == 0) {
+    const float q = bf16_bits_to_f32(m) / max_scale;
+    const uint32_t qb = __float_as_uint(q);
+    if ((q > 0.0f || q != q) && qb > *(volatile uint32_t *)gs_bits) atomicMax(gs_bits, qb);
   }
 }
 
@@ -69,12 +122,61 @@ struct QuantGeom {
   int64_t s0, s1, sR, sK;
 };
 
-// One 16-block given 16 floats already in output order.  Returns the e4m3 code.
-__device__ __forceinline__ float nvfp4_block_scale(float amax, float alpha, uint32_t &code) {
+// Where a quantize kernel gets the global scale from: a device scalar (slot < 0), or the
+// deposits of the amax pass, in which case it also publishes the scale through `gs`.
+struct GlobalScaleSrc {
+  float *gs;
+  int slot, npart;
+  float max_scale;
+};
+
+// 1 / global_scale for the calling block (every thread must call it).
+__device__ __forceinline__ float load_alpha(const GlobalScaleSrc &src, bool publisher) {
+  float gs;
+  if (src.slot < 0) {
+    gs = *src.gs;
+  } else {
+    gs = bf16_bits_to_f32(reduce_amax_partials(src.slot, src.npart)) / src.max_scale;
+    if (publisher && threadIdx.x == 0) *src.gs = gs;
+  }
+  return 1.0f / gs;
+}
+
+// Correctly rounded fp32 reciprocals of the 128 non-negative E4M3 codes (entry 0 is 0, entry
+// 0x7F is NaN): the block scale takes one of these values, so the IEEE division of the spec
+// (about a dozen VALU instructions) becomes one LDS read.  The table is folded at compile time
+// (constant folding of `/` is correctly rounded).
+struct RcpE4M3Table {
+  float v[128];
+  constexpr RcpE4M3Table() : v() {
+    for (int c = 0; c < 128; ++c) {
+      const int e = c >> 3, m = c & 7;
+      float val = 0.0f;
+      if (e == 0) {
+        val = (float)m * 0.001953125f;  // m * 2^-9
+      } else {
+        val = 1.0f + (float)m * 0.125f;
+        for (int i = 7; i < e; ++i) val *= 2.0f;
+        for (int i = e; i < 7; ++i) val *= 0.5f;
+      }
+      v[c] = c == 0 ? 0.0f : (c == 127 ? __builtin_nanf("") : 1.0f / val);
+    }
+  }
+};
+__constant__ RcpE4M3Table g_rcp_e4m3;
+
+// Fills the block's LDS copy of the table (every thread must call it; ends with a barrier).
+__device__ __forceinline__ void load_rcp_table(float *lut) {
+  if (threadIdx.x < 128) lut[threadIdx.x] = g_rcp_e4m3.v[threadIdx.x];
+  __syncthreads();
+}
+
+// Scale of one 16-block.  Returns the multiplier alpha * (1 / fp32(sf)) and the e4m3 code.
+// With code 0 the table gives 0 (alpha is finite then: alpha = inf makes every code 0x7E/0x7F).
+__device__ __forceinline__ float nvfp4_block_scale(float amax, float alpha, const float *lut, uint32_t &code) {
   float s32 = alpha * (amax * 0.16666666666666666f);
   code = f32_to_ue4m3_satfinite(s32);
-  float s = e4m3_to_f32(code);
-  return (s != 0.0f) ? alpha * (1.0f / s) : 0.0f;
+  return alpha * lut[code];
 }
 
 __device__ __forceinline__ uint32_t nvfp4_pack8(uint4 v, float o) {
@@ -93,8 +195,11 @@ __device__ __forceinline__ uint32_t nvfp4_pack8(uint4 v, float o) {
 //   ITER = wave passes per workgroup (independent loads in flight per lane)
 template <int CPR, int ITER>
 __global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
-    uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in,
-    const float *__restrict__ global_scale, QuantGeom g) {
+    uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in, GlobalScaleSrc gsrc,
+    QuantGeom g) {
+  __shared__ float lut[128];
+  load_rcp_table(lut);
+  const float alpha = load_alpha(gsrc, blockIdx.x == 0 && blockIdx.y == 0);
   constexpr int LPR = 8 * CPR;   // lanes per row
   constexpr int RW = 64 / LPR;   // rows per wave pass
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -103,7 +208,6 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
   const int64_t k = ((int64_t)(blockIdx.x % ngroups) * LPR + (lane % LPR)) * 8;
   const int64_t row0 = (int64_t)(blockIdx.x / ngroups) * (4 * RW * ITER) + lane / LPR;
   if (k >= g.Kp) return;
-  const float alpha = 1.0f / *global_scale;
   const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + k;
   const bool kvalid = k < g.K;
 
@@ -121,7 +225,7 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
     uint32_t m = absmax_bf16x8(v[it]);
     m = umax32(m, dpp_u32<DPP_QUAD_XOR1>(m));
     uint32_t code;
-    float o = nvfp4_block_scale(bf16_bits_to_f32(m), alpha, code);
+    float o = nvfp4_block_scale(bf16_bits_to_f32(m), alpha, lut, code);
     if (r >= g.R) code = 0;  // pad rows carry zero scales
     uint32_t packed = nvfp4_pack8(v[it], o);
     uint32_t sfw = code | (dpp_u32<DPP_ROW_SHL(2)>(code) << 8) | (dpp_u32<DPP_ROW_SHL(4)>(code) << 16) |
@@ -138,8 +242,11 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
 // contiguous one), and writes 32 packed bytes and one scale dword.
 template <bool SWIZZLE>
 __global__ __launch_bounds__(256) void quantize_nvfp4_generic_kernel(
-    uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in,
-    const float *__restrict__ global_scale, QuantGeom g) {
+    uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in, GlobalScaleSrc gsrc,
+    QuantGeom g) {
+  __shared__ float lut[128];
+  load_rcp_table(lut);
+  const float alpha = load_alpha(gsrc, blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0);
   const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t chunk = blockIdx.y, lead = blockIdx.z;
   if (r >= g.Rp) return;
@@ -148,7 +255,6 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_generic_kernel(
     *sfp = 0u;
     return;
   }
-  const float alpha = 1.0f / *global_scale;
   const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + r * g.sR;
   uint32_t sfw = 0;
   uint32_t *op = reinterpret_cast<uint32_t *>(out + (lead * g.R + r) * (g.Kp / 2) + chunk * 32);
@@ -168,7 +274,7 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_generic_kernel(
       m = umax32(m, h[i] & 0x7fffu);
     }
     uint32_t code;
-    float o = nvfp4_block_scale(bf16_bits_to_f32(m), alpha, code);
+    float o = nvfp4_block_scale(bf16_bits_to_f32(m), alpha, lut, code);
     sfw |= code << (8 * b);
     float f0[8], f1[8];
 #pragma unroll
@@ -331,7 +437,7 @@ static bool rowmajor_ok(const void *in, int64_t K, int64_t s0, int64_t s1, int64
 }
 
 template <int CPR>
-static void launch_nvfp4_rowmajor(uint8_t *out, uint8_t *sf, const uint16_t *in, const float *gs,
+static void launch_nvfp4_rowmajor(uint8_t *out, uint8_t *sf, const uint16_t *in, const GlobalScaleSrc &gs,
                                   const QuantGeom &g, int64_t lead, hipStream_t st) {
   constexpr int ITER = 4;
   constexpr int ROWS = 4 * (8 / CPR) * ITER;
@@ -343,25 +449,108 @@ static void launch_nvfp4_rowmajor(uint8_t *out, uint8_t *sf, const uint16_t *in,
 
 using namespace ac4k;
 
+namespace ac4k {
+
+// (device, stream) -> scratch slot.  Slots are handed out on first use and never recycled;
+// when they run out the caller gets -1 and takes the two-launch path.
+static int amax_slot(hipStream_t st) {
+  static std::mutex mu;
+  static struct { int dev; hipStream_t st; } table[AMAX_SLOTS];
+  static int used = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return -1;
+  std::lock_guard<std::mutex> lock(mu);
+  int per_dev = 0;
+  for (int i = 0; i < used; ++i) {
+    if (table[i].dev == dev && table[i].st == st) return per_dev;
+    if (table[i].dev == dev) ++per_dev;
+  }
+  if (per_dev >= AMAX_SLOTS || used >= AMAX_SLOTS) return -1;
+  table[used].dev = dev;
+  table[used].st = st;
+  ++used;
+  return per_dev;  // index among this device's streams: each device has its own copy of the scratch
+}
+
+// Launches pass 1 (block maxima into the slot's scratch).  Returns the number of deposits, or
+// 0 when no slot is free / the input is empty (the caller then takes the atomic path).
+static int launch_amax_partials(const void *x, int64_t n, hipStream_t st, int *slot_out) {
+  if (n == 0) return 0;
+  const int slot = amax_slot(st);
+  if (slot < 0) return 0;
+  const uintptr_t addr = reinterpret_cast<uintptr_t>(x);
+  int64_t head = ((16 - (addr & 15)) & 15) / 2;
+  if (head > n) head = n;
+  const int64_t nvec = (n - head) / 8;
+  int64_t blocks = ceil_div(nvec, (int64_t)AMAX_THREADS * AMAX_UNROLL);
+  if (blocks < 1) blocks = 1;
+  if (blocks > AMAX_MAX_BLOCKS) blocks = AMAX_MAX_BLOCKS;
+  hipLaunchKernelGGL(amax_partials_bf16_kernel, dim3((unsigned)blocks), dim3(AMAX_THREADS), 0, st,
+                     static_cast<const uint16_t *>(x), n, head, nvec, slot);
+  *slot_out = slot;
+  return (int)blocks;
+}
+
+// Fallback without scratch: *gs zeroed by a fill kernel, then one atomic max per block.
+static void launch_global_scale_atomic(float *gs, const void *x, int64_t n, float max_scale, hipStream_t st) {
+  hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(1), 0, st, reinterpret_cast<uint32_t *>(gs));
+  if (n == 0) return;
+  const uintptr_t addr = reinterpret_cast<uintptr_t>(x);
+  int64_t head = ((16 - (addr & 15)) & 15) / 2;
+  if (head > n) head = n;
+  const int64_t nvec = (n - head) / 8;
+  int64_t blocks = ceil_div(nvec, (int64_t)AMAX_THREADS * AMAX_UNROLL);
+  if (blocks < 1) blocks = 1;
+  if (blocks > 256) blocks = 256;  // every block ends with an atomic on the same address
+  hipLaunchKernelGGL(amax_scale_bf16_atomic_kernel, dim3((unsigned)blocks), dim3(AMAX_THREADS), 0, st,
+                     reinterpret_cast<uint32_t *>(gs), static_cast<const uint16_t *>(x), n, head, nvec, max_scale);
+}
+
+static void launch_global_scale(float *gs, const void *x, int64_t n, float max_scale, hipStream_t st) {
+  int slot = -1;
+  const int npart = launch_amax_partials(x, n, st, &slot);
+  if (npart > 0)
+    hipLaunchKernelGGL(amax_finalize_kernel, dim3(1), dim3(AMAX_THREADS), 0, st, gs, slot, npart, max_scale);
+  else
+    launch_global_scale_atomic(gs, x, n, max_scale, st);
+}
+
+static int launch_quantize_nvfp4(void *out, void *sf, const void *in, const GlobalScaleSrc &gsrc, int64_t d0,
+                                 int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR, int64_t sK,
+                                 int swizzle, hipStream_t st) {
+  QuantGeom g{d1, R, K, align_up(K, 64), align_up(R, 16), s0, s1, sR, sK};
+  uint8_t *o = static_cast<uint8_t *>(out), *s = static_cast<uint8_t *>(sf);
+  const uint16_t *x = static_cast<const uint16_t *>(in);
+  const int64_t lead = d0 * d1;
+  if (!swizzle && rowmajor_ok(in, K, s0, s1, sR, sK) && ceil_div(g.Kp, 64) * ceil_div(g.Rp, 16) < (1ll << 31)) {
+    const int64_t chunks = g.Kp / 64;
+    if (chunks >= 8)
+      launch_nvfp4_rowmajor<8>(o, s, x, gsrc, g, lead, st);
+    else if (chunks >= 3)
+      launch_nvfp4_rowmajor<4>(o, s, x, gsrc, g, lead, st);
+    else if (chunks == 2)
+      launch_nvfp4_rowmajor<2>(o, s, x, gsrc, g, lead, st);
+    else
+      launch_nvfp4_rowmajor<1>(o, s, x, gsrc, g, lead, st);
+  } else {
+    AC4K_REQUIRE(g.Kp / 64 <= 65535, "reduce dim too large for the strided path (%lld)", (long long)K);
+    dim3 grid((unsigned)ceil_div(g.Rp, 256), (unsigned)(g.Kp / 64), (unsigned)lead);
+    if (swizzle)
+      hipLaunchKernelGGL(quantize_nvfp4_generic_kernel<true>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
+    else
+      hipLaunchKernelGGL(quantize_nvfp4_generic_kernel<false>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
+  }
+  return 0;
+}
+
+}  // namespace ac4k
+
 extern "C" __attribute__((visibility("default"))) int ac4k_global_scale_bf16(float *gs, const void *x, int64_t n, float max_scale,
                                       ac4k_stream_t stream) {
   AC4K_REQUIRE(gs && (x || n == 0), "null pointer argument");
   AC4K_REQUIRE(n >= 0, "n must be non-negative");
   AC4K_REQUIRE((reinterpret_cast<uintptr_t>(x) & 1) == 0, "x must be 2-byte aligned");
-  hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(1), 0, st, reinterpret_cast<uint32_t *>(gs));
-  if (n > 0) {
-    const uintptr_t addr = reinterpret_cast<uintptr_t>(x);
-    int64_t head = ((16 - (addr & 15)) & 15) / 2;
-    if (head > n) head = n;
-    const int64_t nvec = (n - head) / 8;
-    int64_t blocks = ceil_div(nvec, (int64_t)AMAX_THREADS * AMAX_UNROLL);
-    if (blocks < 1) blocks = 1;
-    if (blocks > 2048) blocks = 2048;
-    hipLaunchKernelGGL(amax_scale_bf16_kernel, dim3((unsigned)blocks), dim3(AMAX_THREADS), 0, st,
-                       reinterpret_cast<uint32_t *>(gs), static_cast<const uint16_t *>(x), n, head, nvec,
-                       max_scale);
-  }
+  launch_global_scale(gs, x, n, max_scale, (hipStream_t)stream);
   return check_launch("ac4k_global_scale_bf16");
 }
 
@@ -369,30 +558,28 @@ extern "C" __attribute__((visibility("default"))) int ac4k_quantize_nvfp4(void *
                                    int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
                                    int64_t sK, int swizzle, ac4k_stream_t stream) {
   if (int rc = check_geom(out, sf, in, global_scale, d0, d1, R, K, s0, s1, sR, sK)) return rc;
-  QuantGeom g{d1, R, K, align_up(K, 64), align_up(R, 16), s0, s1, sR, sK};
-  hipStream_t st = (hipStream_t)stream;
-  uint8_t *o = static_cast<uint8_t *>(out), *s = static_cast<uint8_t *>(sf);
-  const uint16_t *x = static_cast<const uint16_t *>(in);
-  const int64_t lead = d0 * d1;
-  if (!swizzle && rowmajor_ok(in, K, s0, s1, sR, sK) && ceil_div(g.Kp, 64) * ceil_div(g.Rp, 16) < (1ll << 31)) {
-    const int64_t chunks = g.Kp / 64;
-    if (chunks >= 8)
-      launch_nvfp4_rowmajor<8>(o, s, x, global_scale, g, lead, st);
-    else if (chunks >= 3)
-      launch_nvfp4_rowmajor<4>(o, s, x, global_scale, g, lead, st);
-    else if (chunks == 2)
-      launch_nvfp4_rowmajor<2>(o, s, x, global_scale, g, lead, st);
-    else
-      launch_nvfp4_rowmajor<1>(o, s, x, global_scale, g, lead, st);
-  } else {
-    AC4K_REQUIRE(g.Kp / 64 <= 65535, "reduce dim too large for the strided path (%lld)", (long long)K);
-    dim3 grid((unsigned)ceil_div(g.Rp, 256), (unsigned)(g.Kp / 64), (unsigned)lead);
-    if (swizzle)
-      hipLaunchKernelGGL(quantize_nvfp4_generic_kernel<true>, grid, dim3(256), 0, st, o, s, x, global_scale, g);
-    else
-      hipLaunchKernelGGL(quantize_nvfp4_generic_kernel<false>, grid, dim3(256), 0, st, o, s, x, global_scale, g);
-  }
+  const GlobalScaleSrc gsrc{const_cast<float *>(global_scale), -1, 0, 0.0f};
+  if (int rc = launch_quantize_nvfp4(out, sf, in, gsrc, d0, d1, R, K, s0, s1, sR, sK, swizzle, (hipStream_t)stream))
+    return rc;
   return check_launch("ac4k_quantize_nvfp4");
+}
+
+extern "C" __attribute__((visibility("default"))) int ac4k_quantize_nvfp4_bf16(void *out, void *sf, float *global_scale, const void *in, int64_t d0,
+                                        int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
+                                        int64_t sK, int swizzle, float max_scale, ac4k_stream_t stream) {
+  if (int rc = check_geom(out, sf, in, global_scale, d0, d1, R, K, s0, s1, sR, sK)) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  // pass 1 leaves one maximum per block in the stream's scratch slot; the quantize kernel
+  // reduces them itself and publishes the scale, so the whole op is two launches
+  int slot = -1;
+  const int npart = launch_amax_partials(in, d0 * d1 * R * K, st, &slot);
+  GlobalScaleSrc gsrc{global_scale, slot, npart, max_scale};
+  if (npart == 0) {
+    launch_global_scale_atomic(global_scale, in, d0 * d1 * R * K, max_scale, st);
+    gsrc.slot = -1;
+  }
+  if (int rc = launch_quantize_nvfp4(out, sf, in, gsrc, d0, d1, R, K, s0, s1, sR, sK, swizzle, st)) return rc;
+  return check_launch("ac4k_quantize_nvfp4_bf16");
 }
 
 namespace ac4k {

@@ -22,6 +22,20 @@ def _global_scale(x: torch.Tensor, max_scale: float) -> torch.Tensor:
     return out
 
 
+_SCALE_MAX_CACHE = {}
+
+
+def _scale_max_tensor(value, dtype, device):
+    """0-dim device scalar for scale_max; the reference builds one with torch.full on every call
+    (quant.py:130-135,177-182), here it is kept per (value, dtype, device)."""
+    key = (value, dtype, device)
+    t = _SCALE_MAX_CACHE.get(key)
+    if t is None:
+        t = torch.full([], value, dtype=dtype, device=device)
+        _SCALE_MAX_CACHE[key] = t
+    return t
+
+
 def _lead_shape(shape, cross_dim, reduce_dim):
     return [shape[i] for i in range(len(shape)) if i != cross_dim and i != reduce_dim]
 
@@ -54,23 +68,24 @@ class Ac4kQuantizeOp(torch.nn.Module):
             if max_scale is None:
                 max_scale = 448 if fp8 else 127
             if fp8:
-                smax = torch.full([], max_scale, dtype=torch.float32, device=dev)
+                smax = _scale_max_tensor(float(max_scale), torch.float32, dev)
                 quantize_fp8(output, sf, input, smax, cross_dim, reduce_dim, swizzle)
             else:
-                smax = torch.full([], max_scale, dtype=torch.int32, device=dev)
+                smax = _scale_max_tensor(int(max_scale), torch.int32, dev)
                 quantize_int8(output, sf, input, smax, cross_dim, reduce_dim)
             return output, sf
 
         if max_scale is None:
-            max_scale = torch.finfo(torch.float8_e4m3fn).max * 6.0
-        global_scale = _global_scale(input, float(max_scale))
+            max_scale = 448.0 * 6.0  # FLOAT8_E4M3_MAX * FLOAT4_E2M1_MAX
         # out [.., cross, align_up(reduce, 64) / 2] u8, sf [.., align_up(reduce, 64) / 64, align_up(cross, 16), 4]
         Kp = align_up(K, 64)
         if output is None:
             output = torch.empty(lead + [R, Kp // 2], dtype=torch.uint8, device=dev)
         if sf is None:
             sf = torch.empty(lead + [Kp // 64, align_up(R, 16), 4], dtype=torch.float8_e4m3fn, device=dev)
-        quantize_nvfp4(output, sf, input, global_scale, cross_dim, reduce_dim, swizzle)
+        global_scale = torch.empty((), dtype=torch.float32, device=dev)
+        _rocm_ops.quantize_nvfp4_with_global_scale(output, sf, global_scale, input, cross_dim, reduce_dim, swizzle,
+                                                   float(max_scale))
         return output, sf, global_scale
 
 

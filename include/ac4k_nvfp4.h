@@ -62,6 +62,13 @@ int ac4k_quantize_nvfp4(void *out, void *sf, const void *in, const float *global
                         int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
                         int64_t sK, int swizzle, ac4k_stream_t stream);
 
+/* The nvfp4 branch of Ac4kQuantizeOp.forward in one call
+ * (python/ac4k_kernel/ops/quant.py:187-242): *global_scale = max|in| / max_scale over the whole
+ * (contiguous) input, then ac4k_quantize_nvfp4 with it.  Two launches (block maxima, then a quantize kernel that reduces them), nothing to initialise. */
+int ac4k_quantize_nvfp4_bf16(void *out, void *sf, float *global_scale, const void *in, int64_t d0,
+                             int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
+                             int64_t sK, int swizzle, float max_scale, ac4k_stream_t stream);
+
 /* Replaces ac4k::quantize_fp8 (lib/cuda/sm120/quantize_fp8.cu:192-290).
  * out: e4m3 [d0,d1,R,align_up(K,16)];  sf: fp32 [d0,d1,align_up(R,16)] = amax/scale_max.
  * swizzle != 0: reduce dim permuted as reshape(-1,2,4,2).permute(0,2,1,3). */

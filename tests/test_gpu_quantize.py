@@ -75,6 +75,25 @@ def test_nvfp4_edges():
     check_nvfp4(big.to(torch.bfloat16), 0, 1)
 
 
+def test_nvfp4_all_scale_codes():
+    # global scale 1 (one element is 6 * 448), then a block whose maximum is 6 * e4m3(c) for every
+    # code c: the kernel's reciprocal table is exercised entry by entry, plus in-between maxima
+    codes = torch.arange(1, 127, dtype=torch.uint8)
+    sv = codes.view(torch.float8_e4m3fn).float()
+    g = torch.Generator().manual_seed(5)
+    x = (torch.rand((126 * 4, 16), generator=g) * 2 - 1)
+    mx = torch.cat([sv * 6.0, sv * 6.0 * 1.03, sv * 6.0 * 0.97, sv * 6.0 * 1.06]).clamp(max=2688.0)
+    x = x * mx[:, None]
+    x[:, 3] = mx * torch.where(torch.rand(126 * 4, generator=g) < 0.5, -1.0, 1.0)
+    x = x.reshape(-1, 64).contiguous()
+    x = torch.cat([x, torch.zeros((1, 64))])
+    x[-1, 0] = 2688.0
+    xb = x.to(torch.bfloat16)
+    check_nvfp4(xb, 0, 1)
+    _, sf, gs = T.quantize_nvfp4(xb, 0, 1)
+    assert gs.item() == 1.0 and len(set(sf.flatten().tolist())) >= 126
+
+
 def test_nvfp4_caller_buffers_and_negative_dims():
     x = make_input((40, 192), seed=3).cuda()
     out = torch.full((40, 96), 0xAA, dtype=torch.uint8, device="cuda")
