@@ -25,8 +25,11 @@ SIGNATURES = {
     "ac4k_quantize_fp8": (_int, [_vp, _vp, _vp, _vp] + [_i64] * 8 + [_int, _vp]),
     "ac4k_quantize_int8": (_int, [_vp, _vp, _vp, _vp] + [_i64] * 8 + [_vp]),
     "ac4k_linear_nvfp4": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
+    "ac4k_linear_nvfp4_skinny_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "ac4k_linear_nvfp4_skinny": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64,
+                                        _vp, _i64, _vp]),
     "ac4k_linear_nvfp4_fused_bf16": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int,
-                                            _i64, _i64, _i64, _vp]),
+                                            _i64, _i64, _i64, _vp, _i64, _vp]),
 }
 
 _lib = None

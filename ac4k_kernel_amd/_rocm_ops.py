@@ -133,8 +133,28 @@ def _check_linear_operand(x, x_sf, x_gs, rows, name):
     return K
 
 
+def _skinny_scratch(device, M, N, K):
+    """Workspace tensor for the decode-sized linear, or None when the shape does not take that path."""
+    nbytes = _L.ac4k_linear_nvfp4_skinny_workspace_bytes(M, N, K)
+    if nbytes <= 0:
+        return None
+    return torch.empty((nbytes,), dtype=torch.uint8, device=device)
+
+
+def _bias_args(bias, N):
+    if bias is None:
+        return None, 0
+    _check(bias.dtype in _DTYPE_TAG, "bias must be bfloat16, half or float")
+    _check(bias.is_cuda and bias.is_contiguous(), "bias must be contiguous")
+    _check(bias.dim() == 2, "bias must be a 2d matrix")
+    _check(bias.size(0) == 1, "bias shape[0] must be 1")
+    _check(bias.size(1) == N, f"bias shape[1] must be {N}")
+    return bias.data_ptr(), _DTYPE_TAG[bias.dtype]
+
+
 def linear_nvfp4(D, A, A_sf, A_global_scale, B, B_sf, B_global_scale, bias=None) -> None:
-    """Checks of linear_nvfp4.cu:759-805."""
+    """Checks of linear_nvfp4.cu:759-805.  Decode-sized problems (M <= 32, K % 256 == 0) take the
+    weight-streaming kernel, everything else the tile kernels."""
     _check(isinstance(D, torch.Tensor) and D.dim() == 2, "d must be a 2d matrix")
     _check(D.dtype in _DTYPE_TAG, "d must be bfloat16, half or float")
     _check(D.is_cuda and D.is_contiguous(), "d must be contiguous")
@@ -145,15 +165,16 @@ def linear_nvfp4(D, A, A_sf, A_global_scale, B, B_sf, B_global_scale, bias=None)
     _check(B.dim() == 2 and B.size(1) == A.size(1), "B size(1) must equal A size(1)")
     _check(B.size(0) == N, f"B size(0) must be {N}")
     _check_linear_operand(B, B_sf, B_global_scale, N, "b")
-    bias_ptr, bias_tag = None, 0
-    if bias is not None:
-        _check(bias.dtype in _DTYPE_TAG, "bias must be bfloat16, half or float")
-        _check(bias.is_cuda and bias.is_contiguous(), "bias must be contiguous")
-        _check(bias.dim() == 2, "bias must be a 2d matrix")
-        _check(bias.size(0) == 1, "bias shape[0] must be 1")
-        _check(bias.size(1) == N, f"bias shape[1] must be {N}")
-        bias_ptr, bias_tag = bias.data_ptr(), _DTYPE_TAG[bias.dtype]
+    bias_ptr, bias_tag = _bias_args(bias, N)
     if M == 0 or N == 0:
+        return
+    scratch = _skinny_scratch(D.device, M, N, K) if M <= 32 else None
+    if scratch is not None:
+        ws = scratch
+        _lib.check(_L.ac4k_linear_nvfp4_skinny(D.data_ptr(), _DTYPE_TAG[D.dtype], A.data_ptr(), A_sf.data_ptr(),
+                                               A_global_scale.data_ptr(), B.data_ptr(), B_sf.data_ptr(),
+                                               B_global_scale.data_ptr(), bias_ptr, bias_tag, M, N, K,
+                                               ws.data_ptr(), ws.numel(), _stream()))
         return
     _lib.check(_L.ac4k_linear_nvfp4(D.data_ptr(), _DTYPE_TAG[D.dtype], A.data_ptr(), A_sf.data_ptr(),
                                     A_global_scale.data_ptr(), B.data_ptr(), B_sf.data_ptr(),
@@ -161,14 +182,15 @@ def linear_nvfp4(D, A, A_sf, A_global_scale, B, B_sf, B_global_scale, bias=None)
 
 
 def linear_nvfp4_fused(D, X, X_q, X_sf, X_global_scale, B, B_sf, B_global_scale, bias=None) -> None:
-    """quantize(X, 0, 1) + linear_nvfp4 in one call for 1 <= M <= 32; X_q / X_sf / X_global_scale
-    receive the quantized activation."""
+    """quantize(X, 0, 1) + linear_nvfp4 for a bf16 activation X [M, K], 1 <= M <= 32;
+    X_q / X_sf / X_global_scale receive the quantized activation."""
     _check(isinstance(D, torch.Tensor) and D.dim() == 2, "d must be a 2d matrix")
     _check(D.dtype in _DTYPE_TAG, "d must be bfloat16, half or float")
     _check(D.is_cuda and D.is_contiguous(), "d must be contiguous")
     M, N = D.shape
     _check_tensor(X, torch.bfloat16, "x")
     _check(X.dim() == 2 and X.size(0) == M, f"x must be [{M}, K]")
+    _check(1 <= M <= 32, "the fused linear takes 1 <= M <= 32")
     K = X.size(1)
     _check(K % 64 == 0, "K must be a multiple of 64")
     _check_tensor(X_q, torch.uint8, "x_q")
@@ -176,12 +198,14 @@ def linear_nvfp4_fused(D, X, X_q, X_sf, X_global_scale, B, B_sf, B_global_scale,
     _check_linear_operand(X_q, X_sf, X_global_scale, M, "x")
     _check(B.dim() == 2 and B.size(0) == N and B.size(1) == K // 2, "weight must be [N, K/2]")
     _check_linear_operand(B, B_sf, B_global_scale, N, "b")
-    bias_ptr, bias_tag = None, 0
-    if bias is not None:
-        _check(bias.dtype in _DTYPE_TAG, "bias must be bfloat16, half or float")
-        _check(bias.is_cuda and bias.is_contiguous() and list(bias.shape) == [1, N], f"bias must be [1, {N}]")
-        bias_ptr, bias_tag = bias.data_ptr(), _DTYPE_TAG[bias.dtype]
+    bias_ptr, bias_tag = _bias_args(bias, N)
+    scratch = _skinny_scratch(D.device, M, N, K)
+    if scratch is None:  # K % 256 != 0: the composition itself
+        quantize_nvfp4_with_global_scale(X_q, X_sf, X_global_scale, X, 0, 1, False, 2688.0)
+        linear_nvfp4(D, X_q, X_sf, X_global_scale, B, B_sf, B_global_scale, bias)
+        return
+    ws = scratch
     _lib.check(_L.ac4k_linear_nvfp4_fused_bf16(D.data_ptr(), _DTYPE_TAG[D.dtype], X.data_ptr(), X_q.data_ptr(),
                                                X_sf.data_ptr(), X_global_scale.data_ptr(), B.data_ptr(),
                                                B_sf.data_ptr(), B_global_scale.data_ptr(), bias_ptr, bias_tag,
-                                               M, N, K, _stream()))
+                                               M, N, K, ws.data_ptr(), ws.numel(), _stream()))

@@ -1009,6 +1009,228 @@ static int launch_tile256(const LinearArgs &a, hipStream_t st) {
   return 0;
 }
 
+// ===========================================================================
+// Decode-sized linear (1 <= M <= 32): bound by streaming the weights once.
+//
+// The activation arrives as its exact fp16 dequantization Ahat [M, K] (without the global
+// scale).  A workgroup (4 waves) owns 128 weight rows and one K-slice; every wave one 32-row
+// tile.  Lane (row r, half h) streams 64 contiguous bytes of its weight row per 256-k step
+// (elements [128h, 128h+128) of the step) and decodes them dword by dword into MFMA operands;
+// the activation slice sits in LDS (shared by the four waves).  The MFMA is issued as
+// D^T = W . Ahat^T so a lane ends up with 4 consecutive n for one m.  K-slices of one row
+// group meet through fp32 partial tiles in a caller-provided workspace; a small second kernel
+// adds them in slice order (deterministic), applies gsA*gsB and the bias, converts and stores.
+// (A last-arriver reduction inside the kernel needs device-scope fences, which write back the
+// XCD's L2 and cost far more than the second launch.)
+// Requires K % 256 == 0 and 16-byte aligned weights.
+// ===========================================================================
+struct SkinnyArgs {
+  void *D;
+  const _Float16 *Ahat;
+  const uint8_t *B;
+  const uint32_t *B_sf;
+  const float *A_gs, *B_gs;
+  const void *bias;
+  float *partial;      // [splitK][M][N]
+  int64_t M, N, K, Np;
+  int ks_len, split_k;
+};
+
+constexpr int SK_ROWS = 128;   // weight rows per workgroup
+constexpr int SK_STEP = 256;   // k per step
+
+template <int D_DT, int BIAS_DT>
+__global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char slds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  // K-slice is the fast grid index: workgroups that run together then read neighbouring pieces of the
+  // same rows (all HBM channels), not the same 512-byte column of different rows (a few channels)
+  const int ksl = blockIdx.x;
+  const int64_t ng = blockIdx.y, n0 = ng * SK_ROWS + wave * 32;
+  const int64_t kbeg = (int64_t)ksl * a.ks_len;
+  const int nsteps = a.ks_len / SK_STEP;  // 1..4
+  const int pitch = a.ks_len * 2 + 16;    // LDS row pitch in bytes (16 bytes of padding: no bank conflicts)
+
+  // weight stream of this lane: all steps of the slice are requested up front
+  int64_t wrow = n0 + r;
+  wrow = wrow < a.N ? wrow : a.N - 1;  // rows past N feed outputs that are never stored
+  const uint8_t *wp = a.B + wrow * (a.K >> 1) + (kbeg >> 1) + h * 64;
+  const uint32_t *sp = a.B_sf + ((kbeg >> 6) + 2 * h) * a.Np + wrow;
+  uint4 W[4][4];
+  uint32_t S[4][2];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    if (t < nsteps) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) W[t][q] = *reinterpret_cast<const uint4 *>(wp + t * 128 + q * 16);  // cached: the four words share a line
+      S[t][0] = sp[(int64_t)(t * 4) * a.Np];
+      S[t][1] = sp[(int64_t)(t * 4 + 1) * a.Np];
+    }
+  }
+  // activation slice -> LDS
+  {
+    const int vec_per_row = a.ks_len / 8;  // 16-byte vectors per row
+    const int total = (int)a.M * vec_per_row;
+    for (int i = tid; i < total; i += 256) {
+      const int m = i / vec_per_row, v = i % vec_per_row;
+      *reinterpret_cast<uint4 *>(slds + m * pitch + v * 16) =
+          *reinterpret_cast<const uint4 *>(a.Ahat + (int64_t)m * a.K + kbeg + v * 8);
+    }
+  }
+  __syncthreads();
+
+  f32x16 acc0, acc1;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc0[e] = acc1[e] = 0.0f;
+  const int am = r < (int)a.M ? r : (int)a.M - 1;  // lanes past M read a valid row; their outputs are dropped
+  const char *arow = slds + am * pitch + h * 256;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    if (t < nsteps) {
+      f16x2 sc[2][2];  // [chunk][block pair] -> scales of blocks (0,1) and (2,3) of each 64-chunk
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        sc[c][0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(S[t][c] & 0x7f7f7f7fu, 1.0f, false);
+        sc[c][1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(S[t][c] & 0x7f7f7f7fu, 1.0f, true);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {       // 16-byte word q: elements [32q, 32q+32) of the lane's 128
+        const uint32_t w[4] = {W[t][q].x, W[t][q].y, W[t][q].z, W[t][q].w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {     // dword d: elements [32q + 8d, +8): block (4q + d) / 2 of the lane
+          const int blk = (4 * q + d) >> 1;   // 0..7: chunk blk/4, block blk%4
+          const f16x2 pair = sc[blk >> 2][(blk & 3) >> 1];
+          f16x8 wdec = (blk & 1) ? decode_dword<true>(w[d], pair) : decode_dword<false>(w[d], pair);
+          const f16x8 afrag = *reinterpret_cast<const f16x8 *>(arow + t * 512 + (q * 4 + d) * 16);
+          if ((q * 4 + d) & 1)
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wdec, afrag, acc1, 0, 0, 0);
+          else
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wdec, afrag, acc0, 0, 0, 0);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc0[e] += acc1[e];
+
+  // acc0: lane <-> m = r, element e <-> n = n0 + (e>>2)*8 + h*4 + (e&3): 4 consecutive n per group
+  const int m = r;
+  if (m >= (int)a.M) return;
+  if (a.split_k > 1) {  // fp32 partial tile of this K-slice; skinny_reduce_kernel adds the slices
+    float *pp = a.partial + ((int64_t)ksl * a.M + m) * a.N;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int64_t n = n0 + g * 8 + h * 4;
+      if (n + 3 < a.N && (a.N & 3) == 0) {
+        *reinterpret_cast<float4 *>(pp + n) = make_float4(acc0[4 * g], acc0[4 * g + 1], acc0[4 * g + 2], acc0[4 * g + 3]);
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (n + q < a.N) pp[n + q] = acc0[4 * g + q];
+      }
+    }
+    return;
+  }
+  using DE = Elem<D_DT>;
+  typename DE::T *Dp = static_cast<typename DE::T *>(a.D);
+  const float scale = (*a.A_gs) * (*a.B_gs);
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int64_t n = n0 + (e >> 2) * 8 + h * 4 + (e & 3);
+    if (n < a.N) {
+      float v = acc0[e] * scale;
+      if constexpr (BIAS_DT != BIAS_NONE) v += Elem<BIAS_DT>::load(a.bias, n);
+      Dp[(int64_t)m * a.N + n] = DE::cvt(v);
+    }
+  }
+}
+
+// D[m, n] = cvt( (sum over K-slices of partial[s][m][n]) * gsA*gsB + bias[n] ), slices added in order
+template <int D_DT, int BIAS_DT>
+__global__ __launch_bounds__(256) void skinny_reduce_kernel(SkinnyArgs a) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t total = a.M * a.N;
+  if (i >= total) return;
+  float v = 0.0f;
+  for (int sidx = 0; sidx < a.split_k; ++sidx) v += a.partial[(int64_t)sidx * total + i];
+  v *= (*a.A_gs) * (*a.B_gs);
+  if constexpr (BIAS_DT != BIAS_NONE) v += Elem<BIAS_DT>::load(a.bias, i % a.N);
+  static_cast<typename Elem<D_DT>::T *>(a.D)[i] = Elem<D_DT>::cvt(v);
+}
+
+// packed activation -> exact fp16 dequantization (without the global scale), one dword per thread
+__global__ __launch_bounds__(256) void decode_activation_kernel(_Float16 *__restrict__ ahat,
+                                                                const uint8_t *__restrict__ A,
+                                                                const uint8_t *__restrict__ A_sf, int64_t M, int64_t K,
+                                                                int64_t Mp) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // dword index
+  if (i >= M * (K >> 3)) return;
+  const int64_t m = i / (K >> 3), k = (i % (K >> 3)) * 8;
+  const uint32_t w = *reinterpret_cast<const uint32_t *>(A + m * (K >> 1) + (k >> 1));
+  const uint32_t code = A_sf[(((k >> 6) * Mp + m) << 2) + ((k >> 4) & 3)] & 0x7fu;
+  const f16x2 sc2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(code, 1.0f, false);
+  const f16x8 d = decode_dword<false>(w, sc2);
+  *reinterpret_cast<f16x8 *>(ahat + m * K + k) = d;
+}
+
+struct SkinnyPlan {
+  int ks_len, split_k;
+  int64_t ahat_bytes, partial_bytes, groups;
+  int lds_bytes;
+};
+
+static bool skinny_plan(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
+  if (M < 1 || M > 32 || K % SK_STEP != 0 || N < 1) return false;
+  int ks = 1024;
+  while (ks > SK_STEP && K % ks != 0) ks >>= 1;
+  p.groups = ceil_div(N, SK_ROWS);
+  // short problems: use smaller slices to get enough workgroups in flight
+  while (ks > SK_STEP && p.groups * (K / ks) < 768) ks >>= 1;
+  p.ks_len = ks;
+  p.split_k = (int)(K / ks);
+  p.ahat_bytes = align_up(M * K * 2, 256);
+  p.partial_bytes = p.split_k > 1 ? (int64_t)p.split_k * M * N * 4 : 0;
+  p.lds_bytes = (int)M * (ks * 2 + 16);
+  return true;
+}
+
+template <int D_DT, int BIAS_DT>
+static int launch_skinny(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_t st) {
+  auto *kern = linear_nvfp4_skinny_kernel<D_DT, BIAS_DT>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 32 * (1024 * 2 + 16));
+    if (e != hipSuccess) return set_error("hipFuncSetAttribute: %s", hipGetErrorString(e));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)p.split_k, (unsigned)p.groups), dim3(256), p.lds_bytes, st, a);
+  if (p.split_k > 1)
+    hipLaunchKernelGGL((skinny_reduce_kernel<D_DT, BIAS_DT>), dim3((unsigned)ceil_div(a.M * a.N, 256)), dim3(256), 0, st, a);
+  return 0;
+}
+
+template <int D_DT>
+static int dispatch_skinny_bias(const SkinnyArgs &a, const SkinnyPlan &p, int bias_dtype, hipStream_t st) {
+  if (!a.bias) return launch_skinny<D_DT, BIAS_NONE>(a, p, st);
+  switch (bias_dtype) {
+    case AC4K_DTYPE_BF16: return launch_skinny<D_DT, AC4K_DTYPE_BF16>(a, p, st);
+    case AC4K_DTYPE_FP16: return launch_skinny<D_DT, AC4K_DTYPE_FP16>(a, p, st);
+    case AC4K_DTYPE_FP32: return launch_skinny<D_DT, AC4K_DTYPE_FP32>(a, p, st);
+  }
+  return set_error("bias must be bfloat16, half or float (dtype tag %d)", bias_dtype);
+}
+
+static int dispatch_skinny(const SkinnyArgs &a, const SkinnyPlan &p, int d_dtype, int bias_dtype, hipStream_t st) {
+  switch (d_dtype) {
+    case AC4K_DTYPE_BF16: return dispatch_skinny_bias<AC4K_DTYPE_BF16>(a, p, bias_dtype, st);
+    case AC4K_DTYPE_FP16: return dispatch_skinny_bias<AC4K_DTYPE_FP16>(a, p, bias_dtype, st);
+    case AC4K_DTYPE_FP32: return dispatch_skinny_bias<AC4K_DTYPE_FP32>(a, p, bias_dtype, st);
+  }
+  return set_error("d must be bfloat16, half or float (dtype tag %d)", d_dtype);
+}
+
 template <int D_DT, int BIAS_DT>
 static int launch_linear(const LinearArgs &a, hipStream_t st) {
   LinearKernel k = forced_kernel();
@@ -1081,14 +1303,77 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4(void *D,
   return check_launch("ac4k_linear_nvfp4");
 }
 
+namespace ac4k {
+
+// shared tail of the two decode-sized entry points: Ahat is in the workspace already
+static int run_skinny(void *D, int d_dtype, const float *A_gs, const void *B, const void *B_sf, const float *B_gs,
+                      const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, const SkinnyPlan &p,
+                      void *workspace, hipStream_t st) {
+  SkinnyArgs a{D,
+               static_cast<const _Float16 *>(workspace),
+               static_cast<const uint8_t *>(B),
+               static_cast<const uint32_t *>(B_sf),
+               A_gs,
+               B_gs,
+               bias,
+               reinterpret_cast<float *>(static_cast<char *>(workspace) + p.ahat_bytes),
+               M,
+               N,
+               K,
+               align_up(N, 16),
+               p.ks_len,
+               p.split_k};
+  return dispatch_skinny(a, p, d_dtype, bias_dtype, st);
+}
+
+static int check_skinny(const SkinnyPlan &p, bool ok, const void *B, void *workspace, int64_t workspace_bytes) {
+  AC4K_REQUIRE(ok, "the decode-sized linear takes 1 <= M <= 32 and K %% 256 == 0");
+  AC4K_REQUIRE(((uintptr_t)B & 15) == 0, "weights must be 16-byte aligned");
+  AC4K_REQUIRE(workspace && ((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
+  AC4K_REQUIRE(workspace_bytes >= p.ahat_bytes + p.partial_bytes, "workspace too small: %lld bytes needed",
+               (long long)(p.ahat_bytes + p.partial_bytes));
+  return 0;
+}
+
+}  // namespace ac4k
+
+extern "C" __attribute__((visibility("default"))) int64_t ac4k_linear_nvfp4_skinny_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  SkinnyPlan p;
+  if (!skinny_plan(M, N, K, p)) return 0;
+  return p.ahat_bytes + p.partial_bytes;
+}
+
+extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_skinny(void *D, int d_dtype, const void *A, const void *A_sf, const float *A_gs,
+                                        const void *B, const void *B_sf, const float *B_gs, const void *bias,
+                                        int bias_dtype, int64_t M, int64_t N, int64_t K, void *workspace,
+                                        int64_t workspace_bytes, ac4k_stream_t stream) {
+  AC4K_REQUIRE(D && A && A_sf && A_gs && B && B_sf && B_gs, "null pointer argument");
+  SkinnyPlan p;
+  const bool ok = skinny_plan(M, N, K, p);
+  if (int rc = check_skinny(p, ok, B, workspace, workspace_bytes)) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t dwords = M * (K >> 3);
+  hipLaunchKernelGGL(decode_activation_kernel, dim3((unsigned)ceil_div(dwords, 256)), dim3(256), 0, st,
+                     static_cast<_Float16 *>(workspace), static_cast<const uint8_t *>(A),
+                     static_cast<const uint8_t *>(A_sf), M, K, align_up(M, 16));
+  if (int rc = run_skinny(D, d_dtype, A_gs, B, B_sf, B_gs, bias, bias_dtype, M, N, K, p, workspace, st))
+    return rc;
+  return check_launch("ac4k_linear_nvfp4_skinny");
+}
+
 extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_fused_bf16(void *D, int d_dtype, const void *X, void *X_q, void *X_sf,
                                             float *X_gs, const void *B, const void *B_sf, const float *B_gs,
                                             const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K,
-                                            ac4k_stream_t stream) {
-  AC4K_REQUIRE(X && X_q && X_sf && X_gs, "null pointer argument");
-  AC4K_REQUIRE(K % 64 == 0, "K must be a multiple of 64 (got %lld)", (long long)K);
+                                            void *workspace, int64_t workspace_bytes, ac4k_stream_t stream) {
+  AC4K_REQUIRE(D && X && X_q && X_sf && X_gs && B && B_sf && B_gs, "null pointer argument");
   AC4K_REQUIRE(M >= 1 && M <= 32, "the fused skinny linear takes 1 <= M <= 32 (got %lld)", (long long)M);
-  if (int rc = ac4k_global_scale_bf16(X_gs, X, M * K, 2688.0f, stream)) return rc;
-  if (int rc = ac4k_quantize_nvfp4(X_q, X_sf, X, X_gs, 1, 1, M, K, 0, 0, K, 1, 0, stream)) return rc;
-  return ac4k_linear_nvfp4(D, d_dtype, X_q, X_sf, X_gs, B, B_sf, B_gs, bias, bias_dtype, M, N, K, stream);
+  SkinnyPlan p;
+  const bool ok = skinny_plan(M, N, K, p);
+  if (int rc = check_skinny(p, ok, B, workspace, workspace_bytes)) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  if (int rc = quantize_activation_with_f16(X_q, X_sf, X_gs, X, M, K, 2688.0f, static_cast<_Float16 *>(workspace), st))
+    return rc;
+  if (int rc = run_skinny(D, d_dtype, X_gs, B, B_sf, B_gs, bias, bias_dtype, M, N, K, p, workspace, st))
+    return rc;
+  return check_launch("ac4k_linear_nvfp4_fused_bf16");
 }

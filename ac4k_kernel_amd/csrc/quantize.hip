@@ -193,10 +193,12 @@ __device__ __forceinline__ uint32_t nvfp4_pack8(uint4 v, float o) {
 // chunk's first lane with three DPP row shifts and stored as one dword.
 //   CPR  = 64-element chunks per wave row (8*CPR lanes per row, 8/CPR rows per wave pass)
 //   ITER = wave passes per workgroup (independent loads in flight per lane)
-template <int CPR, int ITER>
+//   EMIT = also write the dequantized block values e2m1 * fp32(sf) as fp16 (exact) to `f16out`
+//          [rows, K] (2-D inputs only): the decode-sized linear consumes them directly
+template <int CPR, int ITER, bool EMIT>
 __global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
     uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in, GlobalScaleSrc gsrc,
-    QuantGeom g) {
+    QuantGeom g, _Float16 *__restrict__ f16out) {
   __shared__ float lut[128];
   load_rcp_table(lut);
   const float alpha = load_alpha(gsrc, blockIdx.x == 0 && blockIdx.y == 0);
@@ -234,6 +236,19 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
       st_stream_u1(out + (lead * g.R + r) * (g.Kp / 2) + k / 2, packed);
     if ((lane & 7) == 0 && r < g.Rp)
       reinterpret_cast<uint32_t *>(sf)[(lead * (g.Kp / 64) + k / 64) * g.Rp + r] = sfw;
+    if constexpr (EMIT) {
+      if (r < g.R) {
+        const f16x2 sc2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(code, 1.0f, false);
+        const f16x2 sc = {sc2.x, sc2.x};
+        f16x2 d0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 0) * sc;
+        f16x2 d1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 1) * sc;
+        f16x2 d2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 2) * sc;
+        f16x2 d3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 3) * sc;
+        *reinterpret_cast<uint4 *>(f16out + r * g.Kp + k) =
+            make_uint4(__builtin_bit_cast(uint32_t, d0), __builtin_bit_cast(uint32_t, d1),
+                       __builtin_bit_cast(uint32_t, d2), __builtin_bit_cast(uint32_t, d3));
+      }
+    }
   }
 }
 
@@ -438,11 +453,16 @@ static bool rowmajor_ok(const void *in, int64_t K, int64_t s0, int64_t s1, int64
 
 template <int CPR>
 static void launch_nvfp4_rowmajor(uint8_t *out, uint8_t *sf, const uint16_t *in, const GlobalScaleSrc &gs,
-                                  const QuantGeom &g, int64_t lead, hipStream_t st) {
+                                  const QuantGeom &g, int64_t lead, hipStream_t st, _Float16 *f16out = nullptr) {
   constexpr int ITER = 4;
   constexpr int ROWS = 4 * (8 / CPR) * ITER;
   dim3 grid((unsigned)(ceil_div(g.Kp / 64, CPR) * ceil_div(g.Rp, ROWS)), (unsigned)lead);
-  hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER>), grid, dim3(256), 0, st, out, sf, in, gs, g);
+  if (f16out)
+    hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER, true>), grid, dim3(256), 0, st, out, sf, in, gs, g,
+                       f16out);
+  else
+    hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER, false>), grid, dim3(256), 0, st, out, sf, in, gs, g,
+                       f16out);
 }
 
 }  // namespace ac4k
@@ -583,6 +603,25 @@ extern "C" __attribute__((visibility("default"))) int ac4k_quantize_nvfp4_bf16(v
 }
 
 namespace ac4k {
+
+// Internal: quantize a contiguous 2-D activation X [M, K] (K % 64 == 0, 16-byte aligned) like
+// ac4k_quantize_nvfp4_bf16 and also emit its exact fp16 dequantization (without the global
+// scale) to f16out [M, K].  Two launches.
+int quantize_activation_with_f16(void *out, void *sf, float *gs, const void *in, int64_t M, int64_t K,
+                                 float max_scale, _Float16 *f16out, hipStream_t st) {
+  AC4K_REQUIRE(K % 64 == 0 && rowmajor_ok(in, K, 0, 0, K, 1), "activation must be 16-byte aligned with K %% 64 == 0");
+  int slot = -1;
+  const int npart = launch_amax_partials(in, M * K, st, &slot);
+  GlobalScaleSrc gsrc{gs, slot, npart, max_scale};
+  if (npart == 0) {
+    launch_global_scale_atomic(gs, in, M * K, max_scale, st);
+    gsrc.slot = -1;
+  }
+  QuantGeom g{1, M, K, K, align_up(M, 16), 0, 0, K, 1};
+  launch_nvfp4_rowmajor<8>(static_cast<uint8_t *>(out), static_cast<uint8_t *>(sf), static_cast<const uint16_t *>(in),
+                           gsrc, g, 1, st, f16out);
+  return 0;
+}
 
 template <RowFmt FMT, int LPR, int NV>
 static void launch_rowwise_rowmajor(uint8_t *out, float *sf, const uint16_t *in, const void *smax,

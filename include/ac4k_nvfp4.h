@@ -91,16 +91,28 @@ int ac4k_linear_nvfp4(void *D, int d_dtype, const void *A, const void *A_sf, con
                       const void *B, const void *B_sf, const float *B_gs, const void *bias,
                       int bias_dtype, int64_t M, int64_t N, int64_t K, ac4k_stream_t stream);
 
-/* Fused skinny linear: quantize(X,0,1) followed by linear(...) in one call, for decode-sized
- * M (1..32).  No single reference function: it equals the composition the reference's tests
- * make (test/test_linear_bench.py:128-137) — the activation bytes, scales and global scale
- * it produces are those of ac4k_global_scale_bf16 + ac4k_quantize_nvfp4.
- * X bf16 [M,K] contiguous, K % 64 == 0.  The quantized activation is also returned:
- * X_q [M,K/2], X_sf [K/64,align_up(M,16),4], X_gs (1 float). */
+/* Decode-sized linear (1 <= M <= 32, K % 256 == 0): same contract as ac4k_linear_nvfp4
+ * (lib/cuda/sm120/linear_nvfp4.cu:753-901; the reference runs these shapes through its one
+ * 128x128 tile kernel), implemented as a weight-streaming split-K kernel.  It needs scratch:
+ * `workspace` = ac4k_linear_nvfp4_skinny_workspace_bytes(M,N,K) bytes of device memory,
+ * 256-byte aligned, contents irrelevant (it receives the fp16 activation and the fp32 partial
+ * sums of the K-slices).  The size function returns 0 for shapes this path does not take. */
+int64_t ac4k_linear_nvfp4_skinny_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int ac4k_linear_nvfp4_skinny(void *D, int d_dtype, const void *A, const void *A_sf, const float *A_gs,
+                             const void *B, const void *B_sf, const float *B_gs, const void *bias,
+                             int bias_dtype, int64_t M, int64_t N, int64_t K, void *workspace,
+                             int64_t workspace_bytes, ac4k_stream_t stream);
+
+/* Fused decode-sized linear: quantize(X,0,1) followed by linear(...) in one call.  No single
+ * reference function: it equals the composition the reference's tests make
+ * (test/test_linear_bench.py:128-137) — the activation bytes, scales and global scale it
+ * produces are those of ac4k_quantize_nvfp4_bf16, and they are returned:
+ * X bf16 [M,K] contiguous -> X_q [M,K/2], X_sf [K/64,align_up(M,16),4], X_gs (1 float).
+ * workspace as for ac4k_linear_nvfp4_skinny. */
 int ac4k_linear_nvfp4_fused_bf16(void *D, int d_dtype, const void *X, void *X_q, void *X_sf,
                                  float *X_gs, const void *B, const void *B_sf, const float *B_gs,
                                  const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K,
-                                 ac4k_stream_t stream);
+                                 void *workspace, int64_t workspace_bytes, ac4k_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -56,7 +56,7 @@ def test_argument_rejection_without_gpu():
     assert rc != 0 and b"multiple of 16" in lib.ac4k_last_error()
     rc = lib.ac4k_linear_nvfp4(one, 7, one, one, one, one, one, one, None, 0, 4, 4, 64, None)
     assert rc != 0 and b"bfloat16, half or float" in lib.ac4k_last_error()
-    rc = lib.ac4k_linear_nvfp4_fused_bf16(one, 0, one, one, one, one, one, one, one, None, 0, 64, 4, 64, None)
+    rc = lib.ac4k_linear_nvfp4_fused_bf16(one, 0, one, one, one, one, one, one, one, None, 0, 64, 4, 64, one, 0, None)
     assert rc != 0 and b"1 <= M <= 32" in lib.ac4k_last_error()
     with pytest.raises(RuntimeError):
         _lib.check(rc)

@@ -124,6 +124,34 @@ def test_fused_skinny_equals_composition(m):
     torch.testing.assert_close(d, comp, atol=ATOL, rtol=RTOL)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 256, 256), (7, 300, 512), (16, 130, 768), (32, 1000, 1024), (32, 64, 4096),
+                                   (5, 33, 2304)])
+def test_decode_sized_shapes(m, n, k):
+    # the weight-streaming split-K path (M <= 32, K % 256 == 0), ragged N, all output / bias dtypes
+    run_case(m, n, k, seed=m + k, wstd=0.02)
+    run_case(m, n, k, bias_dtype=torch.float32, o_dtype=torch.float32, seed=m, wstd=0.02)
+    run_case(m, n, k, bias_dtype=torch.bfloat16, o_dtype=torch.float16, seed=n, wstd=0.02)
+
+
+@pytest.mark.parametrize("m", [1, 8, 32])
+def test_fused_decode_config5(m):
+    n, k = 28672, 8192
+    x = make_input((m, k), seed=m, outliers=True).cuda()
+    wq = gpu_quant(make_input((n, k), seed=51, std=0.02))
+    d1, (xq, xsf, xgs) = ops().fused_linear(x, *wq, return_quantized=True)
+    d2 = ops().fused_linear(x, *wq)                       # second call: the ticket counters reset themselves
+    assert torch.equal(d1, d2)
+    eq, esf, egs = T.quantize_nvfp4(x.cpu(), 0, 1)
+    assert torch.equal(xq.cpu(), eq) and torch.equal(xsf.cpu().view(torch.uint8), esf) and xgs.item() == egs.item()
+    cols = torch.arange(0, n, 97)
+    cw = cpu(wq)
+    fb = T.dequantize_nvfp4(cw[0][cols], cw[1][:, cols].contiguous(), cw[2])
+    ref = (T.dequantize_nvfp4(eq, esf, egs) @ fb.t()).to(torch.bfloat16)
+    torch.testing.assert_close(d1.cpu()[:, cols], ref, atol=ATOL, rtol=RTOL)
+    full = (gpu_dequant((xq, xsf, xgs), m) @ gpu_dequant(wq, n).t()).to(torch.bfloat16)
+    torch.testing.assert_close(d1, full, atol=ATOL, rtol=RTOL)
+
+
 def test_error_behaviour():
     o = ops()
     aq, bq = gpu_quant(make_input((8, 128), seed=1)), gpu_quant(make_input((16, 128), seed=2))
