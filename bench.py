@@ -1,18 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the NVFP4 path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|linear|quantize|traffic]
+                    [--no-cpu-baseline] [--no-check]
 
 Prints ONE JSON line.  The headline `value` is the NVFP4 linear at M=N=K=8192 (the
 north-star GEMM, also the first shape of the reference's test/test_linear_tflops.py:189)
 in TFLOP/s = 2*M*N*K / t, with the operands already quantized and resident in HBM.  The
 same line carries, under "quantize", the BF16->NVFP4 / FP8 / INT8 quantizers on the
-8192x4096 outlier activations (GB/s = (in + out + sf bytes) / t as in
-test/test_quantize_bandwidth.py:32-33, whole quantize() call) and the 4096x4096 case.
+8192x4096 outlier activations and the 4096x4096 case (GB/s = (in + out + sf bytes) / t as
+in test/test_quantize_bandwidth.py:32-33, whole quantize() call, three rotating input
+buffers), under "linear_shapes" the other GEMM configurations and under "decode" the fused
+decode-sized linear.
 
 A "step" is one pass of the timed op over one batch of synthetic input.  Timing uses
 events recorded on the stream the kernels are launched on (torch's current stream, which
-is the stream handed to the C ABI).
+is the stream handed to the C ABI).  `roofline.traffic` is not measured live: it is the HBM
+byte count per launch taken from the rocprofv3 --pmc summaries in profiles/traffic.json
+(made with `--workload traffic`, see profiles/).
 """
 from __future__ import annotations
 
@@ -59,6 +64,20 @@ def time_gpu(fn, steps, warmup):
     return total, total / steps
 
 
+def measured_traffic(key):
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f).get(key)
+    except (OSError, ValueError):
+        return None
+
+
+def roofline(bound, achieved, traffic_key=None):
+    peak, unit = (HBM_PEAK_GBS, "GB/s") if bound == "hbm" else (MFMA_PEAK_TFLOPS, "TFLOP/s")
+    return {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
+            "traffic": measured_traffic(traffic_key) if traffic_key else None}
+
+
 # --------------------------------------------------------------------------- quantize
 def quant_bytes(shape_rk, precision):
     R, K = shape_rk
@@ -69,7 +88,7 @@ def quant_bytes(shape_rk, precision):
     return 2 * R * K + R * Kp + 4 * Rp
 
 
-def bench_quantize(ops, shape, precision, steps, warmup, outliers, check=True, nbuf=3):
+def bench_quantize(ops, shape, precision, steps, warmup, outliers, check=True, nbuf=3, key=None):
     from oracle import nvfp4_oracle as T
     xs_cpu = [make_input(shape, seed=s, outliers=outliers) for s in range(nbuf)]
     xs = [x.cuda() for x in xs_cpu]
@@ -99,9 +118,7 @@ def bench_quantize(ops, shape, precision, steps, warmup, outliers, check=True, n
     gbs = nbytes / (ms * 1e-3) / 1e9
     return {"workload": f"quantize {precision} {shape[0]}x{shape[1]} bf16" + (" outliers" if outliers else ""),
             "ms": ms, "bytes": nbytes, "GB/s": gbs, "bit_exact_vs_oracle": ok,
-            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": gbs / HBM_PEAK_GBS, "traffic": None},
-            "rotating_buffers": nbuf}
+            "roofline": roofline("hbm", gbs, key), "rotating_buffers": nbuf}
 
 
 def cpu_quantize_baseline(shape, outliers):
@@ -128,7 +145,11 @@ def gpu_dequant(q, rows):
     return (v * s.unsqueeze(-1)).reshape(rows, -1)
 
 
-def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True):
+def linear_bytes(m, n, k):
+    return (m + n) * k // 2 + ((m + 15) // 16 * 16 + (n + 15) // 16 * 16) * k // 16 + m * n * 2 + 8
+
+
+def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True, key=None):
     a, b = make_input((m, k), seed=0), make_input((n, k), seed=1, std=wstd)
     aq, bq = ops.quantize(a.cuda(), 0, 1), ops.quantize(b.cuda(), 0, 1)
     out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
@@ -142,10 +163,30 @@ def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True):
         del ref
     total, ms = time_gpu(lambda: ops.linear(*aq, *bq, out=out), steps, warmup)
     tflops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
+    gbs = linear_bytes(m, n, k) / (ms * 1e-3) / 1e9
+    t_flops, t_bytes = 2.0 * m * n * k / (MFMA_PEAK_TFLOPS * 1e12), linear_bytes(m, n, k) / (HBM_PEAK_GBS * 1e9)
+    rl = roofline("mfma", tflops, key) if t_flops >= t_bytes else roofline("hbm", gbs, key)
     return {"workload": f"NVFP4 linear M={m} N={n} K={k}, bf16 out, operands pre-quantized", "ms": ms,
-            "total_ms": total, "TFLOP/s": tflops, "within_1e-2_of_fp32_dequant_matmul": ok,
-            "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": tflops / MFMA_PEAK_TFLOPS, "traffic": None}}
+            "total_ms": total, "TFLOP/s": tflops, "GB/s": gbs, "within_1e-2_of_fp32_dequant_matmul": ok,
+            "roofline": rl}
+
+
+def bench_decode(ops, m, n, k, steps, warmup, check=True):
+    """Fused decode-sized linear: bf16 activation in, on-the-fly NVFP4 quantize + GEMM."""
+    x = make_input((m, k), seed=2, outliers=True).cuda()
+    wq = ops.quantize(make_input((n, k), seed=3, std=0.02).cuda(), 0, 1)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    ops.fused_linear(x, *wq, out=out)
+    ok = None
+    if check:
+        ref = ops.linear(*ops.quantize(x, 0, 1), *wq)
+        ok = bool(torch.all((out.float() - ref.float()).abs() <= 1e-2 + 1e-2 * ref.float().abs()).item())
+    _, ms = time_gpu(lambda: ops.fused_linear(x, *wq, out=out), steps, warmup)
+    nbytes = n * k // 2 + n * k // 16 + 2 * m * k + 2 * m * n
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return {"workload": f"fused decode linear M={m} N={n} K={k} (bf16 activation quantized on the fly)", "ms": ms,
+            "bytes": nbytes, "GB/s": gbs, "equals_quantize_then_linear_within_1e-2": ok,
+            "roofline": roofline("hbm", gbs)}
 
 
 def cpu_linear_baseline(n, k, rows=256):
@@ -161,12 +202,32 @@ def cpu_linear_baseline(n, k, rows=256):
             "sample": f"oracle fp32 dequantize + torch.matmul of M={rows} rows of the N={n} K={k} problem, 1 run"}
 
 
+def run_traffic(ops):
+    """A few launches of each hot kernel after a plain device copy of known size, for
+    `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` (the copy calibrates the counters)."""
+    src = torch.empty((1 << 28,), dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)  # 256 MiB read + 256 MiB written
+    a = make_input((8192, 8192), seed=0).cuda()
+    aq, bq = ops.quantize(a, 0, 1), ops.quantize(make_input((8192, 8192), seed=1).cuda(), 0, 1)
+    out = torch.empty((8192, 8192), dtype=torch.bfloat16, device="cuda")
+    for _ in range(3):
+        ops.linear(*aq, *bq, out=out)
+    x = make_input((8192, 4096), seed=0, outliers=True).cuda()
+    for prec in ("nvfp4", "fp8e4m3", "int8"):
+        for _ in range(3):
+            ops.quantize(x, 0, 1, precision=prec)
+    torch.cuda.synchronize()
+    print(json.dumps({"traffic_run": "done"}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", choices=["all", "linear", "quantize"])
+    ap.add_argument("--workload", default="all", choices=["all", "linear", "quantize", "traffic"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     args = ap.parse_args()
@@ -177,16 +238,19 @@ def main():
     torch.set_num_threads(min(16, os.cpu_count() or 1))
     from ac4k_kernel_amd import ops
 
+    if args.workload == "traffic":
+        return run_traffic(ops)
     check = not args.no_check
-    line = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+    S, W = args.steps, args.warmup
+    line = {"n_gpus": 1, "steps": S, "warmup": W, "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "data": "synthetic (seed 0, generated on CPU, cast to bf16)"}
     quant = None
     if args.workload in ("all", "quantize"):
         quant = {
-            "cfg2_nvfp4": bench_quantize(ops, (8192, 4096), "nvfp4", args.steps, args.warmup, True, check),
-            "cfg2_fp8e4m3": bench_quantize(ops, (8192, 4096), "fp8e4m3", args.steps, args.warmup, True, check),
-            "cfg2_int8": bench_quantize(ops, (8192, 4096), "int8", args.steps, args.warmup, True, check),
-            "cfg1_nvfp4": bench_quantize(ops, (4096, 4096), "nvfp4", args.steps, args.warmup, False, check),
+            "cfg2_nvfp4": bench_quantize(ops, (8192, 4096), "nvfp4", S, W, True, check, key="quantize_nvfp4_8192x4096"),
+            "cfg2_fp8e4m3": bench_quantize(ops, (8192, 4096), "fp8e4m3", S, W, True, check, key="quantize_fp8_8192x4096"),
+            "cfg2_int8": bench_quantize(ops, (8192, 4096), "int8", S, W, True, check, key="quantize_int8_8192x4096"),
+            "cfg1_nvfp4": bench_quantize(ops, (4096, 4096), "nvfp4", S, W, False, check),
         }
         for k_, v in quant.items():
             log(f"[bench] {k_}: {v['ms'] * 1e3:.1f} us  {v['GB/s']:.0f} GB/s  "
@@ -196,7 +260,7 @@ def main():
             log(f"[bench] cpu quantize oracle: {quant['cpu_baseline']['value']:.2f} GB/s on "
                 f"{quant['cpu_baseline']['cores']} threads")
     if args.workload in ("all", "linear"):
-        lin = bench_linear(ops, 8192, 8192, 8192, args.steps, args.warmup, check=check)
+        lin = bench_linear(ops, 8192, 8192, 8192, S, W, check=check, key="linear_8192")
         log(f"[bench] {lin['workload']}: {lin['ms']:.3f} ms  {lin['TFLOP/s']:.1f} TFLOP/s "
             f"({100 * lin['roofline']['frac']:.1f}% of MFMA peak)  ok={lin['within_1e-2_of_fp32_dequant_matmul']}")
         line.update({"metric": "nvfp4_linear_tflops", "value": lin["TFLOP/s"], "unit": "TFLOP/s",
@@ -206,6 +270,21 @@ def main():
         if not args.no_cpu_baseline:
             line["cpu_baseline"] = cpu_linear_baseline(8192, 8192)
             log(f"[bench] cpu linear oracle: {line['cpu_baseline']['value']:.3f} TFLOP/s")
+        if args.workload == "all":
+            shapes = {"cfg3_4096": bench_linear(ops, 4096, 4096, 4096, S, W, check=check)}
+            for (n, k) in ((14336, 4096), (4096, 14336)):
+                for m in (16, 128, 2048, 8192):
+                    shapes[f"cfg4_M{m}_N{n}_K{k}"] = bench_linear(ops, m, n, k, S, W, wstd=0.02, check=check)
+            for k_, v in shapes.items():
+                log(f"[bench] {k_}: {v['ms'] * 1e3:.1f} us  {v['TFLOP/s']:.1f} TFLOP/s  {v['GB/s']:.0f} GB/s  "
+                    f"{100 * v['roofline']['frac']:.1f}% of {v['roofline']['bound']} peak  "
+                    f"ok={v['within_1e-2_of_fp32_dequant_matmul']}")
+            line["linear_shapes"] = shapes
+            dec = {f"cfg5_M{m}": bench_decode(ops, m, 28672, 8192, S, W, check) for m in (1, 8, 32)}
+            for k_, v in dec.items():
+                log(f"[bench] {k_}: {v['ms'] * 1e3:.1f} us  {v['GB/s']:.0f} GB/s "
+                    f"({100 * v['roofline']['frac']:.1f}% of HBM peak)  ok={v['equals_quantize_then_linear_within_1e-2']}")
+            line["decode"] = dec
         if quant is not None:
             line["quantize"] = quant
     else:
