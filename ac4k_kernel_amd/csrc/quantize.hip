@@ -11,6 +11,7 @@
 //
 // All kernels are bandwidth-bound: the row-major paths move 16 bytes per lane per load,
 // reduce amax inside the wavefront with DPP, and store packed words.
+#include <atomic>
 #include <mutex>
 
 #include "ac4k_common.h"
@@ -303,6 +304,192 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_generic_kernel(
   *sfp = sfw;
 }
 
+// ---------------------------------------------------------------------------
+// Single-launch nvfp4 quantize of a contiguous tensor that fits in the register files.
+//
+// The global scale needs the maximum of the whole tensor before the first nibble can be
+// produced, so a two-kernel quantize reads its input twice.  Here every workgroup keeps its share
+// of the input in registers (NV 16-byte vectors per lane, 1024 lanes, one workgroup per CU),
+// publishes its maximum, waits until every workgroup has published, and quantizes from registers:
+// the input crosses the memory bus once.
+//
+// Grid synchronisation: arrive[w] = (epoch << 16) | bf16 maximum, one word per workgroup, written
+// and polled with device-coherent accesses; the host hands out a new epoch per launch, so nothing
+// is ever cleared.  The wait is bounded (timeout in 100 MHz ticks).  A workgroup that times out -
+// its peers were not all resident, e.g. two such kernels sharing the GPU - returns without writing
+// and without setting done[w]; so does every workgroup when the scale is not a positive finite
+// number.  The REPAIR instantiation is launched right behind on the same stream: workgroups whose
+// done[w] carries the epoch leave at once, the others redo their share with the maxima that are
+// all published by then, using the full-range arithmetic of the two-kernel path.
+//
+// Work split: the tensor is cut into groups of GS = min(NV, 8) segments of 1024 vectors (16 KB);
+// group g of workgroup w is group number g * gridDim.x + w, so that at any moment the grid reads
+// one contiguous stretch of memory, while a workgroup still owns whole runs of rows for the scale
+// layout (scales go through LDS and leave as runs along the row dimension).
+constexpr int OP_THREADS = 1024;
+constexpr int OP_MAX_WGS = 256;
+constexpr int OP_MAX_NV = 16;
+struct OnePassSync {
+  uint32_t arrive[AMAX_SLOTS][OP_MAX_WGS];
+  uint32_t done[AMAX_SLOTS][OP_MAX_WGS];
+};
+__device__ __align__(256) OnePassSync g_onepass;
+
+struct OnePassGeom {
+  uint32_t total_chunks;  // 64-element chunks in the tensor
+  uint32_t ncc;           // chunks per row (K / 64)
+  uint32_t R, Rp, lead;   // rows per leading index, padded rows, number of leading indices
+};
+
+// 16-byte load that bypasses the per-XCD L2 (device-coherent), completed before it returns
+__device__ __forceinline__ uint4 ld_coherent_u4(const void *p) {
+  u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+template <int NV, bool REPAIR>
+__global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
+    uint32_t *__restrict__ out, uint32_t *__restrict__ sf, const uint4 *__restrict__ in, float *__restrict__ gs_out,
+    OnePassGeom g, int slot, uint32_t epoch, float max_scale, uint64_t timeout_ticks) {
+  constexpr int GS = NV < 8 ? NV : 8;  // segments per group
+  constexpr int NG = NV / GS;          // groups per workgroup
+  constexpr uint32_t GC = GS * 128;    // chunks per group
+  __shared__ float lut[128];
+  __shared__ uint32_t sfs[128 * NV];
+  __shared__ uint32_t red[OP_THREADS / 64];
+  __shared__ uint32_t gmax_s;
+  const uint32_t w = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (REPAIR && g_onepass.done[slot][w] == epoch) return;
+
+  uint32_t cb[NG], nvalid[NG];  // first chunk and number of chunks of each group
+#pragma unroll
+  for (int q = 0; q < NG; ++q) {
+    const uint64_t first = ((uint64_t)q * nwg + w) * GC;
+    cb[q] = first < g.total_chunks ? (uint32_t)first : g.total_chunks;
+    const uint32_t left = g.total_chunks - cb[q];
+    nvalid[q] = left < GC ? left : GC;
+  }
+  uint4 v[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const uint32_t lv = (j % GS) * OP_THREADS + tid;  // vector inside the group
+    v[j] = make_uint4(0, 0, 0, 0);
+    if ((lv >> 3) < nvalid[j / GS]) v[j] = in[(uint64_t)cb[j / GS] * 8 + lv];
+  }
+  if (tid < 128) lut[tid] = g_rcp_e4m3.v[tid];
+  uint32_t bm[NV];  // 16-block maxima (bf16 bits)
+  {
+    uint32_t m = 0;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      bm[j] = absmax_bf16x8(v[j]);
+      bm[j] = umax32(bm[j], dpp_u32<DPP_QUAD_XOR1>(bm[j]));
+      m = umax32(m, bm[j]);
+    }
+    if (!REPAIR) {
+      m = group_umax<64>(m);
+      if (lane == 0) red[wave] = m;
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    if (!REPAIR) {
+      uint32_t m = group_umax<16>(red[lane & 15]);
+      if (lane == 0)
+        __hip_atomic_store(&g_onepass.arrive[slot][w], (epoch << 16) | m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const uint32_t tag = epoch & 0xffffu, i0 = lane * 4;
+    const uint64_t t_end = wall_clock64() + timeout_ticks;
+    uint32_t mm = 0;
+    bool ok = false;
+    while (REPAIR || wall_clock64() < t_end) {
+      const uint4 a = ld_coherent_u4(&g_onepass.arrive[slot][i0]);
+      const bool ready = (i0 + 0 >= nwg || (a.x >> 16) == tag) && (i0 + 1 >= nwg || (a.y >> 16) == tag) &&
+                         (i0 + 2 >= nwg || (a.z >> 16) == tag) && (i0 + 3 >= nwg || (a.w >> 16) == tag);
+      if (__all(ready)) {
+        mm = umax32(umax32(i0 + 0 < nwg ? a.x & 0xffffu : 0u, i0 + 1 < nwg ? a.y & 0xffffu : 0u),
+                    umax32(i0 + 2 < nwg ? a.z & 0xffffu : 0u, i0 + 3 < nwg ? a.w & 0xffffu : 0u));
+        ok = true;
+        break;
+      }
+      if (REPAIR) break;  // every maximum was published before the first launch ended
+      __builtin_amdgcn_s_sleep(2);
+    }
+    mm = group_umax<64>(mm);
+    if (lane == 0) gmax_s = ok ? mm : 0xffffffffu;
+  }
+  __syncthreads();
+  const uint32_t gm = gmax_s;
+  if (gm == 0xffffffffu) return;
+  const float gs = bf16_bits_to_f32(gm) / max_scale;
+  const float alpha = 1.0f / gs;
+  // With a positive finite alpha no product below is NaN and no block scale reaches 464 (it is at
+  // most 448 * (1 + 3e-7)), so the clamp and the NaN cases of the full code are not needed.
+  if (!REPAIR && !(alpha > 0.0f && alpha < __builtin_inff())) return;
+  if (w == 0 && tid == 0) *gs_out = gs;
+
+  uint8_t *sfb = reinterpret_cast<uint8_t *>(sfs);
+#pragma unroll
+  for (int q = 0; q < NG; ++q) {
+    uint32_t code[GS];
+    float o[GS];
+#pragma unroll
+    for (int jj = 0; jj < GS; ++jj) {
+      const int j = q * GS + jj;
+      if (REPAIR) {
+        o[jj] = nvfp4_block_scale(bf16_bits_to_f32(bm[j]), alpha, lut, code[jj]);
+      } else {
+        const float s32 = alpha * (bf16_bits_to_f32(bm[j]) * 0.16666666666666666f);
+        code[jj] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(s32, 0.0f, 0, false);
+        o[jj] = lut[code[jj]];
+      }
+    }
+#pragma unroll
+    for (int jj = 0; jj < GS; ++jj) {
+      const int j = q * GS + jj;
+      const uint32_t lv = jj * OP_THREADS + tid;
+      uint32_t packed;
+      if (REPAIR) {
+        packed = nvfp4_pack8(v[j], o[jj]);
+      } else {
+        const float oo = alpha * o[jj];
+        const float f[8] = {bf16_lo(v[j].x) * oo, bf16_hi(v[j].x) * oo, bf16_lo(v[j].y) * oo, bf16_hi(v[j].y) * oo,
+                            bf16_lo(v[j].z) * oo, bf16_hi(v[j].z) * oo, bf16_lo(v[j].w) * oo, bf16_hi(v[j].w) * oo};
+        packed = f32x8_to_e2m1x8(f);
+      }
+      if ((lv >> 3) < nvalid[q]) {
+        st_stream_u1(out + (uint64_t)cb[q] * 8 + lv, packed);
+        // scale byte (lv % 8) / 2 of chunk lv / 8; both lanes of a 16-block hold the same code
+        if ((lane & 1) == 0) sfb[q * GC * 4 + (lv >> 1)] = (uint8_t)code[jj];
+      }
+    }
+  }
+  __syncthreads();
+  // scales: LDS holds one dword per chunk in (row, chunk column) order; memory wants, per chunk
+  // column, runs along the rows
+#pragma unroll
+  for (int q = 0; q < NG; ++q) {
+    if (nvalid[q] == 0) continue;
+    const uint32_t row_first = cb[q] / g.ncc, row_last = (cb[q] + nvalid[q] - 1) / g.ncc;
+    const uint32_t span = row_last - row_first + 1;
+    for (uint32_t i = tid; i < span * g.ncc; i += OP_THREADS) {
+      const uint32_t cc = i / span, row = row_first + (i - cc * span);
+      const uint32_t ch = row * g.ncc + cc;
+      if (ch < cb[q] || ch >= cb[q] + nvalid[q]) continue;
+      const uint32_t l = g.lead > 1 ? row / g.R : 0u, r = row - l * g.R;
+      sf[((uint64_t)l * g.ncc + cc) * g.Rp + r] = sfs[q * GC + (ch - cb[q])];
+    }
+  }
+  // zero scales of the pad rows R..Rp-1, shared out evenly
+  if (g.Rp > g.R) {
+    const uint32_t pad = g.Rp - g.R, npad = g.lead * g.ncc * pad, per = (npad + nwg - 1) / nwg;
+    const uint32_t hi = (w + 1) * per < npad ? (w + 1) * per : npad;
+    for (uint32_t i = w * per + tid; i < hi; i += OP_THREADS) sf[(uint64_t)(i / pad) * g.Rp + g.R + i % pad] = 0u;
+  }
+  if (!REPAIR && tid == 0) g_onepass.done[slot][w] = epoch;
+}
+
 // ===========================================================================
 // per-row fp8 / int8
 // ===========================================================================
@@ -472,23 +659,31 @@ using namespace ac4k;
 namespace ac4k {
 
 // (device, stream) -> scratch slot.  Slots are handed out on first use and never recycled;
-// when they run out the caller gets -1 and takes the two-launch path.
-static int amax_slot(hipStream_t st) {
+// when they run out the caller gets -1 and takes the path without scratch.  With `epoch` the
+// call also draws the next launch number of the slot (1, 2, ...: the single-launch quantizer
+// tags its synchronisation words with it).
+static int amax_slot(hipStream_t st, uint32_t *epoch = nullptr) {
   static std::mutex mu;
-  static struct { int dev; hipStream_t st; } table[AMAX_SLOTS];
+  static struct { int dev; hipStream_t st; uint32_t epoch; } table[AMAX_SLOTS];
   static int used = 0;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return -1;
   std::lock_guard<std::mutex> lock(mu);
-  int per_dev = 0;
-  for (int i = 0; i < used; ++i) {
-    if (table[i].dev == dev && table[i].st == st) return per_dev;
-    if (table[i].dev == dev) ++per_dev;
+  int per_dev = 0, hit = -1;
+  for (int i = 0; i < used && hit < 0; ++i) {
+    if (table[i].dev == dev && table[i].st == st)
+      hit = i;
+    else if (table[i].dev == dev)
+      ++per_dev;
   }
-  if (per_dev >= AMAX_SLOTS || used >= AMAX_SLOTS) return -1;
-  table[used].dev = dev;
-  table[used].st = st;
-  ++used;
+  if (hit < 0) {
+    if (used >= AMAX_SLOTS) return -1;
+    hit = used++;
+    table[hit].dev = dev;
+    table[hit].st = st;
+    table[hit].epoch = 0;
+  }
+  if (epoch) *epoch = ++table[hit].epoch;
   return per_dev;  // index among this device's streams: each device has its own copy of the scratch
 }
 
@@ -533,6 +728,65 @@ static void launch_global_scale(float *gs, const void *x, int64_t n, float max_s
     hipLaunchKernelGGL(amax_finalize_kernel, dim3(1), dim3(AMAX_THREADS), 0, st, gs, slot, npart, max_scale);
   else
     launch_global_scale_atomic(gs, x, n, max_scale, st);
+}
+
+// Bound of the single-launch quantizer's grid wait in 100 MHz ticks (200 us); 0 sends every
+// workgroup to the repair launch, a negative value switches the single-launch path off.
+static std::atomic<int64_t> g_sync_timeout_ticks{20000};
+
+static int device_cu_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  int n = cached[dev].load();
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cached[dev].store(n);
+  }
+  return n;
+}
+
+template <int NV>
+static void launch_onepass(uint32_t *out, uint32_t *sf, const uint4 *in, float *gs, const OnePassGeom &g, int nwg,
+                           int slot, uint32_t epoch, float max_scale, uint64_t ticks, hipStream_t st) {
+  hipLaunchKernelGGL((quantize_nvfp4_onepass_kernel<NV, false>), dim3(nwg), dim3(OP_THREADS), 0, st, out, sf, in, gs,
+                     g, slot, epoch, max_scale, ticks);
+  hipLaunchKernelGGL((quantize_nvfp4_onepass_kernel<NV, true>), dim3(nwg), dim3(OP_THREADS), 0, st, out, sf, in, gs,
+                     g, slot, epoch, max_scale, ticks);
+}
+
+// Global scale + nvfp4 quantize of a dense [lead, R, K] tensor in one pass over the input, when
+// the shape allows it.  Returns false (nothing launched) when the caller has to take the
+// two-kernel path.
+static bool try_quantize_nvfp4_onepass(void *out, void *sf, float *gs, const void *in, int64_t d0, int64_t d1,
+                                       int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR, int64_t sK,
+                                       int swizzle, float max_scale, hipStream_t st) {
+  const int64_t ticks = g_sync_timeout_ticks.load();
+  if (ticks < 0 || swizzle || sK != 1 || K % 64 != 0 || sR != K) return false;
+  if ((d1 > 1 && s1 != R * K) || (d0 > 1 && s0 != d1 * R * K)) return false;
+  if (reinterpret_cast<uintptr_t>(in) & 15) return false;
+  const int64_t lead = d0 * d1, chunks = lead * R * (K / 64);
+  int nwg = device_cu_count();
+  if (nwg > OP_MAX_WGS) nwg = OP_MAX_WGS;
+  if (nwg < 8 || chunks > (int64_t)nwg * 128 * OP_MAX_NV) return false;
+  uint32_t epoch = 0;
+  const int slot = amax_slot(st, &epoch);
+  if (slot < 0) return false;
+  const OnePassGeom g{(uint32_t)chunks, (uint32_t)(K / 64), (uint32_t)R, (uint32_t)align_up(R, 16), (uint32_t)lead};
+  const int64_t per_wg = ceil_div(chunks, (int64_t)nwg * 128);  // 16 KB segments per workgroup
+  uint32_t *o = static_cast<uint32_t *>(out), *s = static_cast<uint32_t *>(sf);
+  const uint4 *x = static_cast<const uint4 *>(in);
+  if (per_wg <= 1)
+    launch_onepass<1>(o, s, x, gs, g, nwg, slot, epoch, max_scale, (uint64_t)ticks, st);
+  else if (per_wg <= 2)
+    launch_onepass<2>(o, s, x, gs, g, nwg, slot, epoch, max_scale, (uint64_t)ticks, st);
+  else if (per_wg <= 4)
+    launch_onepass<4>(o, s, x, gs, g, nwg, slot, epoch, max_scale, (uint64_t)ticks, st);
+  else if (per_wg <= 8)
+    launch_onepass<8>(o, s, x, gs, g, nwg, slot, epoch, max_scale, (uint64_t)ticks, st);
+  else
+    launch_onepass<16>(o, s, x, gs, g, nwg, slot, epoch, max_scale, (uint64_t)ticks, st);
+  return true;
 }
 
 static int launch_quantize_nvfp4(void *out, void *sf, const void *in, const GlobalScaleSrc &gsrc, int64_t d0,
@@ -589,6 +843,8 @@ extern "C" __attribute__((visibility("default"))) int ac4k_quantize_nvfp4_bf16(v
                                         int64_t sK, int swizzle, float max_scale, ac4k_stream_t stream) {
   if (int rc = check_geom(out, sf, in, global_scale, d0, d1, R, K, s0, s1, sR, sK)) return rc;
   hipStream_t st = (hipStream_t)stream;
+  if (try_quantize_nvfp4_onepass(out, sf, global_scale, in, d0, d1, R, K, s0, s1, sR, sK, swizzle, max_scale, st))
+    return check_launch("ac4k_quantize_nvfp4_bf16");
   // pass 1 leaves one maximum per block in the stream's scratch slot; the quantize kernel
   // reduces them itself and publishes the scale, so the whole op is two launches
   int slot = -1;
@@ -681,4 +937,8 @@ extern "C" __attribute__((visibility("default"))) int ac4k_quantize_int8(void *o
                                   int64_t sK, ac4k_stream_t stream) {
   return quantize_rowwise<RowFmt::INT8>(out, sf, in, scale_max, d0, d1, R, K, s0, s1, sR, sK, 0,
                                         (hipStream_t)stream, "ac4k_quantize_int8");
+}
+
+extern "C" __attribute__((visibility("default"))) void ac4k_set_quantize_sync_timeout_us(int64_t us) {
+  ac4k::g_sync_timeout_ticks.store(us < 0 ? -1 : us * 100);
 }

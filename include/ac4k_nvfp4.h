@@ -64,10 +64,17 @@ int ac4k_quantize_nvfp4(void *out, void *sf, const void *in, const float *global
 
 /* The nvfp4 branch of Ac4kQuantizeOp.forward in one call
  * (python/ac4k_kernel/ops/quant.py:187-242): *global_scale = max|in| / max_scale over the whole
- * (contiguous) input, then ac4k_quantize_nvfp4 with it.  Two launches (block maxima, then a quantize kernel that reduces them), nothing to initialise. */
+ * (contiguous) input, then ac4k_quantize_nvfp4 with it.  Two launches, nothing to initialise, no host synchronisation. */
 int ac4k_quantize_nvfp4_bf16(void *out, void *sf, float *global_scale, const void *in, int64_t d0,
                              int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
                              int64_t sK, int swizzle, float max_scale, ac4k_stream_t stream);
+
+/* Tuning knob of ac4k_quantize_nvfp4_bf16 (no counterpart in the reference).  Dense tensors of up to
+ * 64 MiB are quantized in one pass over the input by a kernel whose workgroups wait for each other;
+ * the wait is bounded by this many microseconds (default 200), after which the workgroups that gave
+ * up are redone by a second launch that is always enqueued behind the first.  0 sends every workgroup
+ * down that second path (used by the tests); a negative value selects the two-kernel quantizer. */
+void ac4k_set_quantize_sync_timeout_us(int64_t us);
 
 /* Replaces ac4k::quantize_fp8 (lib/cuda/sm120/quantize_fp8.cu:192-290).
  * out: e4m3 [d0,d1,R,align_up(K,16)];  sf: fp32 [d0,d1,align_up(R,16)] = amax/scale_max.

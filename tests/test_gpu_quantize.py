@@ -94,6 +94,55 @@ def test_nvfp4_all_scale_codes():
     assert gs.item() == 1.0 and len(set(sf.flatten().tolist())) >= 126
 
 
+# Dense shapes with the reduce dim a multiple of 64 take the single-launch quantizer; its three ways
+# through (grid wait passes, every workgroup sent to the repair launch, two-kernel path) must agree
+# with the oracle bit for bit.
+ONEPASS_SHAPES = [((64, 128), 0, 1), ((8192, 4096), 0, 1), ((4096, 4096), 0, 1), ((1000, 2048), 0, 1),
+                  ((33, 14336), 0, 1), ((2049, 192), 0, 1), ((3, 37, 256), 1, 2), ((2, 3, 40, 128), 2, 3),
+                  ((5000, 64), 0, 1), ((1, 8192), 0, 1), ((32, 8192), 0, 1), ((6100, 5120), 0, 1)]
+
+
+@pytest.mark.parametrize("timeout_us", [200, 0, -1])
+def test_nvfp4_single_launch_paths(timeout_us):
+    from ac4k_kernel_amd import _lib
+    L = _lib.load()
+    L.ac4k_set_quantize_sync_timeout_us(timeout_us)
+    try:
+        for i, (shape, c, r) in enumerate(ONEPASS_SHAPES):
+            check_nvfp4(make_input(shape, seed=40 + i, outliers=True), c, r)
+        # repeated calls on one stream reuse the synchronisation words with a new launch number
+        x = make_input((512, 1024), seed=3)
+        for _ in range(5):
+            check_nvfp4(x, 0, 1)
+        # scales that are not positive finite numbers go down the repair path
+        check_nvfp4(torch.zeros(128, 256, dtype=torch.bfloat16), 0, 1)
+        z = make_input((128, 256), seed=5)
+        z[5, 7] = float("inf")
+        check_nvfp4(z, 0, 1)
+    finally:
+        L.ac4k_set_quantize_sync_timeout_us(200)
+
+
+def test_nvfp4_single_launch_two_streams():
+    """Two streams quantize at once: whichever way the workgroups get scheduled (waits may time out),
+    both results are exact."""
+    xs = [make_input((4096, 2048), seed=70 + i, outliers=True) for i in range(2)]
+    exp = [T.quantize_nvfp4(x, 0, 1, False) for x in xs]
+    dev = [x.cuda() for x in xs]
+    streams = [torch.cuda.Stream() for _ in xs]
+    torch.cuda.synchronize()
+    res = [[], []]
+    for _ in range(4):
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                res[i].append(ops().quantize(dev[i], 0, 1))
+    torch.cuda.synchronize()
+    for i in range(2):
+        for out, sf, gs in res[i]:
+            assert gs.item() == exp[i][2].item()
+            assert torch.equal(out.cpu(), exp[i][0]) and torch.equal(sf.cpu().view(torch.uint8), exp[i][1])
+
+
 def test_nvfp4_caller_buffers_and_negative_dims():
     x = make_input((40, 192), seed=3).cuda()
     out = torch.full((40, 96), 0xAA, dtype=torch.uint8, device="cuda")
