@@ -28,13 +28,22 @@ def _check(cond: bool, msg: str) -> None:
 
 
 def _check_tensor(t, dtype, name: str) -> None:
+    # one combined test on the hot path; the individual messages are only built on failure
+    if isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dtype and t.is_contiguous():
+        return
     _check(isinstance(t, torch.Tensor), f"{name} must be a tensor")
     _check(t.is_cuda, f"{name} must be a CUDA tensor")
     _check(t.is_contiguous(), f"{name} must be contiguous")
     _check(t.dtype == dtype, f"Inconsistency of Tensor type: {name} must be {dtype}")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """hipStream_t of torch's current stream on the current device."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 

@@ -313,14 +313,17 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_generic_kernel(
 // publishes its maximum, waits until every workgroup has published, and quantizes from registers:
 // the input crosses the memory bus once.
 //
-// Grid synchronisation: arrive[w] = (epoch << 16) | bf16 maximum, one word per workgroup, written
-// and polled with device-coherent accesses; the host hands out a new epoch per launch, so nothing
-// is ever cleared.  The wait is bounded (timeout in 100 MHz ticks).  A workgroup that times out -
-// its peers were not all resident, e.g. two such kernels sharing the GPU - returns without writing
-// and without setting done[w]; so does every workgroup when the scale is not a positive finite
-// number.  The REPAIR instantiation is launched right behind on the same stream: workgroups whose
-// done[w] carries the epoch leave at once, the others redo their share with the maxima that are
-// all published by then, using the full-range arithmetic of the two-kernel path.
+// Grid synchronisation: arrive[w] = (tag << 16) | bf16 maximum, one word per workgroup, written
+// and polled with device-coherent accesses.  The tag is a 16-bit launch number kept in device
+// memory (epoch[slot] + 1, never the 0 of untouched memory) and advanced by the repair launch, so
+// nothing is ever cleared and a call replays correctly from a captured graph.  The wait is bounded
+// (timeout in 100 MHz ticks).  A workgroup that times out - its peers were not all resident, e.g.
+// two such kernels sharing the GPU - returns without writing and without setting done[w]; so does
+// every workgroup when the scale is not a positive finite number.  The REPAIR instantiation is
+// launched right behind on the same stream: workgroups whose done[w] carries the tag leave at once,
+// the others redo their share with the maxima that are all published by then, using the full-range
+// arithmetic of the two-kernel path.  Every launch uses the same number of workgroups on a device,
+// so each launch overwrites every word the next one polls.
 //
 // Work split: the tensor is cut into groups of GS = min(NV, 8) segments of 1024 vectors (16 KB);
 // group g of workgroup w is group number g * gridDim.x + w, so that at any moment the grid reads
@@ -332,8 +335,21 @@ constexpr int OP_MAX_NV = 16;
 struct OnePassSync {
   uint32_t arrive[AMAX_SLOTS][OP_MAX_WGS];
   uint32_t done[AMAX_SLOTS][OP_MAX_WGS];
+  uint32_t epoch[AMAX_SLOTS];
 };
 __device__ __align__(256) OnePassSync g_onepass;
+
+// Build with -DAC4K_ONEPASS_TIMELINE to record, per workgroup, the 100 MHz clock at the phase
+// boundaries of the single-launch quantizer (a profiling aid; not compiled into the library).
+#ifdef AC4K_ONEPASS_TIMELINE
+__device__ uint64_t g_onepass_timeline[OP_MAX_WGS][8];
+#define AC4K_TL(i)                                                         \
+  do {                                                                     \
+    if (!REPAIR && threadIdx.x == 0) g_onepass_timeline[blockIdx.x][i] = wall_clock64(); \
+  } while (0)
+#else
+#define AC4K_TL(i)
+#endif
 
 struct OnePassGeom {
   uint32_t total_chunks;  // 64-element chunks in the tensor
@@ -351,7 +367,7 @@ __device__ __forceinline__ uint4 ld_coherent_u4(const void *p) {
 template <int NV, bool REPAIR>
 __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
     uint32_t *__restrict__ out, uint32_t *__restrict__ sf, const uint4 *__restrict__ in, float *__restrict__ gs_out,
-    OnePassGeom g, int slot, uint32_t epoch, float max_scale, uint64_t timeout_ticks) {
+    OnePassGeom g, int slot, float max_scale, uint64_t timeout_ticks) {
   constexpr int GS = NV < 8 ? NV : 8;  // segments per group
   constexpr int NG = NV / GS;          // groups per workgroup
   constexpr uint32_t GC = GS * 128;    // chunks per group
@@ -360,8 +376,18 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
   __shared__ uint32_t red[OP_THREADS / 64];
   __shared__ uint32_t gmax_s;
   const uint32_t w = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  if (REPAIR && g_onepass.done[slot][w] == epoch) return;
+  // the launch tag: the main launch derives it from the slot's counter, the repair launch reads it
+  // back from workgroup 0's word (published whatever happened next) and advances the counter
+  uint32_t tag;
+  if (REPAIR) {
+    tag = g_onepass.arrive[slot][0] >> 16;
+    if (w == 0 && tid == 0) g_onepass.epoch[slot] = tag;
+    if (g_onepass.done[slot][w] == (tag | 0x80000000u)) return;
+  } else {
+    tag = (g_onepass.epoch[slot] + 1) & 0xffffu;
+  }
 
+  AC4K_TL(0);
   uint32_t cb[NG], nvalid[NG];  // first chunk and number of chunks of each group
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
@@ -393,13 +419,14 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
     }
   }
   __syncthreads();
+  AC4K_TL(1);
   if (wave == 0) {
     if (!REPAIR) {
       uint32_t m = group_umax<16>(red[lane & 15]);
       if (lane == 0)
-        __hip_atomic_store(&g_onepass.arrive[slot][w], (epoch << 16) | m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&g_onepass.arrive[slot][w], (tag << 16) | m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    const uint32_t tag = epoch & 0xffffu, i0 = lane * 4;
+    const uint32_t i0 = lane * 4;
     const uint64_t t_end = wall_clock64() + timeout_ticks;
     uint32_t mm = 0;
     bool ok = false;
@@ -421,6 +448,7 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
   }
   __syncthreads();
   const uint32_t gm = gmax_s;
+  AC4K_TL(2);
   if (gm == 0xffffffffu) return;
   const float gs = bf16_bits_to_f32(gm) / max_scale;
   const float alpha = 1.0f / gs;
@@ -466,6 +494,7 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
     }
   }
   __syncthreads();
+  AC4K_TL(3);
   // scales: LDS holds one dword per chunk in (row, chunk column) order; memory wants, per chunk
   // column, runs along the rows
 #pragma unroll
@@ -487,7 +516,8 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
     const uint32_t hi = (w + 1) * per < npad ? (w + 1) * per : npad;
     for (uint32_t i = w * per + tid; i < hi; i += OP_THREADS) sf[(uint64_t)(i / pad) * g.Rp + g.R + i % pad] = 0u;
   }
-  if (!REPAIR && tid == 0) g_onepass.done[slot][w] = epoch;
+  AC4K_TL(4);
+  if (!REPAIR && tid == 0) g_onepass.done[slot][w] = tag | 0x80000000u;
 }
 
 // ===========================================================================
@@ -659,31 +689,24 @@ using namespace ac4k;
 namespace ac4k {
 
 // (device, stream) -> scratch slot.  Slots are handed out on first use and never recycled;
-// when they run out the caller gets -1 and takes the path without scratch.  With `epoch` the
-// call also draws the next launch number of the slot (1, 2, ...: the single-launch quantizer
-// tags its synchronisation words with it).
-static int amax_slot(hipStream_t st, uint32_t *epoch = nullptr) {
+// when they run out the caller gets -1 and takes the path without scratch.  A call captured into
+// a graph keeps the slot of the stream it was captured on.
+static int amax_slot(hipStream_t st) {
   static std::mutex mu;
-  static struct { int dev; hipStream_t st; uint32_t epoch; } table[AMAX_SLOTS];
+  static struct { int dev; hipStream_t st; } table[AMAX_SLOTS];
   static int used = 0;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return -1;
   std::lock_guard<std::mutex> lock(mu);
-  int per_dev = 0, hit = -1;
-  for (int i = 0; i < used && hit < 0; ++i) {
-    if (table[i].dev == dev && table[i].st == st)
-      hit = i;
-    else if (table[i].dev == dev)
-      ++per_dev;
+  int per_dev = 0;
+  for (int i = 0; i < used; ++i) {
+    if (table[i].dev == dev && table[i].st == st) return per_dev;
+    if (table[i].dev == dev) ++per_dev;
   }
-  if (hit < 0) {
-    if (used >= AMAX_SLOTS) return -1;
-    hit = used++;
-    table[hit].dev = dev;
-    table[hit].st = st;
-    table[hit].epoch = 0;
-  }
-  if (epoch) *epoch = ++table[hit].epoch;
+  if (used >= AMAX_SLOTS) return -1;
+  table[used].dev = dev;
+  table[used].st = st;
+  ++used;
   return per_dev;  // index among this device's streams: each device has its own copy of the scratch
 }
 
@@ -748,11 +771,11 @@ static int device_cu_count() {
 
 template <int NV>
 static void launch_onepass(uint32_t *out, uint32_t *sf, const uint4 *in, float *gs, const OnePassGeom &g, int nwg,
-                           int slot, uint32_t epoch, float max_scale, uint64_t ticks, hipStream_t st) {
+                           int slot, float max_scale, uint64_t ticks, hipStream_t st) {
   hipLaunchKernelGGL((quantize_nvfp4_onepass_kernel<NV, false>), dim3(nwg), dim3(OP_THREADS), 0, st, out, sf, in, gs,
-                     g, slot, epoch, max_scale, ticks);
+                     g, slot, max_scale, ticks);
   hipLaunchKernelGGL((quantize_nvfp4_onepass_kernel<NV, true>), dim3(nwg), dim3(OP_THREADS), 0, st, out, sf, in, gs,
-                     g, slot, epoch, max_scale, ticks);
+                     g, slot, max_scale, ticks);
 }
 
 // Global scale + nvfp4 quantize of a dense [lead, R, K] tensor in one pass over the input, when
@@ -769,23 +792,22 @@ static bool try_quantize_nvfp4_onepass(void *out, void *sf, float *gs, const voi
   int nwg = device_cu_count();
   if (nwg > OP_MAX_WGS) nwg = OP_MAX_WGS;
   if (nwg < 8 || chunks > (int64_t)nwg * 128 * OP_MAX_NV) return false;
-  uint32_t epoch = 0;
-  const int slot = amax_slot(st, &epoch);
+  const int slot = amax_slot(st);
   if (slot < 0) return false;
   const OnePassGeom g{(uint32_t)chunks, (uint32_t)(K / 64), (uint32_t)R, (uint32_t)align_up(R, 16), (uint32_t)lead};
   const int64_t per_wg = ceil_div(chunks, (int64_t)nwg * 128);  // 16 KB segments per workgroup
   uint32_t *o = static_cast<uint32_t *>(out), *s = static_cast<uint32_t *>(sf);
   const uint4 *x = static_cast<const uint4 *>(in);
   if (per_wg <= 1)
-    launch_onepass<1>(o, s, x, gs, g, nwg, slot, epoch, max_scale, (uint64_t)ticks, st);
+    launch_onepass<1>(o, s, x, gs, g, nwg, slot, max_scale, (uint64_t)ticks, st);
   else if (per_wg <= 2)
-    launch_onepass<2>(o, s, x, gs, g, nwg, slot, epoch, max_scale, (uint64_t)ticks, st);
+    launch_onepass<2>(o, s, x, gs, g, nwg, slot, max_scale, (uint64_t)ticks, st);
   else if (per_wg <= 4)
-    launch_onepass<4>(o, s, x, gs, g, nwg, slot, epoch, max_scale, (uint64_t)ticks, st);
+    launch_onepass<4>(o, s, x, gs, g, nwg, slot, max_scale, (uint64_t)ticks, st);
   else if (per_wg <= 8)
-    launch_onepass<8>(o, s, x, gs, g, nwg, slot, epoch, max_scale, (uint64_t)ticks, st);
+    launch_onepass<8>(o, s, x, gs, g, nwg, slot, max_scale, (uint64_t)ticks, st);
   else
-    launch_onepass<16>(o, s, x, gs, g, nwg, slot, epoch, max_scale, (uint64_t)ticks, st);
+    launch_onepass<16>(o, s, x, gs, g, nwg, slot, max_scale, (uint64_t)ticks, st);
   return true;
 }
 

@@ -29,7 +29,11 @@ def linear(x, x_scale, x_global_scale, weight, weight_scale, weight_global_scale
     [K/64, align_up(rows,16), 4] layout, *_global_scale 0-dim fp32.  bias is [N] or [1, N] in
     bf16/fp16/fp32; out defaults to a new bf16 [M, N] and may be bf16, fp16 or fp32.
     """
-    return Ac4kLinearOp()(x, x_scale, x_global_scale, weight, weight_scale, weight_global_scale, bias, out=out)
+    return _LINEAR_OP.forward(x, x_scale, x_global_scale, weight, weight_scale, weight_global_scale, bias, out=out)
+
+
+# one stateless module instance serves every call of the functional form
+_LINEAR_OP = Ac4kLinearOp()
 
 
 def fused_linear(x, weight, weight_scale, weight_global_scale, bias=None, out=None, return_quantized=False):

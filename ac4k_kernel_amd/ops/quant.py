@@ -103,5 +103,9 @@ def quantize(input, cross_dim, reduce_dim, max_scale=None, precision="nvfp4", sw
       int8    output [.., cross, align_up(reduce,16)] int8, sf [.., align_up(cross,16)] fp32
     where `..` are the remaining input dims in their original order.
     """
-    return Ac4kQuantizeOp()(input, cross_dim, reduce_dim, max_scale=max_scale, precision=precision,
-                            swizzle=swizzle, output=output, sf=sf)
+    return _QUANTIZE_OP.forward(input, cross_dim, reduce_dim, max_scale=max_scale, precision=precision,
+                                swizzle=swizzle, output=output, sf=sf)
+
+
+# one stateless module instance serves every call of the functional form
+_QUANTIZE_OP = Ac4kQuantizeOp()

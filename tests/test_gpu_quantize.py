@@ -143,6 +143,30 @@ def test_nvfp4_single_launch_two_streams():
             assert torch.equal(out.cpu(), exp[i][0]) and torch.equal(sf.cpu().view(torch.uint8), exp[i][1])
 
 
+def test_nvfp4_graph_replay():
+    """A captured quantize call replays correctly: nothing in it depends on host-side state that
+    changes from launch to launch, and eager calls in between do not disturb it."""
+    shape = (2048, 1024)
+    static = make_input(shape, seed=1).cuda()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops().quantize(static, 0, 1)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out, sf, gs = ops().quantize(static, 0, 1)
+    for seed in (11, 12, 13, 14):
+        x = make_input(shape, seed=seed, outliers=True)
+        static.copy_(x.cuda())
+        graph.replay()
+        torch.cuda.synchronize()
+        eo, es, eg = T.quantize_nvfp4(x, 0, 1, False)
+        assert gs.item() == eg.item()
+        assert torch.equal(out.cpu(), eo) and torch.equal(sf.cpu().view(torch.uint8), es)
+        check_nvfp4(make_input((300, 640), seed=seed), 0, 1)  # eager work between the replays
+
+
 def test_nvfp4_caller_buffers_and_negative_dims():
     x = make_input((40, 192), seed=3).cuda()
     out = torch.full((40, 96), 0xAA, dtype=torch.uint8, device="cuda")
