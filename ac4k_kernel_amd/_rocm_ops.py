@@ -162,8 +162,9 @@ def _bias_args(bias, N):
 
 
 def linear_nvfp4(D, A, A_sf, A_global_scale, B, B_sf, B_global_scale, bias=None) -> None:
-    """Checks of linear_nvfp4.cu:759-805.  Decode-sized problems (M <= 32, K % 256 == 0) take the
-    weight-streaming kernel, everything else the tile kernels."""
+    """Checks of linear_nvfp4.cu:759-805.  Shapes for which the library asks for scratch (decode-sized
+    M <= 32, or few output tiles with a long K) get a workspace tensor and the split-K kernels,
+    everything else the tile kernels."""
     _check(isinstance(D, torch.Tensor) and D.dim() == 2, "d must be a 2d matrix")
     _check(D.dtype in _DTYPE_TAG, "d must be bfloat16, half or float")
     _check(D.is_cuda and D.is_contiguous(), "d must be contiguous")
@@ -177,7 +178,7 @@ def linear_nvfp4(D, A, A_sf, A_global_scale, B, B_sf, B_global_scale, bias=None)
     bias_ptr, bias_tag = _bias_args(bias, N)
     if M == 0 or N == 0:
         return
-    scratch = _skinny_scratch(D.device, M, N, K) if M <= 32 else None
+    scratch = _skinny_scratch(D.device, M, N, K)
     if scratch is not None:
         ws = scratch
         _lib.check(_L.ac4k_linear_nvfp4_skinny(D.data_ptr(), _DTYPE_TAG[D.dtype], A.data_ptr(), A_sf.data_ptr(),

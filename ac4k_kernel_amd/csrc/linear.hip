@@ -603,28 +603,37 @@ __global__ __launch_bounds__(512) void linear_nvfp4_tile256w8_kernel(LinearArgs 
 }
 
 // ===========================================================================
-// 256x256 tile, packed operands in LDS, decode after the fragment load.
+// BM x 256 tile (BM = 256 or 128), packed operands in LDS, decode after the fragment load.
 //
 // The packed A/B slices and their scale dwords go from global memory straight into LDS with
 // LDS-DMA loads (global_load_lds: no VGPR staging, no LDS store instruction), three stages of
-// 128 k each.  A wave (4 waves, 2x2, 128x128 each) reads for every 32-row fragment ONE 16-byte
-// word per lane per 64-chunk: lane (row r, half h) owns elements [32h, 32h+32) of the chunk;
-// dword s of that word feeds MFMA sub-step s.  The same k-slot assignment is used for A and
-// B, so the permutation of k inside a chunk cancels in the dot product.  Decode per dword:
+// 128 k each.  A wave (4 waves, 2x2, (BM/2)x128 each) reads for every 32-row fragment ONE
+// 16-byte word per lane per 64-chunk: lane (row r, half h) owns elements [32h, 32h+32) of the
+// chunk; dword s of that word feeds MFMA sub-step s.  The same k-slot assignment is used for A
+// and B, so the permutation of k inside a chunk cancels in the dot product.  Decode per dword:
 // 4 x v_cvt_scalef32_pk_f16_fp4 + 4 x v_pk_mul_f16 by the block scale (E4M3 -> fp16 with
-// v_cvt_scalef32_pk_f16_fp8, splat through op_sel), i.e. 4 VALU per MFMA, which issue in the
-// shadow of the previous MFMA.  There is one workgroup barrier per 128 k, placed in the
-// middle of the step so that the next stage is readable before the current one ends.
+// v_cvt_scalef32_pk_f16_fp8, splat through op_sel); the decode of a sub-step is interleaved with
+// the MFMAs of the previous one.  A single wave issues roughly one VALU instruction per six
+// cycles, so the 4.6 VALU per MFMA of the 256-row tile stretch a 32-cycle MFMA slot to about 41
+// cycles; that, not LDS or HBM, bounds the loop.  There is one workgroup barrier per 128 k,
+// placed in the middle of the step so that the next stage is readable before the current one ends.
+// Split-K: blockIdx.y selects a contiguous range of stages; with more than one range the
+// accumulators go to an fp32 partial buffer and a second kernel adds the ranges.
 // Requires K % 128 == 0 and 16-byte aligned operands.
 // ===========================================================================
-constexpr int P_BK = 128;                       // k per stage (two 64-chunks)
+constexpr int P_BK = 128;     // k per stage (two 64-chunks)
 constexpr int P_STAGES = 3;
-constexpr int P_ROW = 64;                       // packed bytes per row per stage: [chunk][half] x 16 B
-constexpr int P_OFF_B = 256 * P_ROW;            // B rows follow the 256 A rows
-constexpr int P_OFF_SFA = 2 * 256 * P_ROW;      // scale dwords: [chunk][256 rows]
-constexpr int P_OFF_SFB = P_OFF_SFA + 2 * 1024;
-constexpr int P_STAGE_BYTES = P_OFF_SFB + 2 * 1024;  // 36864
-constexpr int P_LDS_BYTES = P_STAGES * P_STAGE_BYTES;
+constexpr int P_ROW = 64;     // packed bytes per row per stage: [chunk][half] x 16 B
+constexpr int P_BN = 256;
+
+template <int BM>
+struct PLayout {               // byte offsets inside one LDS stage
+  static constexpr int OFF_B = BM * P_ROW;                 // B rows follow the A rows
+  static constexpr int OFF_SFA = OFF_B + P_BN * P_ROW;     // scale dwords: [chunk][BM rows]
+  static constexpr int OFF_SFB = OFF_SFA + 2 * BM * 4;     // [chunk][256 rows]
+  static constexpr int STAGE_BYTES = OFF_SFB + 2 * P_BN * 4;
+  static constexpr int LDS_BYTES = P_STAGES * STAGE_BYTES;
+};
 
 // LDS-DMA: global_load_lds with a scalar 64-bit base, a 32-bit lane offset and the LDS
 // destination of lane 0 in M0 (lane l lands at M0 + size * l).  Issued through inline asm so
@@ -640,8 +649,9 @@ __device__ __forceinline__ void dma4(const void *sbase, uint32_t voff, uint32_t 
                :: "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }
 
+template <int MI>
 struct DecFrags {
-  f16x8 a[4], b[4];
+  f16x8 a[MI], b[4];
 };
 
 // dword `w` (8 nibbles) times block scale `sc` (both halves of `sc2` hold candidates, HI picks)
@@ -660,11 +670,39 @@ __device__ __forceinline__ uint32_t dword_of(const uint4 &v) {
   return S == 0 ? v.x : S == 1 ? v.y : S == 2 ? v.z : v.w;
 }
 
-template <int D_DT, int BIAS_DT>
-__global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArgs a) {
-  extern __shared__ __attribute__((aligned(16))) char plds[];
+// Build with -DAC4K_LINEAR_TIMELINE to record per workgroup the 100 MHz clock at kernel entry,
+// loop entry, loop exit and kernel exit plus the shader cycles spent in the loop (a profiling
+// aid; not compiled into the library).
+#ifdef AC4K_LINEAR_TIMELINE
+__device__ uint64_t g_linear_timeline[8192][6];
+#define AC4K_LTL(i, v)                                                     \
+  do {                                                                     \
+    if (threadIdx.x == 0 && blockIdx.x < 8192) g_linear_timeline[blockIdx.x][i] = (v); \
+  } while (0)
+#else
+#define AC4K_LTL(i, v)
+#endif
 
-  const int64_t tiles_m = ceil_div(a.M, L_BM), tiles_n = ceil_div(a.N, L_BN);
+struct SplitK {
+  float *partial;  // [splits][M][N] fp32, or null: convert and store to D
+  int splits;
+};
+
+// MI = 32-row fragments per wave along M: 4 (BM = 256) or 2 (BM = 128).
+template <int D_DT, int BIAS_DT, int MI>
+__global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArgs a, SplitK sk) {
+  extern __shared__ __attribute__((aligned(16))) char plds[];
+  AC4K_LTL(0, wall_clock64());
+  constexpr int BM = 64 * MI;              // two waves along M
+  using PL = PLayout<BM>;
+  constexpr int NDA = BM / 4 / 16;         // 16-row A transfers per wave per stage
+  constexpr int NDB = P_BN / 4 / 16;       // 16-row B transfers per wave per stage
+  constexpr int NSA = 2 * (BM / 64);       // scale transfers of A per stage: chunks x 64-row blocks
+  constexpr int NS = (NSA + 8) / 4;        // scale transfers per wave
+  constexpr int NPIECES = NDA + NDB + NS;
+  static_assert((NSA + 8) % 4 == 0, "scale transfers must split evenly over the waves");
+
+  const int64_t tiles_m = ceil_div(a.M, BM), tiles_n = ceil_div(a.N, P_BN);
   const int64_t ntiles = tiles_m * tiles_n;
   int64_t pid = blockIdx.x;
   {  // contiguous run of tiles per XCD (workgroups are dealt round-robin to the 8 XCDs)
@@ -682,21 +720,28 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int half = lane >> 5;
-  const int nkt = (int)(a.K / P_BK);
+  // this workgroup's range of 128-k stages
+  const int nkt_all = (int)(a.K / P_BK);
+  const int kt0 = (int)((int64_t)nkt_all * blockIdx.y / sk.splits);
+  const int nkt = (int)((int64_t)nkt_all * (blockIdx.y + 1) / sk.splits) - kt0;
 
   // LDS-DMA.  One transfer moves 16 rows x 64 B: lane l reads piece l%4 of row l/4, so four
   // adjacent lanes cover one 64-byte sector, and lands at LDS base + 16*l, i.e. row-major 64-byte
-  // rows.  Per operand a wave moves its 64 rows in 4 transfers; the 32-bit lane offset is loop
-  // invariant and the 64-bit part is a scalar base that advances by 64 bytes per stage.
+  // rows.  The 32-bit lane offset is loop invariant and the 64-bit part is a scalar base that
+  // advances by 64 bytes per stage.
   const int swave = __builtin_amdgcn_readfirstlane(wave);
   const int64_t kb = a.K >> 1;
-  uint32_t offA[4], offB[4];
+  uint32_t offA[NDA], offB[NDB];
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    int64_t ra = (swave * 4 + q) * 16 + (lane >> 2), rb = ra;
-    ra = tm * L_BM + ra < a.M ? ra : a.M - 1 - tm * L_BM;  // rows past the matrix read the last valid row
-    rb = tn * L_BN + rb < a.N ? rb : a.N - 1 - tn * L_BN;
+  for (int q = 0; q < NDA; ++q) {
+    int64_t ra = (swave * NDA + q) * 16 + (lane >> 2);
+    ra = tm * BM + ra < a.M ? ra : a.M - 1 - tm * BM;  // rows past the matrix read the last valid row
     offA[q] = (uint32_t)(ra * kb + (lane & 3) * 16);
+  }
+#pragma unroll
+  for (int q = 0; q < NDB; ++q) {
+    int64_t rb = (swave * NDB + q) * 16 + (lane >> 2);
+    rb = tn * P_BN + rb < a.N ? rb : a.N - 1 - tn * P_BN;
     offB[q] = (uint32_t)(rb * kb + (lane & 3) * 16);
   }
   auto uniform_ptr = [](const void *p) {  // pin a wave-uniform pointer to scalar registers
@@ -704,94 +749,127 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
     return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
   };
-  const uint8_t *baseA = uniform_ptr(a.A + tm * L_BM * kb), *baseB = uniform_ptr(a.B + tn * L_BN * kb);
-  int64_t sra = tm * L_BM + swave * 64 + lane, srb = tn * L_BN + swave * 64 + lane;
-  sra = sra < a.Mp ? sra : a.Mp - 1;
-  srb = srb < a.Np ? srb : a.Np - 1;
-  const uint32_t offSA = (uint32_t)sra * 4u, offSB = (uint32_t)srb * 4u;  // byte offsets inside a scale plane
+  const uint8_t *baseA = uniform_ptr(a.A + tm * BM * kb + (int64_t)kt0 * P_ROW);
+  const uint8_t *baseB = uniform_ptr(a.B + tn * P_BN * kb + (int64_t)kt0 * P_ROW);
+  // scale transfers: piece g = swave * NS + p.  g < NSA: operand A, chunk g / (BM/64), 64-row block
+  // g % (BM/64); otherwise operand B, chunk (g-NSA) / 4, block (g-NSA) % 4.  Source base, bytes
+  // per stage and LDS offset are wave-uniform and fixed, computed here so that the loop body
+  // stays free of branches.
   const uint8_t *sfA8 = uniform_ptr(a.A_sf), *sfB8 = uniform_ptr(a.B_sf);
+  uint32_t offS[NS], ldsS[NS];
+  const uint8_t *baseS[NS];
+  int64_t strideS[NS];
+#pragma unroll
+  for (int p2 = 0; p2 < NS; ++p2) {
+    const int gq = swave * NS + p2;
+    const bool isB = gq >= NSA;
+    const int gl = isB ? gq - NSA : gq, nb = isB ? 4 : BM / 64;
+    const int c = gl / nb, rb = gl % nb;
+    const int64_t rows = isB ? a.Np : a.Mp;
+    int64_t sr = (isB ? tn * P_BN : tm * BM) + rb * 64 + lane;
+    sr = sr < rows ? sr : rows - 1;
+    offS[p2] = (uint32_t)sr * 4u;  // byte offset inside a scale plane
+    strideS[p2] = 2 * rows * 4;    // two planes (chunks) per stage
+    baseS[p2] = uniform_ptr((isB ? sfB8 : sfA8) + c * rows * 4 + kt0 * strideS[p2]);
+    ldsS[p2] = (uint32_t)__builtin_amdgcn_readfirstlane((isB ? PL::OFF_SFB + c * P_BN * 4 : PL::OFF_SFA + c * BM * 4) + rb * 256);
+  }
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)plds;
   // `kt` may run past the last stage: the source is clamped (re-reading the last slice) and the
   // destination is a stage buffer nobody reads again, which keeps the main loop free of branches
   auto issue_piece = [&](int kt_dst, int q) {
-    const uint32_t st = lds_base + (kt_dst % P_STAGES) * P_STAGE_BYTES;
+    const uint32_t st = lds_base + (kt_dst % P_STAGES) * PL::STAGE_BYTES;
     const int kt = kt_dst < nkt ? kt_dst : nkt - 1;
-    if (q < 8) {
-      const int r = q >> 1;
-      if (q & 1)
-        dma16(baseB + (int64_t)kt * P_ROW, offB[r], st + P_OFF_B + (swave * 4 + r) * 1024);
-      else
-        dma16(baseA + (int64_t)kt * P_ROW, offA[r], st + (swave * 4 + r) * 1024);
+    if (q < NDA) {
+      dma16(baseA + (int64_t)kt * P_ROW, offA[q], st + (swave * NDA + q) * 1024);
+    } else if (q < NDA + NDB) {
+      const int r = q - NDA;
+      dma16(baseB + (int64_t)kt * P_ROW, offB[r], st + PL::OFF_B + (swave * NDB + r) * 1024);
     } else {
-      const int c = (q - 8) >> 1;
-      if (q & 1)
-        dma4(sfB8 + ((int64_t)kt * 2 + c) * a.Np * 4, offSB, st + P_OFF_SFB + c * 1024 + swave * 256);
-      else
-        dma4(sfA8 + ((int64_t)kt * 2 + c) * a.Mp * 4, offSA, st + P_OFF_SFA + c * 1024 + swave * 256);
+      const int p2 = q - NDA - NDB;
+      dma4(baseS[p2] + kt * strideS[p2], offS[p2], st + ldsS[p2]);
     }
   };
   auto issue_stage = [&](int kt) {
 #pragma unroll
-    for (int q = 0; q < 12; ++q) issue_piece(kt, q);
+    for (int q = 0; q < NPIECES; ++q) issue_piece(kt, q);
+  };
+  // pieces of stage kt+2 issued in quarter `qr` (0..3) of the second half of a step
+  auto issue_quarter = [&](int kt_dst, int qr) {
+#pragma unroll
+    for (int q = 0; q < NDA; ++q)
+      if (q * 4 / NDA == qr) issue_piece(kt_dst, q);
+#pragma unroll
+    for (int q = 0; q < NDB; ++q)
+      if (q * 4 / NDB == qr) issue_piece(kt_dst, NDA + q);
+#pragma unroll
+    for (int q = 0; q < NS; ++q)
+      if (q * 4 / NS == qr) issue_piece(kt_dst, NDA + NDB + q);
   };
 
-  f32x16 acc[4][4];
+  f32x16 acc[MI][4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   // fragment addresses inside a stage (bytes)
-  const int fa_off = (wm * 128 + (lane & 31)) * P_ROW + half * 16;
-  const int fb_off = P_OFF_B + (wn * 128 + (lane & 31)) * P_ROW + half * 16;
-  const int sa_off = P_OFF_SFA + (wm * 128 + (lane & 31)) * 4;
-  const int sb_off = P_OFF_SFB + (wn * 128 + (lane & 31)) * 4;
+  const int fa_off = (wm * (32 * MI) + (lane & 31)) * P_ROW + half * 16;
+  const int fb_off = PL::OFF_B + (wn * 128 + (lane & 31)) * P_ROW + half * 16;
+  const int sa_off = PL::OFF_SFA + (wm * (32 * MI) + (lane & 31)) * 4;
+  const int sb_off = PL::OFF_SFB + (wn * 128 + (lane & 31)) * 4;
   const int sh = half * 16;
 
-  uint4 PA[2][4], PB[2][4];  // packed fragments of a 64-chunk, double buffered by chunk parity
-  f16x2 SA[2][4], SB[2][4];  // their two block scales (blocks 2*half, 2*half+1) as fp16
+  uint4 PA[2][MI], PB[2][4];  // packed fragments of a 64-chunk, double buffered by chunk parity
+  f16x2 SA[2][MI], SB[2][4];  // their two block scales (blocks 2*half, 2*half+1) as fp16
   auto load_chunk = [&](int kt, int c) {
-    const char *st = plds + (kt % P_STAGES) * P_STAGE_BYTES;
-#ifdef EXP_NO_LDSREAD
-    if (kt > 0) return;
-#endif
+    const char *st = plds + (kt % P_STAGES) * PL::STAGE_BYTES;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      PA[c][i] = *reinterpret_cast<const uint4 *>(st + fa_off + c * 32 + i * 32 * P_ROW);
+      if (i < MI) PA[c][i] = *reinterpret_cast<const uint4 *>(st + fa_off + c * 32 + i * 32 * P_ROW);
       PB[c][i] = *reinterpret_cast<const uint4 *>(st + fb_off + c * 32 + i * 32 * P_ROW);
-      uint32_t wa = *reinterpret_cast<const uint32_t *>(st + sa_off + c * 1024 + i * 128);
-      uint32_t wb = *reinterpret_cast<const uint32_t *>(st + sb_off + c * 1024 + i * 128);
-      SA[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((wa >> sh) & 0x7f7fu, 1.0f, false);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (i < MI) {
+        uint32_t wa = *reinterpret_cast<const uint32_t *>(st + sa_off + c * (BM * 4) + i * 128);
+        SA[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((wa >> sh) & 0x7f7fu, 1.0f, false);
+      }
+      uint32_t wb = *reinterpret_cast<const uint32_t *>(st + sb_off + c * (P_BN * 4) + i * 128);
       SB[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((wb >> sh) & 0x7f7fu, 1.0f, false);
     }
   };
 
-  DecFrags D[2];
-  auto decode = [&](DecFrags &d, int c, auto S) {
+  DecFrags<MI> D[2];
+  auto decode = [&](DecFrags<MI> &d, int c, auto S) {
     constexpr int s = decltype(S)::value;
-#ifdef EXP_NO_DEC
-    if (c >= 0) return;
-#endif
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      d.a[i] = decode_dword<(s >= 2)>(dword_of<s>(PA[c][i]), SA[c][i]);
+      if (i < MI) d.a[i] = decode_dword<(s >= 2)>(dword_of<s>(PA[c][i]), SA[c][i]);
       d.b[i] = decode_dword<(s >= 2)>(dword_of<s>(PB[c][i]), SB[c][i]);
     }
   };
-  auto mfma16 = [&](const DecFrags &d) {
+  auto mfma16 = [&](const DecFrags<MI> &d) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(d.b[j], d.a[i], acc[i][j], 0, 0, 0);  // D^T block
   };
-  auto interleave = [&]() {  // 16 x (1 MFMA, 4 VALU): the decode rides in the MFMA shadow
+  auto interleave = [&]() {  // the decode of the next sub-step rides in the shadow of the MFMAs
+    if constexpr (MI == 4) {
 #pragma unroll
-    for (int g = 0; g < 16; ++g) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      for (int g = 0; g < 16; ++g) {  // 16 x (1 MFMA, 4 VALU)
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      }
+    } else {
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {  // 8 x (1 MFMA, 6 VALU)
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -803,19 +881,21 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   // prologue: stages 0 and 1 in flight, stage 0 visible, chunk 0 fragments and first decode
   issue_stage(0);
   if (nkt > 1) issue_stage(1);
-  if (nkt > 1) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (nkt > 1) {
+    static_assert(NPIECES == 12 || NPIECES == 9, "wait count below is spelled out per variant");
+    if constexpr (NPIECES == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
   __syncthreads();
   load_chunk(0, 0);
   decode(D[0], 0, I0{});
 
-#ifdef EXP_TIMING
-  long long tA = 0, tB = 0, tC = 0, tprev = __builtin_readcyclecounter(), tstart = tprev;
-  const long long rt0 = wall_clock64();
-#define TPOINT(acc_) { long long tn_ = __builtin_readcyclecounter(); acc_ += tn_ - tprev; tprev = tn_; }
-#else
-#define TPOINT(acc_)
+#ifdef AC4K_LINEAR_TIMELINE
+  const uint64_t tl_c0 = __builtin_readcyclecounter();
 #endif
+  AC4K_LTL(1, wall_clock64());
   for (int kt = 0; kt < nkt; ++kt) {
     // chunk 0: sub-steps 0..3 (fragments of chunk 1 are fetched meanwhile)
     load_chunk(kt, 1);
@@ -832,51 +912,73 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     mfma16(D[1]);
     interleave();
     // stage kt+1 must be complete (own DMA done, then everybody's); stage kt-1 is free after this
-    TPOINT(tA)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    TPOINT(tB)
     // chunk 1: sub-steps 4..7 (chunk 0 of the next stage is fetched meanwhile); the DMA of stage
     // kt+2 is spread over these sub-steps
     decode(D[1], 1, I1{});
-#ifndef EXP_NO_DMA
-    issue_piece(kt + 2, 0); issue_piece(kt + 2, 1); issue_piece(kt + 2, 8);
-#endif
+    issue_quarter(kt + 2, 0);
     mfma16(D[0]);
     interleave();
     load_chunk(kt + 1, 0);  // past the end this reads a stale stage; the result is never used
     decode(D[0], 1, I2{});
-#ifndef EXP_NO_DMA
-    issue_piece(kt + 2, 2); issue_piece(kt + 2, 3); issue_piece(kt + 2, 9);
-#endif
+    issue_quarter(kt + 2, 1);
     mfma16(D[1]);
     interleave();
     decode(D[1], 1, I3{});
-#ifndef EXP_NO_DMA
-    issue_piece(kt + 2, 4); issue_piece(kt + 2, 5); issue_piece(kt + 2, 10);
-#endif
+    issue_quarter(kt + 2, 2);
     mfma16(D[0]);
     interleave();
     decode(D[0], 0, I0{});  // first sub-step of the next stage (unused after the last step)
-#ifndef EXP_NO_DMA
-    issue_piece(kt + 2, 6); issue_piece(kt + 2, 7); issue_piece(kt + 2, 11);
-#endif
+    issue_quarter(kt + 2, 3);
     mfma16(D[1]);
     interleave();
-    TPOINT(tC)
   }
-#ifdef EXP_TIMING
-  long long tloop = __builtin_readcyclecounter() - tstart;
+  AC4K_LTL(2, wall_clock64());
+#ifdef AC4K_LINEAR_TIMELINE
+  AC4K_LTL(4, __builtin_readcyclecounter() - tl_c0);
+  {
+    uint32_t xcc, hwid;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+    AC4K_LTL(5, (xcc & 0xf) | (hwid << 8));
+  }
 #endif
 
   // ---- epilogue.  The MFMAs were issued with the operands swapped, so acc[i][j] holds the
   // TRANSPOSED 32x32 block: lane l, element e <-> n = j*32 + (e>>2)*8 + (l>>5)*4 + (e&3),
-  // m = i*32 + (l&31): four consecutive n per lane.  2-byte outputs are staged through LDS (free
-  // now) so that every lane stores 16 bytes and a wave store covers whole 256-byte row segments.
+  // m = i*32 + (l&31): four consecutive n per lane.
+  const int64_t m0 = tm * BM + wm * (32 * MI), n0 = tn * P_BN + wn * 128;
+  if (sk.partial) {  // split-K: raw fp32 sums of this K range; the reduce kernel scales and converts
+    float *pp = sk.partial + (int64_t)blockIdx.y * a.M * a.N;
+    const bool v4 = (a.N & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      const int64_t m = m0 + i * 32 + (lane & 31);
+      if (m >= a.M) continue;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int64_t n = n0 + j * 32 + g * 8 + half * 4;
+          if (v4 && n + 3 < a.N) {
+            *reinterpret_cast<float4 *>(pp + m * a.N + n) =
+                make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+          } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              if (n + q < a.N) pp[m * a.N + n + q] = acc[i][j][4 * g + q];
+          }
+        }
+    }
+    AC4K_LTL(3, wall_clock64());
+    return;
+  }
+  // 2-byte outputs are staged through LDS (free now) so that every lane stores 16 bytes and a
+  // wave store covers whole 256-byte row segments.
   const float scale = (*a.A_gs) * (*a.B_gs);
   using DE = Elem<D_DT>;
   typename DE::T *Dp = static_cast<typename DE::T *>(a.D);
-  const int64_t m0 = tm * L_BM + wm * 128, n0 = tn * L_BN + wn * 128;
   float bias4[4][4][4];  // [j][g][e&3]
   if constexpr (BIAS_DT != BIAS_NONE) {
 #pragma unroll
@@ -897,10 +999,11 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   const bool vec_ok = sizeof(typename DE::T) == 2 && (a.N % 8 == 0) && ((uintptr_t)a.D % 16 == 0);
   if (vec_ok) {
     constexpr int PITCH = 272;  // bytes per staged row: 128 outputs + 16 bytes of padding
+    static_assert(4 * 64 * PITCH <= PL::LDS_BYTES, "epilogue staging must fit in LDS");
     __syncthreads();            // every wave is done reading the operand stages
     char *stg = plds + wave * (64 * PITCH);
 #pragma unroll
-    for (int p = 0; p < 2; ++p) {
+    for (int p = 0; p < MI / 2; ++p) {
 #pragma unroll
       for (int ii = 0; ii < 2; ++ii) {
         const int i = 2 * p + ii;
@@ -928,7 +1031,7 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < MI; ++i) {
       const int64_t m = m0 + i * 32 + (lane & 31);
 #pragma unroll
       for (int j = 0; j < 4; ++j)
@@ -939,28 +1042,30 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
         }
     }
   }
-#ifdef EXP_TIMING
-  if (blockIdx.x == 0 && tid == 0) {
-    long long tend = __builtin_readcyclecounter();
-    Dp[0] = DE::cvt((float)tA); Dp[1] = DE::cvt((float)tB); Dp[2] = DE::cvt((float)tC);
-    Dp[3] = DE::cvt((float)tloop); Dp[4] = DE::cvt((float)(tend - tstart)); Dp[5] = DE::cvt((float)(wall_clock64() - rt0));
-  }
-#endif
+  AC4K_LTL(3, wall_clock64());
 }
 
-template <int D_DT, int BIAS_DT>
-static int launch_tile256p(const LinearArgs &a, hipStream_t st) {
-  auto *kern = linear_nvfp4_tile256p_kernel<D_DT, BIAS_DT>;
+template <int D_DT, int BIAS_DT, int MI>
+static int launch_tile256p_mi(const LinearArgs &a, const SplitK &sk, hipStream_t st) {
+  auto *kern = linear_nvfp4_tile256p_kernel<D_DT, BIAS_DT, MI>;
+  using PL = PLayout<64 * MI>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, P_LDS_BYTES);
-    if (e != hipSuccess) return set_error("hipFuncSetAttribute(LDS=%d): %s", P_LDS_BYTES, hipGetErrorString(e));
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, PL::LDS_BYTES);
+    if (e != hipSuccess) return set_error("hipFuncSetAttribute(LDS=%d): %s", PL::LDS_BYTES, hipGetErrorString(e));
     attr_set = true;
   }
-  const int64_t ntiles = ceil_div(a.M, L_BM) * ceil_div(a.N, L_BN);
-  hipLaunchKernelGGL(kern, dim3((unsigned)ntiles), dim3(256), P_LDS_BYTES, st, a);
+  const int64_t ntiles = ceil_div(a.M, 64 * MI) * ceil_div(a.N, P_BN);
+  hipLaunchKernelGGL(kern, dim3((unsigned)ntiles, (unsigned)sk.splits), dim3(256), PL::LDS_BYTES, st, a, sk);
   return 0;
+}
+
+// the packed-LDS kernel with the tile height that suits M; no split-K (one K range, output to D)
+template <int D_DT, int BIAS_DT>
+static int launch_tile256p(const LinearArgs &a, hipStream_t st) {
+  const SplitK one{nullptr, 1};
+  return a.M <= 128 ? launch_tile256p_mi<D_DT, BIAS_DT, 2>(a, one, st) : launch_tile256p_mi<D_DT, BIAS_DT, 4>(a, one, st);
 }
 
 constexpr int L_LDS_BYTES = 2 * 2 * L_TILE_HALVES * (int)sizeof(_Float16);  // 128 KiB
@@ -1231,13 +1336,18 @@ static int dispatch_skinny(const SkinnyArgs &a, const SkinnyPlan &p, int d_dtype
   return set_error("d must be bfloat16, half or float (dtype tag %d)", d_dtype);
 }
 
+// shapes the packed-LDS kernel takes: whole 128-k stages, 16-byte aligned rows, 32-bit lane offsets
+static bool packed_kernel_ok(const LinearArgs &a) {
+  return a.K % P_BK == 0 && (((uintptr_t)a.A | (uintptr_t)a.B) & 15) == 0 && (a.K >> 1) * 256 < (1ll << 31);
+}
+
 template <int D_DT, int BIAS_DT>
 static int launch_linear(const LinearArgs &a, hipStream_t st) {
   LinearKernel k = forced_kernel();
   const bool big_ok = a.K % L_BK == 0 && (((uintptr_t)a.A | (uintptr_t)a.B) & 15) == 0;
-  const bool packed_ok = big_ok && a.K % P_BK == 0 && (a.K >> 1) * 256 < (1ll << 31);
+  const bool packed_ok = packed_kernel_ok(a);
   if (k == LinearKernel::AUTO) {
-    if (a.M > 128 && a.N > 128 && packed_ok)
+    if (a.M > 32 && a.N >= 128 && packed_ok)
       k = LinearKernel::TILE256P;
     else if (a.M > 128 && a.N > 128 && big_ok)
       k = LinearKernel::TILE256;
@@ -1305,6 +1415,72 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4(void *D,
 
 namespace ac4k {
 
+// Split-K for problems with too few output tiles to fill the GPU (32 < M, few tiles, long K):
+// the packed-LDS kernel runs `splits` K ranges per tile into fp32 partial buffers in the
+// workspace and skinny_reduce_kernel adds them.
+struct MidPlan {
+  int splits;
+  int64_t partial_bytes;
+};
+
+static bool mid_plan(int64_t M, int64_t N, int64_t K, MidPlan &p) {
+  if (M <= 32 || N < 128 || K % P_BK != 0 || (K >> 1) * 256 >= (1ll << 31)) return false;
+  const bool small = M <= 128;
+  const int64_t tiles = ceil_div(M, small ? 128 : 256) * ceil_div(N, P_BN);
+  const int64_t stages = K / P_BK;
+  if (tiles >= 192) return false;
+  // Rough cost in microseconds of running `s` K ranges per tile on 256 CUs: rounds of
+  // workgroups x stages per range x time per stage, fixed prologue/epilogue, and for s > 1 the
+  // partial sums written and read back at about 3 TB/s plus the second launch.
+  const double stage_us = small ? 1.45 : 2.9;
+  double best = 0.0;
+  int64_t best_s = 1;
+  for (int64_t s = 1; s <= 32 && s * 2 <= stages; ++s) {
+    const double rounds = (double)ceil_div(tiles * s, 256);
+    double t = rounds * (double)ceil_div(stages, s) * stage_us + 6.0;
+    if (s > 1) t += (double)s * (double)(M * N) * 8.0 / 3.0e6 + 4.0;
+    if (s == 1 || t < best) {
+      best = t;
+      best_s = s;
+    }
+  }
+  if (best_s < 2) return false;
+  p.splits = (int)best_s;
+  p.partial_bytes = best_s * M * N * 4;
+  return true;
+}
+
+template <int D_DT, int BIAS_DT>
+static int launch_mid(const LinearArgs &a, const MidPlan &p, float *partial, hipStream_t st) {
+  const SplitK sk{partial, p.splits};
+  const int rc = a.M <= 128 ? launch_tile256p_mi<D_DT, BIAS_DT, 2>(a, sk, st) : launch_tile256p_mi<D_DT, BIAS_DT, 4>(a, sk, st);
+  if (rc) return rc;
+  SkinnyArgs r{a.D, nullptr, nullptr, nullptr, a.A_gs, a.B_gs, a.bias, partial, a.M, a.N, a.K, a.Np, 0, p.splits};
+  hipLaunchKernelGGL((skinny_reduce_kernel<D_DT, BIAS_DT>), dim3((unsigned)ceil_div(a.M * a.N, 256)), dim3(256), 0, st, r);
+  return 0;
+}
+
+template <int D_DT>
+static int dispatch_mid_bias(const LinearArgs &a, const MidPlan &p, float *partial, int bias_dtype, hipStream_t st) {
+  if (!a.bias) return launch_mid<D_DT, BIAS_NONE>(a, p, partial, st);
+  switch (bias_dtype) {
+    case AC4K_DTYPE_BF16: return launch_mid<D_DT, AC4K_DTYPE_BF16>(a, p, partial, st);
+    case AC4K_DTYPE_FP16: return launch_mid<D_DT, AC4K_DTYPE_FP16>(a, p, partial, st);
+    case AC4K_DTYPE_FP32: return launch_mid<D_DT, AC4K_DTYPE_FP32>(a, p, partial, st);
+  }
+  return set_error("bias must be bfloat16, half or float (dtype tag %d)", bias_dtype);
+}
+
+static int dispatch_mid(const LinearArgs &a, const MidPlan &p, float *partial, int d_dtype, int bias_dtype,
+                        hipStream_t st) {
+  switch (d_dtype) {
+    case AC4K_DTYPE_BF16: return dispatch_mid_bias<AC4K_DTYPE_BF16>(a, p, partial, bias_dtype, st);
+    case AC4K_DTYPE_FP16: return dispatch_mid_bias<AC4K_DTYPE_FP16>(a, p, partial, bias_dtype, st);
+    case AC4K_DTYPE_FP32: return dispatch_mid_bias<AC4K_DTYPE_FP32>(a, p, partial, bias_dtype, st);
+  }
+  return set_error("d must be bfloat16, half or float (dtype tag %d)", d_dtype);
+}
+
 // shared tail of the two decode-sized entry points: Ahat is in the workspace already
 static int run_skinny(void *D, int d_dtype, const float *A_gs, const void *B, const void *B_sf, const float *B_gs,
                       const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, const SkinnyPlan &p,
@@ -1327,7 +1503,7 @@ static int run_skinny(void *D, int d_dtype, const float *A_gs, const void *B, co
 }
 
 static int check_skinny(const SkinnyPlan &p, bool ok, const void *B, void *workspace, int64_t workspace_bytes) {
-  AC4K_REQUIRE(ok, "the decode-sized linear takes 1 <= M <= 32 and K %% 256 == 0");
+  AC4K_REQUIRE(ok, "no workspace-assisted path for this shape (ac4k_linear_nvfp4_skinny_workspace_bytes returns 0)");
   AC4K_REQUIRE(((uintptr_t)B & 15) == 0, "weights must be 16-byte aligned");
   AC4K_REQUIRE(workspace && ((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
   AC4K_REQUIRE(workspace_bytes >= p.ahat_bytes + p.partial_bytes, "workspace too small: %lld bytes needed",
@@ -1339,8 +1515,10 @@ static int check_skinny(const SkinnyPlan &p, bool ok, const void *B, void *works
 
 extern "C" __attribute__((visibility("default"))) int64_t ac4k_linear_nvfp4_skinny_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   SkinnyPlan p;
-  if (!skinny_plan(M, N, K, p)) return 0;
-  return p.ahat_bytes + p.partial_bytes;
+  if (skinny_plan(M, N, K, p)) return p.ahat_bytes + p.partial_bytes;
+  MidPlan mp;
+  if (mid_plan(M, N, K, mp)) return mp.partial_bytes;
+  return 0;
 }
 
 extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_skinny(void *D, int d_dtype, const void *A, const void *A_sf, const float *A_gs,
@@ -1348,10 +1526,22 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_skinny(v
                                         int bias_dtype, int64_t M, int64_t N, int64_t K, void *workspace,
                                         int64_t workspace_bytes, ac4k_stream_t stream) {
   AC4K_REQUIRE(D && A && A_sf && A_gs && B && B_sf && B_gs, "null pointer argument");
+  hipStream_t st = (hipStream_t)stream;
+  MidPlan mp;
+  if (M > 32 && mid_plan(M, N, K, mp)) {  // few tiles, long K: split-K over the tile kernel
+    AC4K_REQUIRE((((uintptr_t)A | (uintptr_t)B) & 15) == 0, "A and B must be 16-byte aligned");
+    AC4K_REQUIRE(workspace && ((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
+    AC4K_REQUIRE(workspace_bytes >= mp.partial_bytes, "workspace too small: %lld bytes needed",
+                 (long long)mp.partial_bytes);
+    LinearArgs la{D, static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B),
+                  static_cast<const uint32_t *>(A_sf), static_cast<const uint32_t *>(B_sf), A_gs, B_gs, bias,
+                  M, N, K, align_up(M, 16), align_up(N, 16)};
+    if (int rc = dispatch_mid(la, mp, static_cast<float *>(workspace), d_dtype, bias_dtype, st)) return rc;
+    return check_launch("ac4k_linear_nvfp4_skinny");
+  }
   SkinnyPlan p;
   const bool ok = skinny_plan(M, N, K, p);
   if (int rc = check_skinny(p, ok, B, workspace, workspace_bytes)) return rc;
-  hipStream_t st = (hipStream_t)stream;
   const int64_t dwords = M * (K >> 3);
   hipLaunchKernelGGL(decode_activation_kernel, dim3((unsigned)ceil_div(dwords, 256)), dim3(256), 0, st,
                      static_cast<_Float16 *>(workspace), static_cast<const uint8_t *>(A),

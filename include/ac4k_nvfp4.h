@@ -98,12 +98,16 @@ int ac4k_linear_nvfp4(void *D, int d_dtype, const void *A, const void *A_sf, con
                       const void *B, const void *B_sf, const float *B_gs, const void *bias,
                       int bias_dtype, int64_t M, int64_t N, int64_t K, ac4k_stream_t stream);
 
-/* Decode-sized linear (1 <= M <= 32, K % 256 == 0): same contract as ac4k_linear_nvfp4
- * (lib/cuda/sm120/linear_nvfp4.cu:753-901; the reference runs these shapes through its one
- * 128x128 tile kernel), implemented as a weight-streaming split-K kernel.  It needs scratch:
- * `workspace` = ac4k_linear_nvfp4_skinny_workspace_bytes(M,N,K) bytes of device memory,
- * 256-byte aligned, contents irrelevant (it receives the fp16 activation and the fp32 partial
- * sums of the K-slices).  The size function returns 0 for shapes this path does not take. */
+/* Linear for shapes that need device scratch to run well: same contract as ac4k_linear_nvfp4
+ * (lib/cuda/sm120/linear_nvfp4.cu:753-901; the reference runs every shape through its one
+ * 128x128 tile kernel).  Two families:
+ *   - decode-sized, 1 <= M <= 32 and K % 256 == 0: a weight-streaming split-K kernel; the
+ *     workspace receives the fp16 activation and the fp32 partial sums of the K-slices;
+ *   - 32 < M with too few output tiles to fill the GPU and K % 128 == 0: split-K over the tile
+ *     kernel; the workspace receives the fp32 partial sums.
+ * `workspace` = ac4k_linear_nvfp4_skinny_workspace_bytes(M,N,K) bytes of device memory, 256-byte
+ * aligned, contents irrelevant.  The size function returns 0 for shapes that gain nothing from
+ * scratch; those go to ac4k_linear_nvfp4. */
 int64_t ac4k_linear_nvfp4_skinny_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int ac4k_linear_nvfp4_skinny(void *D, int d_dtype, const void *A, const void *A_sf, const float *A_gs,
                              const void *B, const void *B_sf, const float *B_gs, const void *bias,

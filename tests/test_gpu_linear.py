@@ -152,6 +152,45 @@ def test_fused_decode_config5(m):
     torch.testing.assert_close(d1, full, atol=ATOL, rtol=RTOL)
 
 
+# 32 < M with few output tiles: the 128-row packed tile, with split-K through a workspace when K is
+# long enough, and without (short K, or N too small for the packed kernel)
+MID_SHAPES = [(33, 512, 1024), (64, 256, 4096), (100, 300, 2048), (128, 1024, 4096), (128, 4096, 1024),
+              (129, 512, 2048), (200, 333, 1536), (256, 512, 8192), (128, 520, 512), (48, 128, 256),
+              (96, 2050, 1152), (128, 14336, 4096)]
+
+
+@pytest.mark.parametrize("m,n,k", MID_SHAPES)
+def test_mid_m_shapes(m, n, k):
+    from ac4k_kernel_amd import _lib
+    run_case(m, n, k, seed=m + k, wstd=0.02)
+    if _lib.load().ac4k_linear_nvfp4_skinny_workspace_bytes(m, n, k) > 0:
+        # the split-K reduction applies bias and output type in its own kernel
+        run_case(m, n, k, bias_dtype=torch.float32, o_dtype=torch.float16, seed=m + k + 1, wstd=0.02)
+        run_case(m, n, k, bias_dtype=torch.bfloat16, o_dtype=torch.float32, seed=m + k + 2, wstd=0.02)
+
+
+def test_mid_m_workspace_entry_matches_plain_entry():
+    """The workspace-assisted entry point and ac4k_linear_nvfp4 compute the same contract; with fp32
+    output they agree to accumulation-order noise."""
+    from ac4k_kernel_amd import _lib
+    L = _lib.load()
+    m, n, k = 128, 1024, 4096
+    aq, bq = gpu_quant(make_input((m, k), seed=1)), gpu_quant(make_input((n, k), seed=2, std=0.02))
+    nbytes = L.ac4k_linear_nvfp4_skinny_workspace_bytes(m, n, k)
+    assert nbytes > 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    d1 = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    d2 = torch.empty_like(d1)
+    st = torch.cuda.current_stream().cuda_stream
+    args = (aq[0].data_ptr(), aq[1].data_ptr(), aq[2].data_ptr(), bq[0].data_ptr(), bq[1].data_ptr(), bq[2].data_ptr(),
+            None, 0, m, n, k)
+    _lib.check(L.ac4k_linear_nvfp4(d1.data_ptr(), 2, *args, st))
+    _lib.check(L.ac4k_linear_nvfp4_skinny(d2.data_ptr(), 2, *args, ws.data_ptr(), nbytes, st))
+    torch.testing.assert_close(d1.cpu(), d2.cpu(), atol=1e-5, rtol=1e-4)
+    assert L.ac4k_linear_nvfp4_skinny(d2.data_ptr(), 2, *args, ws.data_ptr(), nbytes - 1, st) != 0
+    assert b"workspace too small" in L.ac4k_last_error()
+
+
 def test_error_behaviour():
     o = ops()
     aq, bq = gpu_quant(make_input((8, 128), seed=1)), gpu_quant(make_input((16, 128), seed=2))
