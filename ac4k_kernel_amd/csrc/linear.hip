@@ -37,10 +37,12 @@ struct Elem<AC4K_DTYPE_BF16> {
   static __device__ __forceinline__ float load(const void *p, int64_t i) {
     return bf16_bits_to_f32(static_cast<const uint16_t *>(p)[i]);
   }
-  static __device__ __forceinline__ T cvt(float f) {  // round to nearest even, NaN kept quiet
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (T)((u >> 16) | 0x40u);
-    return (T)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+  // round to nearest even, NaN stays NaN: v_cvt_pk_bf16_f32
+  static __device__ __forceinline__ T cvt(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+  static __device__ __forceinline__ uint32_t cvt2(float lo, float hi) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
   }
 };
 template <>
@@ -50,6 +52,10 @@ struct Elem<AC4K_DTYPE_FP16> {
     return (float)static_cast<const _Float16 *>(p)[i];
   }
   static __device__ __forceinline__ T cvt(float f) { return (_Float16)f; }
+  static __device__ __forceinline__ uint32_t cvt2(float lo, float hi) {
+    const f16x2 v = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
 };
 template <>
 struct Elem<AC4K_DTYPE_FP32> {
@@ -58,6 +64,7 @@ struct Elem<AC4K_DTYPE_FP32> {
     return static_cast<const float *>(p)[i];
   }
   static __device__ __forceinline__ T cvt(float f) { return f; }
+  static __device__ __forceinline__ uint32_t cvt2(float lo, float) { return __float_as_uint(lo); }  // unused: 4-byte outputs are not packed
 };
 constexpr int BIAS_NONE = 3;
 
@@ -819,7 +826,7 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   const int fb_off = PL::OFF_B + (wn * 128 + (lane & 31)) * P_ROW + half * 16;
   const int sa_off = PL::OFF_SFA + (wm * (32 * MI) + (lane & 31)) * 4;
   const int sb_off = PL::OFF_SFB + (wn * 128 + (lane & 31)) * 4;
-  const int sh = half * 16;
+  const int sh = half * 16;  // a lane needs the two scale bytes of its half of the chunk
 
   uint4 PA[2][MI], PB[2][4];  // packed fragments of a 64-chunk, double buffered by chunk parity
   f16x2 SA[2][MI], SB[2][4];  // their two block scales (blocks 2*half, 2*half+1) as fp16
@@ -834,7 +841,7 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     for (int i = 0; i < 4; ++i) {
       if (i < MI) {
         uint32_t wa = *reinterpret_cast<const uint32_t *>(st + sa_off + c * (BM * 4) + i * 128);
-        SA[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((wa >> sh) & 0x7f7fu, 1.0f, false);
+        SA[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((wa >> sh) & 0x7f7fu, 1.0f, false);  // scales are unsigned e4m3
       }
       uint32_t wb = *reinterpret_cast<const uint32_t *>(st + sb_off + c * (P_BN * 4) + i * 128);
       SB[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((wb >> sh) & 0x7f7fu, 1.0f, false);
@@ -1011,11 +1018,8 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
         for (int j = 0; j < 4; ++j)
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            typename DE::T h[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) h[q] = DE::cvt(value(i, j, g * 4 + q));
-            uint2 w;
-            __builtin_memcpy(&w, h, 8);
+            const uint2 w = make_uint2(DE::cvt2(value(i, j, g * 4), value(i, j, g * 4 + 1)),
+                                       DE::cvt2(value(i, j, g * 4 + 2), value(i, j, g * 4 + 3)));
             *reinterpret_cast<uint2 *>(stg + (ii * 32 + (lane & 31)) * PITCH + (j * 32 + g * 8 + half * 4) * 2) = w;
           }
       }
