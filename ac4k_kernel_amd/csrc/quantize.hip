@@ -520,6 +520,75 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
   if (!REPAIR && tid == 0) g_onepass.done[slot][w] = tag | 0x80000000u;
 }
 
+// ---------------------------------------------------------------------------
+// Tiny dense tensors (at most NV * 1024 vectors of 8 elements): one workgroup holds everything in
+// registers, so global scale and quantize are one launch with an ordinary
+// workgroup barrier in between.  EMIT also writes the dequantized block values e2m1 * fp32(sf) as
+// fp16 (exact) to f16out [rows, K] for the decode-sized linear.
+template <int NV, bool EMIT>
+__global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_single_wg_kernel(
+    uint32_t *__restrict__ out, uint32_t *__restrict__ sf, const uint4 *__restrict__ in, float *__restrict__ gs_out,
+    OnePassGeom g, float max_scale, _Float16 *__restrict__ f16out) {
+  __shared__ float lut[128];
+  __shared__ uint32_t red[OP_THREADS / 64];
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t nvec = g.total_chunks * 8;
+  uint4 v[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const uint32_t lv = j * OP_THREADS + tid;
+    v[j] = make_uint4(0, 0, 0, 0);
+    if (lv < nvec) v[j] = in[lv];
+  }
+  if (tid < 128) lut[tid] = g_rcp_e4m3.v[tid];
+  uint32_t bm[NV], m = 0;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    bm[j] = absmax_bf16x8(v[j]);
+    bm[j] = umax32(bm[j], dpp_u32<DPP_QUAD_XOR1>(bm[j]));
+    m = umax32(m, bm[j]);
+  }
+  m = group_umax<64>(m);
+  if (lane == 0) red[wave] = m;
+  __syncthreads();
+  const uint32_t gm = group_umax<16>(red[lane & 15]);
+  const float gs = bf16_bits_to_f32(gm) / max_scale;
+  if (tid == 0) *gs_out = gs;
+  const float alpha = 1.0f / gs;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const uint32_t lv = j * OP_THREADS + tid;
+    uint32_t code;
+    const float o = nvfp4_block_scale(bf16_bits_to_f32(bm[j]), alpha, lut, code);
+    const uint32_t packed = nvfp4_pack8(v[j], o);
+    const uint32_t sfw = code | (dpp_u32<DPP_ROW_SHL(2)>(code) << 8) | (dpp_u32<DPP_ROW_SHL(4)>(code) << 16) |
+                         (dpp_u32<DPP_ROW_SHL(6)>(code) << 24);
+    if (lv < nvec) {
+      out[lv] = packed;
+      if ((lane & 7) == 0) {
+        const uint32_t ch = lv >> 3, row = ch / g.ncc, cc = ch - row * g.ncc;
+        const uint32_t l = g.lead > 1 ? row / g.R : 0u, r = row - l * g.R;
+        sf[((uint64_t)l * g.ncc + cc) * g.Rp + r] = sfw;
+      }
+      if constexpr (EMIT) {
+        const f16x2 sc2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(code, 1.0f, false);
+        const f16x2 sc = {sc2.x, sc2.x};
+        const f16x2 d0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 0) * sc;
+        const f16x2 d1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 1) * sc;
+        const f16x2 d2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 2) * sc;
+        const f16x2 d3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 3) * sc;
+        reinterpret_cast<uint4 *>(f16out)[lv] =
+            make_uint4(__builtin_bit_cast(uint32_t, d0), __builtin_bit_cast(uint32_t, d1),
+                       __builtin_bit_cast(uint32_t, d2), __builtin_bit_cast(uint32_t, d3));
+      }
+    }
+  }
+  if (g.Rp > g.R) {  // zero scales of the pad rows R..Rp-1
+    const uint32_t pad = g.Rp - g.R, npad = g.lead * g.ncc * pad;
+    for (uint32_t i = tid; i < npad; i += OP_THREADS) sf[(uint64_t)(i / pad) * g.Rp + g.R + i % pad] = 0u;
+  }
+}
+
 // ===========================================================================
 // per-row fp8 / int8
 // ===========================================================================
@@ -649,6 +718,200 @@ __global__ __launch_bounds__(256) void quantize_rowwise_generic_kernel(
   }
 }
 
+// ===========================================================================
+// Cross dim contiguous, reduce dim strided (the layout of V in attention: quantize(v, 3, N_dim)).
+//
+// A lane (kb = lane % 4, rg = lane / 4) owns eight consecutive rows (one 16-byte load along the
+// contiguous cross dim) and the 16 reduce positions of output block kb of a 64-chunk: 16 loads,
+// each of which a wave issues as four 256-byte row segments.  Blocks run along the loop index,
+// so block maxima, products and nibble/byte packing all stay inside the lane - no transposition -
+// and the swizzles are only a different choice of the 16 source positions.  Four adjacent lanes
+// hold the four blocks of a chunk: their stores of one row are contiguous.
+// ===========================================================================
+
+// bf16 component j (0..7) of a 16-byte vector as float
+__device__ __forceinline__ float bf16_comp(const uint4 &v, int j) {
+  const uint32_t w = (j >> 1) == 0 ? v.x : (j >> 1) == 1 ? v.y : (j >> 1) == 2 ? v.z : v.w;
+  return (j & 1) ? bf16_hi(w) : bf16_lo(w);
+}
+
+// element-wise |bf16| maximum of two vectors of eight
+__device__ __forceinline__ uint4 absmax_bf16x8_pairwise(uint4 acc, uint4 v) {
+  auto mx = [](uint32_t a, uint32_t b) {
+    const u16x2 r = __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b & 0x7fff7fffu));
+    return __builtin_bit_cast(uint32_t, r);
+  };
+  return make_uint4(mx(acc.x, v.x), mx(acc.y, v.y), mx(acc.z, v.z), mx(acc.w, v.w));
+}
+__device__ __forceinline__ uint32_t u16_comp(const uint4 &v, int j) {
+  const uint32_t w = (j >> 1) == 0 ? v.x : (j >> 1) == 1 ? v.y : (j >> 1) == 2 ? v.z : v.w;
+  return (j & 1) ? (w >> 16) : (w & 0xffffu);
+}
+
+// source position inside a 32-group (nvfp4) or 16-group (fp8) of output position p
+__device__ __forceinline__ int nvfp4_swizzle_src(int p) { return ((p & 7) >> 1) * 8 + (p >> 3) * 2 + (p & 1); }
+__device__ __forceinline__ int fp8_swizzle_src(int p) { return ((p & 3) >> 1) * 8 + (p >> 2) * 2 + (p & 1); }
+
+template <bool SWIZZLE>
+__global__ __launch_bounds__(256) void quantize_nvfp4_crossmajor_kernel(
+    uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in, GlobalScaleSrc gsrc,
+    QuantGeom g) {
+  __shared__ float lut[128];
+  load_rcp_table(lut);
+  const float alpha = load_alpha(gsrc, blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kb = lane & 3, rg = lane >> 2;
+  const int64_t cc = (int64_t)blockIdx.x * 4 + wave;            // 64-chunk along the reduce dim
+  const int64_t row0 = (int64_t)blockIdx.y * 128 + rg * 8;      // first of the lane's eight rows
+  const int64_t lead = blockIdx.z;
+  if (cc * 64 >= g.Kp || row0 >= g.Rp) return;
+  const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + row0;
+  const bool rows_valid = row0 < g.R;  // R % 8 == 0: all eight or none
+
+  uint4 v[16];
+  uint4 m8 = make_uint4(0, 0, 0, 0);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int p = (kb & 1) * 16 + i;  // output position inside the 32-group
+    const int64_t k = cc * 64 + (kb >> 1) * 32 + (SWIZZLE ? nvfp4_swizzle_src(p) : p);
+    v[i] = make_uint4(0, 0, 0, 0);
+    if (rows_valid && k < g.K) v[i] = *reinterpret_cast<const uint4 *>(src + k * g.sK);
+  }
+#pragma unroll
+  for (int i = 0; i < 16; ++i) m8 = absmax_bf16x8_pairwise(m8, v[i]);
+
+  uint32_t code[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float o = nvfp4_block_scale(bf16_bits_to_f32(u16_comp(m8, j)), alpha, lut, code[j]);
+    if (!rows_valid) code[j] = 0;  // pad rows carry zero scales
+    float f0[8], f1[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      f0[i] = bf16_comp(v[i], j) * o;
+      f1[i] = bf16_comp(v[8 + i], j) * o;
+    }
+    const uint2 packed = (o != o) ? make_uint2(0x77777777u, 0x77777777u) : make_uint2(f32x8_to_e2m1x8(f0), f32x8_to_e2m1x8(f1));
+    if (rows_valid)
+      *reinterpret_cast<uint2 *>(out + (lead * g.R + row0 + j) * (g.Kp / 2) + cc * 32 + kb * 8) = packed;
+  }
+  // scale dword of (row, chunk) = the codes of the four lanes of the quad; lane kb stores rows 2kb, 2kb+1
+  uint32_t sfw[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    sfw[j] = dpp_u32<0x00>(code[j]) | (dpp_u32<0x55>(code[j]) << 8) | (dpp_u32<0xAA>(code[j]) << 16) |
+             (dpp_u32<0xFF>(code[j]) << 24);
+  const uint2 mine = kb == 0 ? make_uint2(sfw[0], sfw[1])
+                   : kb == 1 ? make_uint2(sfw[2], sfw[3])
+                   : kb == 2 ? make_uint2(sfw[4], sfw[5]) : make_uint2(sfw[6], sfw[7]);
+  *reinterpret_cast<uint2 *>(reinterpret_cast<uint32_t *>(sf) + (lead * (g.Kp / 64) + cc) * g.Rp + row0 + 2 * kb) = mine;
+}
+
+// ---- per-row fp8 / int8 with the reduce dim strided: the row maximum is collected with atomic
+// maxima of bf16 bit patterns into the (zeroed) scale array, the quantize kernel reads them, and a
+// last kernel turns them into amax / scale_max in place.
+__global__ void fill_u32_kernel(uint32_t *__restrict__ p, int64_t n, uint32_t v) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+constexpr int CM_KSPAN = 2048;  // reduce positions per workgroup of the maximum kernel
+
+__global__ __launch_bounds__(256) void rowwise_crossmajor_amax_kernel(uint32_t *__restrict__ amax_bits,
+                                                                       const uint16_t *__restrict__ in, QuantGeom g) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kq = lane & 3, rg = lane >> 2;
+  const int64_t row0 = (int64_t)blockIdx.y * 128 + rg * 8;
+  const int64_t lead = blockIdx.z;
+  const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + row0;
+  uint4 m8 = make_uint4(0, 0, 0, 0);
+  if (row0 < g.R) {
+    const int64_t kbeg = (int64_t)blockIdx.x * CM_KSPAN, kend = kbeg + CM_KSPAN < g.K ? kbeg + CM_KSPAN : g.K;
+    for (int64_t k = kbeg + wave * 4 + kq; k < kend; k += 64) {  // four loads in flight per lane
+      uint4 a[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        a[u] = make_uint4(0, 0, 0, 0);
+        if (k + u * 16 < kend) a[u] = *reinterpret_cast<const uint4 *>(src + (k + u * 16) * g.sK);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) m8 = absmax_bf16x8_pairwise(m8, a[u]);
+    }
+  }
+  // quad (same rows, different k) -> one value per row; then across the four waves through LDS
+  auto quad_max = [](uint32_t w) {
+    u16x2 x = __builtin_bit_cast(u16x2, w);
+    x = __builtin_elementwise_max(x, __builtin_bit_cast(u16x2, dpp_u32<DPP_QUAD_XOR1>(w)));
+    const uint32_t y = __builtin_bit_cast(uint32_t, x);
+    x = __builtin_elementwise_max(x, __builtin_bit_cast(u16x2, dpp_u32<DPP_QUAD_XOR2>(y)));
+    return __builtin_bit_cast(uint32_t, x);
+  };
+  m8 = make_uint4(quad_max(m8.x), quad_max(m8.y), quad_max(m8.z), quad_max(m8.w));
+  __shared__ uint4 red[4][16];
+  if (kq == 0) red[wave][rg] = m8;
+  __syncthreads();
+  if (wave == 0 && kq == 0 && row0 < g.R) {
+    uint4 t = red[0][rg];
+#pragma unroll
+    for (int w2 = 1; w2 < 4; ++w2) t = absmax_bf16x8_pairwise(t, red[w2][rg]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t b = u16_comp(t, j);
+      if (b) atomicMax(amax_bits + lead * g.Rp + row0 + j, b);
+    }
+  }
+}
+
+template <RowFmt FMT, bool SWIZZLE>
+__global__ __launch_bounds__(256) void quantize_rowwise_crossmajor_kernel(
+    uint8_t *__restrict__ out, const uint32_t *__restrict__ amax_bits, const uint16_t *__restrict__ in,
+    const void *__restrict__ smax_p, QuantGeom g) {
+  const float smax = load_scale_max<FMT>(smax_p);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kb = lane & 3, rg = lane >> 2;
+  const int64_t k0 = ((int64_t)blockIdx.x * 4 + wave) * 64 + kb * 16;  // the lane's 16 output positions
+  const int64_t row0 = (int64_t)blockIdx.y * 128 + rg * 8;
+  const int64_t lead = blockIdx.z;
+  if (k0 >= g.Kp || row0 >= g.R) return;
+  const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + row0;
+  uint4 v[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int64_t k = k0 + (SWIZZLE ? fp8_swizzle_src(i) : i);
+    v[i] = make_uint4(0, 0, 0, 0);
+    if (k < g.K) v[i] = *reinterpret_cast<const uint4 *>(src + k * g.sK);
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float amax = bf16_bits_to_f32(amax_bits[lead * g.Rp + row0 + j]);
+    const float recp = smax / amax;
+    const bool nan_row = (FMT == RowFmt::FP8) && (amax == 0.0f);
+    float f[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) f[i] = bf16_comp(v[i], j) * recp;
+    uint4 w;
+    if (FMT == RowFmt::FP8) {
+      w = make_uint4(f32x4_to_e4m3x4(f[0], f[1], f[2], f[3]), f32x4_to_e4m3x4(f[4], f[5], f[6], f[7]),
+                     f32x4_to_e4m3x4(f[8], f[9], f[10], f[11]), f32x4_to_e4m3x4(f[12], f[13], f[14], f[15]));
+      if (nan_row) w = make_uint4(0x7f7f7f7fu, 0x7f7f7f7fu, 0x7f7f7f7fu, 0x7f7f7f7fu);
+    } else {
+      auto p4 = [&](int b) {
+        return f32_to_s8_sat(f[b]) | (f32_to_s8_sat(f[b + 1]) << 8) | (f32_to_s8_sat(f[b + 2]) << 16) |
+               (f32_to_s8_sat(f[b + 3]) << 24);
+      };
+      w = make_uint4(p4(0), p4(4), p4(8), p4(12));
+    }
+    *reinterpret_cast<uint4 *>(out + (lead * g.R + row0 + j) * g.Kp + k0) = w;
+  }
+}
+
+// amax bit patterns -> amax / scale_max, in place (pad rows hold 0 -> 0 / scale_max)
+template <RowFmt FMT>
+__global__ void rowwise_crossmajor_finalize_kernel(float *__restrict__ sf, const void *__restrict__ smax_p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) sf[i] = bf16_bits_to_f32(__float_as_uint(sf[i])) / load_scale_max<FMT>(smax_p);
+}
+
 // ---------------------------------------------------------------------------
 // host launchers
 // ---------------------------------------------------------------------------
@@ -666,6 +929,12 @@ static int check_geom(const void *out, const void *sf, const void *in, const voi
 static bool rowmajor_ok(const void *in, int64_t K, int64_t s0, int64_t s1, int64_t sR, int64_t sK) {
   return sK == 1 && K % 8 == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0 && sR % 8 == 0 &&
          s0 % 8 == 0 && s1 % 8 == 0;
+}
+
+// cross dim contiguous, every row group of eight 16-byte aligned
+static bool crossmajor_ok(const void *in, int64_t R, int64_t s0, int64_t s1, int64_t sR, int64_t sK) {
+  return sR == 1 && R % 8 == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0 && sK % 8 == 0 && s0 % 8 == 0 &&
+         s1 % 8 == 0;
 }
 
 template <int CPR>
@@ -778,6 +1047,25 @@ static void launch_onepass(uint32_t *out, uint32_t *sf, const uint4 *in, float *
                      g, slot, max_scale, ticks);
 }
 
+// One workgroup streams at a few tens of GB/s, so this only pays for tensors of a few KB: above two
+// 16 KB segments the two-launch paths are faster.
+constexpr int SINGLE_WG_MAX_SEGS = 2;
+
+template <bool EMIT>
+static void launch_single_wg(uint32_t *out, uint32_t *sf, const uint4 *in, float *gs, const OnePassGeom &g,
+                             float max_scale, _Float16 *f16out, hipStream_t st) {
+  const int64_t segs = ceil_div((int64_t)g.total_chunks, 128);  // 1024-vector segments
+#define AC4K_SINGLE_WG(NV)                                                                                       \
+  hipLaunchKernelGGL((quantize_nvfp4_single_wg_kernel<NV, EMIT>), dim3(1), dim3(OP_THREADS), 0, st, out, sf, in, \
+                     gs, g, max_scale, f16out)
+  static_assert(SINGLE_WG_MAX_SEGS == 2, "instantiations below");
+  if (segs <= 1)
+    AC4K_SINGLE_WG(1);
+  else
+    AC4K_SINGLE_WG(2);
+#undef AC4K_SINGLE_WG
+}
+
 // Global scale + nvfp4 quantize of a dense [lead, R, K] tensor in one pass over the input, when
 // the shape allows it.  Returns false (nothing launched) when the caller has to take the
 // two-kernel path.
@@ -792,9 +1080,14 @@ static bool try_quantize_nvfp4_onepass(void *out, void *sf, float *gs, const voi
   int nwg = device_cu_count();
   if (nwg > OP_MAX_WGS) nwg = OP_MAX_WGS;
   if (nwg < 8 || chunks > (int64_t)nwg * 128 * OP_MAX_NV) return false;
+  const OnePassGeom g{(uint32_t)chunks, (uint32_t)(K / 64), (uint32_t)R, (uint32_t)align_up(R, 16), (uint32_t)lead};
+  if (chunks <= 128 * SINGLE_WG_MAX_SEGS) {  // tiny: one workgroup, one launch, no grid wait
+    launch_single_wg<false>(static_cast<uint32_t *>(out), static_cast<uint32_t *>(sf), static_cast<const uint4 *>(in), gs,
+                            g, max_scale, nullptr, st);
+    return true;
+  }
   const int slot = amax_slot(st);
   if (slot < 0) return false;
-  const OnePassGeom g{(uint32_t)chunks, (uint32_t)(K / 64), (uint32_t)R, (uint32_t)align_up(R, 16), (uint32_t)lead};
   const int64_t per_wg = ceil_div(chunks, (int64_t)nwg * 128);  // 16 KB segments per workgroup
   uint32_t *o = static_cast<uint32_t *>(out), *s = static_cast<uint32_t *>(sf);
   const uint4 *x = static_cast<const uint4 *>(in);
@@ -828,6 +1121,12 @@ static int launch_quantize_nvfp4(void *out, void *sf, const void *in, const Glob
       launch_nvfp4_rowmajor<2>(o, s, x, gsrc, g, lead, st);
     else
       launch_nvfp4_rowmajor<1>(o, s, x, gsrc, g, lead, st);
+  } else if (crossmajor_ok(in, R, s0, s1, sR, sK) && ceil_div(g.Rp, 128) <= 65535) {
+    dim3 grid((unsigned)ceil_div(g.Kp / 64, 4), (unsigned)ceil_div(g.Rp, 128), (unsigned)lead);
+    if (swizzle)
+      hipLaunchKernelGGL(quantize_nvfp4_crossmajor_kernel<true>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
+    else
+      hipLaunchKernelGGL(quantize_nvfp4_crossmajor_kernel<false>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
   } else {
     AC4K_REQUIRE(g.Kp / 64 <= 65535, "reduce dim too large for the strided path (%lld)", (long long)K);
     dim3 grid((unsigned)ceil_div(g.Rp, 256), (unsigned)(g.Kp / 64), (unsigned)lead);
@@ -888,6 +1187,12 @@ namespace ac4k {
 int quantize_activation_with_f16(void *out, void *sf, float *gs, const void *in, int64_t M, int64_t K,
                                  float max_scale, _Float16 *f16out, hipStream_t st) {
   AC4K_REQUIRE(K % 64 == 0 && rowmajor_ok(in, K, 0, 0, K, 1), "activation must be 16-byte aligned with K %% 64 == 0");
+  if (M * (K / 64) <= 128 * SINGLE_WG_MAX_SEGS) {
+    const OnePassGeom og{(uint32_t)(M * (K / 64)), (uint32_t)(K / 64), (uint32_t)M, (uint32_t)align_up(M, 16), 1u};
+    launch_single_wg<true>(static_cast<uint32_t *>(out), static_cast<uint32_t *>(sf), static_cast<const uint4 *>(in), gs,
+                           og, max_scale, f16out, st);
+    return 0;
+  }
   int slot = -1;
   const int npart = launch_amax_partials(in, M * K, st, &slot);
   GlobalScaleSrc gsrc{gs, slot, npart, max_scale};
@@ -935,6 +1240,21 @@ static int quantize_rowwise(void *out, float *sf, const void *in, const void *sm
       launch_rowwise_rowmajor<FMT, 64, 8>(o, sf, x, smax, g, lead, st);
     else
       launch_rowwise_rowmajor<FMT, 64, 16>(o, sf, x, smax, g, lead, st);
+  } else if (crossmajor_ok(in, R, s0, s1, sR, sK) && ceil_div(g.Rp, 128) <= 65535 && ceil_div(K, CM_KSPAN) <= 65535) {
+    // row maxima as bf16 bit patterns in the scale array, quantize from them, then scale them in place
+    uint32_t *bits = reinterpret_cast<uint32_t *>(sf);
+    const int64_t nsf = lead * g.Rp;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)ceil_div(nsf, 256)), dim3(256), 0, st, bits, nsf, 0u);
+    hipLaunchKernelGGL(rowwise_crossmajor_amax_kernel,
+                       dim3((unsigned)ceil_div(K, CM_KSPAN), (unsigned)ceil_div(g.Rp, 128), (unsigned)lead), dim3(256), 0,
+                       st, bits, x, g);
+    dim3 grid((unsigned)ceil_div(g.Kp / 16, 16), (unsigned)ceil_div(g.Rp, 128), (unsigned)lead);
+    if (swizzle)
+      hipLaunchKernelGGL((quantize_rowwise_crossmajor_kernel<FMT, true>), grid, dim3(256), 0, st, o, bits, x, smax, g);
+    else
+      hipLaunchKernelGGL((quantize_rowwise_crossmajor_kernel<FMT, false>), grid, dim3(256), 0, st, o, bits, x, smax, g);
+    hipLaunchKernelGGL(rowwise_crossmajor_finalize_kernel<FMT>, dim3((unsigned)ceil_div(nsf, 256)), dim3(256), 0, st, sf,
+                       smax, nsf);
   } else {
     dim3 grid((unsigned)ceil_div(g.Rp, 256), (unsigned)lead);
     if (swizzle)

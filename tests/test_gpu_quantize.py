@@ -143,6 +143,26 @@ def test_nvfp4_single_launch_two_streams():
             assert torch.equal(out.cpu(), exp[i][0]) and torch.equal(sf.cpu().view(torch.uint8), exp[i][1])
 
 
+# cross dim contiguous, reduce dim strided (the layout of V in the reference's attention wrappers,
+# python/ac4k_kernel/ops/attention.py:116,169; its bandwidth test uses (1, 75600, 40, 128))
+CROSSMAJOR_SHAPES = [((1, 756, 40, 128), 3, 1), ((2, 100, 3, 40), 3, 1), ((200, 128), 1, 0), ((77, 8), 1, 0),
+                     ((5, 1000, 24), 2, 1), ((3, 2, 4100, 16), 3, 2), ((2100, 136), 1, 0)]
+
+
+@pytest.mark.parametrize("shape,cross,red", CROSSMAJOR_SHAPES)
+@pytest.mark.parametrize("swz", [False, True])
+def test_crossmajor_layouts(shape, cross, red, swz):
+    x = make_input(shape, seed=shape[-1] + red, outliers=True)
+    check_nvfp4(x, cross, red, swz)
+    out, sf = ops().quantize(x.cuda(), cross, red, precision="fp8e4m3", swizzle=swz)
+    eo, es = T.quantize_fp8(x, cross, red, None, swz)
+    assert torch.equal(out.cpu().view(torch.uint8), eo) and torch.equal(sf.cpu(), es)
+    if not swz:
+        out, sf = ops().quantize(x.cuda(), cross, red, precision="int8")
+        eo, es = T.quantize_int8(x, cross, red)
+        assert torch.equal(out.cpu(), eo) and torch.equal(sf.cpu(), es)
+
+
 def test_nvfp4_graph_replay():
     """A captured quantize call replays correctly: nothing in it depends on host-side state that
     changes from launch to launch, and eager calls in between do not disturb it."""
