@@ -675,6 +675,37 @@ __global__ __launch_bounds__(256) void quantize_rowwise_rowmajor_kernel(
   }
 }
 
+// Rows longer than the register budget of the kernel above: one wave per row, two passes over the
+// row (the second one is served by the caches), 16-byte loads, 8-byte stores.
+template <RowFmt FMT>
+__global__ __launch_bounds__(256) void quantize_rowwise_longrow_kernel(
+    uint8_t *__restrict__ out, float *__restrict__ sf, const uint16_t *__restrict__ in,
+    const void *__restrict__ smax_p, QuantGeom g) {
+  const float smax = load_scale_max<FMT>(smax_p);
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t lead = blockIdx.y;
+  if (r >= g.Rp) return;
+  if (r >= g.R) {
+    if (lane == 0) sf[lead * g.Rp + r] = 0.0f / smax;
+    return;
+  }
+  const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + r * g.sR;
+  uint32_t m = 0;
+  for (int64_t k = lane * 8; k < g.K; k += 512) m = umax32(m, absmax_bf16x8(*reinterpret_cast<const uint4 *>(src + k)));
+  m = group_umax<64>(m);
+  const float amax = bf16_bits_to_f32(m);
+  if (lane == 0) sf[lead * g.Rp + r] = amax / smax;
+  const float recp = smax / amax;
+  const bool nan_row = (FMT == RowFmt::FP8) && (amax == 0.0f);
+  uint8_t *op = out + (lead * g.R + r) * g.Kp;
+  for (int64_t k = lane * 8; k < g.Kp; k += 512) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (k < g.K) v = *reinterpret_cast<const uint4 *>(src + k);
+    st_stream_u2(op + k, rowfmt_pack8<FMT>(v, recp, nan_row));
+  }
+}
+
 // Generic path: any strides / swizzle / K.  One lane per row, two passes over the row.
 template <RowFmt FMT, bool SWIZZLE>
 __global__ __launch_bounds__(256) void quantize_rowwise_generic_kernel(
@@ -1223,7 +1254,7 @@ static int quantize_rowwise(void *out, float *sf, const void *in, const void *sm
   uint8_t *o = static_cast<uint8_t *>(out);
   const uint16_t *x = static_cast<const uint16_t *>(in);
   const int64_t lead = d0 * d1;
-  if (!swizzle && rowmajor_ok(in, K, s0, s1, sR, sK) && K <= 8192) {
+  if (!swizzle && rowmajor_ok(in, K, s0, s1, sR, sK) && K <= 16384) {
     if (K <= 64)
       launch_rowwise_rowmajor<FMT, 8, 1>(o, sf, x, smax, g, lead, st);
     else if (K <= 128)
@@ -1238,8 +1269,13 @@ static int quantize_rowwise(void *out, float *sf, const void *in, const void *sm
       launch_rowwise_rowmajor<FMT, 64, 4>(o, sf, x, smax, g, lead, st);
     else if (K <= 4096)
       launch_rowwise_rowmajor<FMT, 64, 8>(o, sf, x, smax, g, lead, st);
-    else
+    else if (K <= 8192)
       launch_rowwise_rowmajor<FMT, 64, 16>(o, sf, x, smax, g, lead, st);
+    else
+      launch_rowwise_rowmajor<FMT, 64, 32>(o, sf, x, smax, g, lead, st);
+  } else if (!swizzle && rowmajor_ok(in, K, s0, s1, sR, sK)) {  // rows too long for the register file
+    dim3 grid((unsigned)ceil_div(g.Rp, 4), (unsigned)lead);
+    hipLaunchKernelGGL((quantize_rowwise_longrow_kernel<FMT>), grid, dim3(256), 0, st, o, sf, x, smax, g);
   } else if (crossmajor_ok(in, R, s0, s1, sR, sK) && ceil_div(g.Rp, 128) <= 65535 && ceil_div(K, CM_KSPAN) <= 65535) {
     // row maxima as bf16 bit patterns in the scale array, quantize from them, then scale them in place
     uint32_t *bits = reinterpret_cast<uint32_t *>(sf);
