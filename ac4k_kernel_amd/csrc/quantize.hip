@@ -336,6 +336,7 @@ struct OnePassSync {
   uint32_t arrive[AMAX_SLOTS][OP_MAX_WGS];
   uint32_t done[AMAX_SLOTS][OP_MAX_WGS];
   uint32_t epoch[AMAX_SLOTS];
+  uint32_t giveup[AMAX_SLOTS];  // launches left for which the grid wait is skipped (see below)
 };
 __device__ __align__(256) OnePassSync g_onepass;
 
@@ -378,13 +379,24 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
   const uint32_t w = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // the launch tag: the main launch derives it from the slot's counter, the repair launch reads it
   // back from workgroup 0's word (published whatever happened next) and advances the counter
+  // A workgroup whose wait really ran out marks done[w] with bit 30; the repair launch then arms
+  // giveup[slot], and for that many launches the main kernel does not wait at all (its work is
+  // redone by the repair launch, at the speed of the two-kernel path), so that a GPU shared with
+  // other kernels costs one 200 us stall in 65 launches, not one per launch.
   uint32_t tag;
   if (REPAIR) {
     tag = g_onepass.arrive[slot][0] >> 16;
     if (w == 0 && tid == 0) g_onepass.epoch[slot] = tag;
-    if (g_onepass.done[slot][w] == (tag | 0x80000000u)) return;
+    const uint32_t d = g_onepass.done[slot][w];
+    if (d == (tag | 0x80000000u)) return;
+    if (d == (tag | 0x40000000u) && tid == 0) g_onepass.giveup[slot] = 64;
   } else {
     tag = (g_onepass.epoch[slot] + 1) & 0xffffu;
+    const uint32_t gu = g_onepass.giveup[slot];
+    if (gu) {
+      timeout_ticks = 0;
+      if (w == 0 && tid == 0) g_onepass.giveup[slot] = gu - 1;
+    }
   }
 
   AC4K_TL(0);
@@ -444,7 +456,10 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
       __builtin_amdgcn_s_sleep(2);
     }
     mm = group_umax<64>(mm);
-    if (lane == 0) gmax_s = ok ? mm : 0xffffffffu;
+    if (lane == 0) {
+      gmax_s = ok ? mm : 0xffffffffu;
+      if (!REPAIR && !ok && timeout_ticks) g_onepass.done[slot][w] = tag | 0x40000000u;  // a wait that ran out
+    }
   }
   __syncthreads();
   const uint32_t gm = gmax_s;
