@@ -262,22 +262,10 @@ __device__ __forceinline__ PackedRow load_row(const uint8_t *base, const uint32_
 // decode 16-block `q` (0..3) of a packed row into its two 16-byte LDS chunks
 __device__ __forceinline__ void decode_block_to_lds(_Float16 *tile, int row, int q, uint32_t w0, uint32_t w1,
                                                     uint32_t sfw) {
-#ifdef EXP_NO_DECODE
-  return;
-#endif
   f16x2 sp = scale_pattern(sfw >> (8 * q));
   f16x2 lo[4], hi[4];
-#ifdef EXP_NO_VALU
-  for (int i = 0; i < 4; ++i) { lo[i] = __builtin_bit_cast(f16x2, w0); hi[i] = __builtin_bit_cast(f16x2, w1 + sfw); }
-#else
   decode8(w0, sp, lo);
   decode8(w1, sp, hi);
-#endif
-#ifdef EXP_NO_WRITE
-  if (__builtin_bit_cast(uint32_t, lo[0]) != 0x12345678u || __builtin_bit_cast(uint32_t, hi[3]) != 0x9abcdef0u ||
-      __builtin_bit_cast(uint32_t, lo[1]) + __builtin_bit_cast(uint32_t, lo[2]) + __builtin_bit_cast(uint32_t, lo[3]) +
-      __builtin_bit_cast(uint32_t, hi[0]) + __builtin_bit_cast(uint32_t, hi[1]) + __builtin_bit_cast(uint32_t, hi[2]) != 0x1111u) return;
-#endif
   uint4 v0 = make_uint4(__builtin_bit_cast(uint32_t, lo[0]), __builtin_bit_cast(uint32_t, lo[1]),
                         __builtin_bit_cast(uint32_t, lo[2]), __builtin_bit_cast(uint32_t, lo[3]));
   uint4 v1 = make_uint4(__builtin_bit_cast(uint32_t, hi[0]), __builtin_bit_cast(uint32_t, hi[1]),
@@ -297,9 +285,6 @@ struct Frags {
 
 __device__ __forceinline__ void load_frags(Frags &f, const _Float16 *cA, const _Float16 *cB, int arow, int brow,
                                            int chunk) {
-#ifdef EXP_NO_LDSREAD
-  if (chunk >= 0) return;
-#endif
 #pragma unroll
   for (int i = 0; i < 4; ++i) f.a[i] = lds_frag(cA, arow + i * 32, chunk);
 #pragma unroll
@@ -491,123 +476,6 @@ __device__ __forceinline__ void decode_half_block(_Float16 *tile, int row, int h
   decode_block_to_lds(tile, row, half * 2 + b, w0, w1, r.sf);
 }
 
-template <int D_DT, int BIAS_DT>
-__global__ __launch_bounds__(512) void linear_nvfp4_tile256w8_kernel(LinearArgs a) {
-  extern __shared__ __attribute__((aligned(16))) _Float16 lds[];  // [2 buffers][A tile | B tile]
-
-  const int64_t tiles_m = ceil_div(a.M, L_BM), tiles_n = ceil_div(a.N, L_BN);
-  const int64_t ntiles = tiles_m * tiles_n;
-  int64_t pid = blockIdx.x;
-  {  // contiguous run of tiles per XCD (workgroups are dealt round-robin to the 8 XCDs)
-    const int64_t per = ntiles / 8, rem = ntiles % 8;
-    const int64_t xcd = pid % 8, idx = pid / 8;
-    pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
-  }
-  constexpr int GROUP_M = 4;
-  const int64_t group = pid / (GROUP_M * tiles_n);
-  const int64_t first_m = group * GROUP_M;
-  const int64_t gsize = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
-  const int64_t tm = first_m + (pid % (GROUP_M * tiles_n)) % gsize;
-  const int64_t tn = (pid % (GROUP_M * tiles_n)) / gsize;
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 2, wn = wave & 3;
-  const int ld_row = tid >> 1, ld_half = tid & 1;
-  int64_t arow = tm * L_BM + ld_row, brow = tn * L_BN + ld_row;
-  arow = arow < a.M ? arow : a.M - 1;  // rows past the matrix feed accumulators that are never stored
-  brow = brow < a.N ? brow : a.N - 1;
-  const int nk = (int)(a.K / L_BK), klast = nk - 1;
-  const int fa_row = wm * 128 + (lane & 31), fb_row = wn * 64 + (lane & 31), half = lane >> 5;
-
-  f32x16 acc[4][2];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-
-  PackedHalfRow ra0 = load_half_row(a.A, a.A_sf, a.Mp, a.K, arow, ld_half, 0);
-  PackedHalfRow rb0 = load_half_row(a.B, a.B_sf, a.Np, a.K, brow, ld_half, 0);
-#pragma unroll
-  for (int b = 0; b < 2; ++b) {
-    decode_half_block(lds, ld_row, ld_half, b, ra0);
-    decode_half_block(lds + L_TILE_HALVES, ld_row, ld_half, b, rb0);
-  }
-  ra0 = load_half_row(a.A, a.A_sf, a.Mp, a.K, arow, ld_half, 1 < klast ? 1 : klast);
-  rb0 = load_half_row(a.B, a.B_sf, a.Np, a.K, brow, ld_half, 1 < klast ? 1 : klast);
-  PackedHalfRow ra1 = load_half_row(a.A, a.A_sf, a.Mp, a.K, arow, ld_half, 2 < klast ? 2 : klast);
-  PackedHalfRow rb1 = load_half_row(a.B, a.B_sf, a.Np, a.K, brow, ld_half, 2 < klast ? 2 : klast);
-  __syncthreads();
-
-  f16x8 fa[4], fb[2];
-  auto frags = [&](const _Float16 *cA, const _Float16 *cB, int ks) {
-#ifdef EXP_NO_LDSREAD
-    if (ks >= 0) return;
-#endif
-#pragma unroll
-    for (int i = 0; i < 4; ++i) fa[i] = lds_frag(cA, fa_row + i * 32, ks * 2 + half);
-#pragma unroll
-    for (int j = 0; j < 2; ++j) fb[j] = lds_frag(cB, fb_row + j * 32, ks * 2 + half);
-  };
-  auto mfma8 = [&]() {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
-  };
-
-  for (int kt = 0; kt < nk; ++kt) {
-    const _Float16 *cA = lds + (kt & 1) * (2 * L_TILE_HALVES);
-    const _Float16 *cB = cA + L_TILE_HALVES;
-    _Float16 *nA = lds + ((kt + 1) & 1) * (2 * L_TILE_HALVES);
-    _Float16 *nB = nA + L_TILE_HALVES;
-    // ra0/rb0 hold step kt+1 (decoded now), ra1/rb1 hold step kt+2 (possibly still in flight)
-    frags(cA, cB, 0);
-    decode_half_block(nA, ld_row, ld_half, 0, ra0);
-    decode_half_block(nA, ld_row, ld_half, 1, ra0);
-    mfma8();
-    frags(cA, cB, 1);
-    decode_half_block(nB, ld_row, ld_half, 0, rb0);
-    mfma8();
-    frags(cA, cB, 2);
-    decode_half_block(nB, ld_row, ld_half, 1, rb0);
-    mfma8();
-    frags(cA, cB, 3);
-    __syncthreads();  // next buffer complete; nobody reads the current buffer any more
-    const int kn = kt + 3 < klast ? kt + 3 : klast;
-    ra0 = ra1;
-    rb0 = rb1;
-    ra1 = load_half_row(a.A, a.A_sf, a.Mp, a.K, arow, ld_half, kn);
-    rb1 = load_half_row(a.B, a.B_sf, a.Np, a.K, brow, ld_half, kn);
-    mfma8();
-  }
-
-  const float scale = (*a.A_gs) * (*a.B_gs);
-  using DE = Elem<D_DT>;
-  typename DE::T *D = static_cast<typename DE::T *>(a.D);
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int64_t n = tn * L_BN + wn * 64 + j * 32 + (lane & 31);
-    float bv = 0.0f;
-    if constexpr (BIAS_DT != BIAS_NONE) {
-      if (n < a.N) bv = Elem<BIAS_DT>::load(a.bias, n);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int64_t m = tm * L_BM + wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (m < a.M && n < a.N) {
-          float v = acc[i][j][e] * scale;
-          if constexpr (BIAS_DT != BIAS_NONE) v += bv;
-          D[m * a.N + n] = DE::cvt(v);
-        }
-      }
-    }
-  }
-}
 
 // ===========================================================================
 // BM x 256 tile (BM = 256 or 128), packed operands in LDS, decode after the fragment load.
@@ -1074,33 +942,17 @@ static int launch_tile256p(const LinearArgs &a, hipStream_t st) {
 
 constexpr int L_LDS_BYTES = 2 * 2 * L_TILE_HALVES * (int)sizeof(_Float16);  // 128 KiB
 
-enum class LinearKernel { AUTO, TILE128, TILE256, TILE256W8, TILE256P };
+enum class LinearKernel { AUTO, TILE128, TILE256, TILE256P };
 
 static LinearKernel forced_kernel() {  // benchmarking aid: AC4K_LINEAR_KERNEL=tile128|tile256
   static const LinearKernel k = [] {
     const char *e = getenv("AC4K_LINEAR_KERNEL");
     if (e && !strcmp(e, "tile128")) return LinearKernel::TILE128;
     if (e && !strcmp(e, "tile256")) return LinearKernel::TILE256;
-    if (e && !strcmp(e, "tile256w8")) return LinearKernel::TILE256W8;
     if (e && !strcmp(e, "tile256p")) return LinearKernel::TILE256P;
     return LinearKernel::AUTO;
   }();
   return k;
-}
-
-template <int D_DT, int BIAS_DT>
-static int launch_tile256w8(const LinearArgs &a, hipStream_t st) {
-  auto *kern = linear_nvfp4_tile256w8_kernel<D_DT, BIAS_DT>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, L_LDS_BYTES);
-    if (e != hipSuccess) return set_error("hipFuncSetAttribute(LDS=%d): %s", L_LDS_BYTES, hipGetErrorString(e));
-    attr_set = true;
-  }
-  const int64_t ntiles = ceil_div(a.M, L_BM) * ceil_div(a.N, L_BN);
-  hipLaunchKernelGGL(kern, dim3((unsigned)ntiles), dim3(512), L_LDS_BYTES, st, a);
-  return 0;
 }
 
 template <int D_DT, int BIAS_DT>
@@ -1360,7 +1212,6 @@ static int launch_linear(const LinearArgs &a, hipStream_t st) {
   }
   if (k == LinearKernel::TILE256P && packed_ok) return launch_tile256p<D_DT, BIAS_DT>(a, st);
   if (k == LinearKernel::TILE256 && big_ok) return launch_tile256<D_DT, BIAS_DT>(a, st);
-  if (k == LinearKernel::TILE256W8 && big_ok) return launch_tile256w8<D_DT, BIAS_DT>(a, st);
   const int64_t ntiles = ceil_div(a.M, T_BM) * ceil_div(a.N, T_BN);
   hipLaunchKernelGGL((linear_nvfp4_tile128_kernel<D_DT, BIAS_DT>), dim3((unsigned)ntiles), dim3(256), 0, st, a);
   return 0;

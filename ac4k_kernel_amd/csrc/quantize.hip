@@ -188,7 +188,36 @@ __device__ __forceinline__ uint32_t nvfp4_pack8(uint4 v, float o) {
   return (o != o) ? 0x77777777u : f32x8_to_e2m1x8(f);
 }
 
-// Row-major fast path: reduce dim contiguous, no swizzle, K % 8 == 0, 16-byte aligned rows.
+// The swizzles on a contiguous reduce dim are small in-register transpositions between adjacent
+// lanes (a lane holds 8 consecutive elements = 4 dwords of 2).
+// nvfp4, 32-groups = 4 lanes: out[t*8 + q*2 + r] = in[q*8 + t*2 + r], i.e. lane t / dword q receives
+// lane q / dword t: a 4x4 transpose of dwords inside the quad, done as two butterfly stages.
+__device__ __forceinline__ uint4 swizzle_nvfp4_quad(uint4 v, int lane) {
+  uint32_t d[4] = {v.x, v.y, v.z, v.w};
+  const bool o1 = lane & 1, o2 = lane & 2;
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {  // 2x2 blocks: (q even, t odd) <-> (q odd, t even)
+    const uint32_t got = dpp_u32<DPP_QUAD_XOR1>(o1 ? d[2 * b] : d[2 * b + 1]);
+    if (o1) d[2 * b] = got; else d[2 * b + 1] = got;
+  }
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {  // off-diagonal 2x2 blocks: (q < 2, t >= 2) <-> (q >= 2, t < 2)
+    const uint32_t got = dpp_u32<DPP_QUAD_XOR2>(o2 ? d[c] : d[c + 2]);
+    if (o2) d[c] = got; else d[c + 2] = got;
+  }
+  return make_uint4(d[0], d[1], d[2], d[3]);
+}
+// fp8, 16-groups = 2 lanes: out[t*4 + q*2 + r] = in[q*8 + t*2 + r]: lane 0 gets dwords (a0, b0, a1, b1)
+// and lane 1 gets (a2, b2, a3, b3) of the pair's inputs a (lane 0) and b (lane 1).
+__device__ __forceinline__ uint4 swizzle_fp8_pair(uint4 v, int lane) {
+  const bool o = lane & 1;
+  // each lane needs two dwords of its partner: lane 0 wants b0, b1; lane 1 wants a2, a3
+  const uint32_t g0 = dpp_u32<DPP_QUAD_XOR1>(o ? v.x : v.z);  // lane 0 receives b.x, lane 1 receives a.z
+  const uint32_t g1 = dpp_u32<DPP_QUAD_XOR1>(o ? v.y : v.w);  // lane 0 receives b.y, lane 1 receives a.w
+  return o ? make_uint4(g0, v.z, g1, v.w) : make_uint4(v.x, g0, v.y, g1);
+}
+
+// Row-major fast path: reduce dim contiguous, K % 8 == 0, 16-byte aligned rows.
 // A lane owns 8 consecutive elements (half a 16-block); lane pairs share the block amax
 // through one DPP quad_perm; the four scale bytes of a 64-chunk are gathered into the
 // chunk's first lane with three DPP row shifts and stored as one dword.
@@ -196,7 +225,7 @@ __device__ __forceinline__ uint32_t nvfp4_pack8(uint4 v, float o) {
 //   ITER = wave passes per workgroup (independent loads in flight per lane)
 //   EMIT = also write the dequantized block values e2m1 * fp32(sf) as fp16 (exact) to `f16out`
 //          [rows, K] (2-D inputs only): the decode-sized linear consumes them directly
-template <int CPR, int ITER, bool EMIT>
+template <int CPR, int ITER, bool EMIT, bool SWIZZLE>
 __global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
     uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in, GlobalScaleSrc gsrc,
     QuantGeom g, _Float16 *__restrict__ f16out) {
@@ -221,6 +250,7 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
     v[it] = make_uint4(0, 0, 0, 0);
     if (kvalid && r < g.R)
       v[it] = ld_stream_u4(src + r * g.sR);
+    if (SWIZZLE) v[it] = swizzle_nvfp4_quad(v[it], lane);
   }
 #pragma unroll
   for (int it = 0; it < ITER; ++it) {
@@ -656,7 +686,7 @@ __device__ __forceinline__ uint2 rowfmt_pack8(uint4 v, float recp, bool nan_row)
 // Row-major fast path: the whole row lives in registers between the amax pass and the
 // convert pass, so the input is read from memory once.  LPR lanes share a row (DPP / swizzle
 // reduction), each lane holds NV 16-byte vectors at a stride of LPR*8 elements.
-template <RowFmt FMT, int LPR, int NV>
+template <RowFmt FMT, int LPR, int NV, bool SWIZZLE>
 __global__ __launch_bounds__(256) void quantize_rowwise_rowmajor_kernel(
     uint8_t *__restrict__ out, float *__restrict__ sf, const uint16_t *__restrict__ in,
     const void *__restrict__ smax_p, QuantGeom g) {
@@ -674,6 +704,7 @@ __global__ __launch_bounds__(256) void quantize_rowwise_rowmajor_kernel(
     v[j] = make_uint4(0, 0, 0, 0);
     if (r < g.R && k < g.K) v[j] = ld_stream_u4(src + k);
     m = umax32(m, absmax_bf16x8(v[j]));
+    if (SWIZZLE) v[j] = swizzle_fp8_pair(v[j], threadIdx.x);
   }
   m = group_umax<LPR>(m);
   const float amax = bf16_bits_to_f32(m);
@@ -985,16 +1016,20 @@ static bool crossmajor_ok(const void *in, int64_t R, int64_t s0, int64_t s1, int
 
 template <int CPR>
 static void launch_nvfp4_rowmajor(uint8_t *out, uint8_t *sf, const uint16_t *in, const GlobalScaleSrc &gs,
-                                  const QuantGeom &g, int64_t lead, hipStream_t st, _Float16 *f16out = nullptr) {
+                                  const QuantGeom &g, int64_t lead, hipStream_t st, _Float16 *f16out = nullptr,
+                                  bool swizzle = false) {
   constexpr int ITER = 4;
   constexpr int ROWS = 4 * (8 / CPR) * ITER;
   dim3 grid((unsigned)(ceil_div(g.Kp / 64, CPR) * ceil_div(g.Rp, ROWS)), (unsigned)lead);
   if (f16out)
-    hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER, true>), grid, dim3(256), 0, st, out, sf, in, gs, g,
-                       f16out);
+    hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER, true, false>), grid, dim3(256), 0, st, out, sf, in, gs,
+                       g, f16out);
+  else if (swizzle)
+    hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER, false, true>), grid, dim3(256), 0, st, out, sf, in, gs,
+                       g, f16out);
   else
-    hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER, false>), grid, dim3(256), 0, st, out, sf, in, gs, g,
-                       f16out);
+    hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER, false, false>), grid, dim3(256), 0, st, out, sf, in,
+                       gs, g, f16out);
 }
 
 }  // namespace ac4k
@@ -1157,16 +1192,17 @@ static int launch_quantize_nvfp4(void *out, void *sf, const void *in, const Glob
   uint8_t *o = static_cast<uint8_t *>(out), *s = static_cast<uint8_t *>(sf);
   const uint16_t *x = static_cast<const uint16_t *>(in);
   const int64_t lead = d0 * d1;
-  if (!swizzle && rowmajor_ok(in, K, s0, s1, sR, sK) && ceil_div(g.Kp, 64) * ceil_div(g.Rp, 16) < (1ll << 31)) {
+  if (rowmajor_ok(in, K, s0, s1, sR, sK) && ceil_div(g.Kp, 64) * ceil_div(g.Rp, 16) < (1ll << 31)) {
     const int64_t chunks = g.Kp / 64;
+    const bool sw = swizzle != 0;
     if (chunks >= 8)
-      launch_nvfp4_rowmajor<8>(o, s, x, gsrc, g, lead, st);
+      launch_nvfp4_rowmajor<8>(o, s, x, gsrc, g, lead, st, nullptr, sw);
     else if (chunks >= 3)
-      launch_nvfp4_rowmajor<4>(o, s, x, gsrc, g, lead, st);
+      launch_nvfp4_rowmajor<4>(o, s, x, gsrc, g, lead, st, nullptr, sw);
     else if (chunks == 2)
-      launch_nvfp4_rowmajor<2>(o, s, x, gsrc, g, lead, st);
+      launch_nvfp4_rowmajor<2>(o, s, x, gsrc, g, lead, st, nullptr, sw);
     else
-      launch_nvfp4_rowmajor<1>(o, s, x, gsrc, g, lead, st);
+      launch_nvfp4_rowmajor<1>(o, s, x, gsrc, g, lead, st, nullptr, sw);
   } else if (crossmajor_ok(in, R, s0, s1, sR, sK) && ceil_div(g.Rp, 128) <= 65535) {
     dim3 grid((unsigned)ceil_div(g.Kp / 64, 4), (unsigned)ceil_div(g.Rp, 128), (unsigned)lead);
     if (swizzle)
@@ -1254,10 +1290,14 @@ int quantize_activation_with_f16(void *out, void *sf, float *gs, const void *in,
 
 template <RowFmt FMT, int LPR, int NV>
 static void launch_rowwise_rowmajor(uint8_t *out, float *sf, const uint16_t *in, const void *smax,
-                                    const QuantGeom &g, int64_t lead, hipStream_t st) {
+                                    const QuantGeom &g, int64_t lead, hipStream_t st, bool swizzle) {
   dim3 grid((unsigned)ceil_div(g.Rp, 256 / LPR), (unsigned)lead);
-  hipLaunchKernelGGL((quantize_rowwise_rowmajor_kernel<FMT, LPR, NV>), grid, dim3(256), 0, st, out, sf, in,
-                     smax, g);
+  if (swizzle && FMT == RowFmt::FP8)
+    hipLaunchKernelGGL((quantize_rowwise_rowmajor_kernel<FMT, LPR, NV, FMT == RowFmt::FP8>), grid, dim3(256), 0, st, out,
+                       sf, in, smax, g);
+  else
+    hipLaunchKernelGGL((quantize_rowwise_rowmajor_kernel<FMT, LPR, NV, false>), grid, dim3(256), 0, st, out, sf, in,
+                       smax, g);
 }
 
 template <RowFmt FMT>
@@ -1269,25 +1309,26 @@ static int quantize_rowwise(void *out, float *sf, const void *in, const void *sm
   uint8_t *o = static_cast<uint8_t *>(out);
   const uint16_t *x = static_cast<const uint16_t *>(in);
   const int64_t lead = d0 * d1;
-  if (!swizzle && rowmajor_ok(in, K, s0, s1, sR, sK) && K <= 16384) {
+  if (rowmajor_ok(in, K, s0, s1, sR, sK) && K <= 16384) {
+    const bool sw = swizzle != 0;
     if (K <= 64)
-      launch_rowwise_rowmajor<FMT, 8, 1>(o, sf, x, smax, g, lead, st);
+      launch_rowwise_rowmajor<FMT, 8, 1>(o, sf, x, smax, g, lead, st, sw);
     else if (K <= 128)
-      launch_rowwise_rowmajor<FMT, 16, 1>(o, sf, x, smax, g, lead, st);
+      launch_rowwise_rowmajor<FMT, 16, 1>(o, sf, x, smax, g, lead, st, sw);
     else if (K <= 256)
-      launch_rowwise_rowmajor<FMT, 32, 1>(o, sf, x, smax, g, lead, st);
+      launch_rowwise_rowmajor<FMT, 32, 1>(o, sf, x, smax, g, lead, st, sw);
     else if (K <= 512)
-      launch_rowwise_rowmajor<FMT, 64, 1>(o, sf, x, smax, g, lead, st);
+      launch_rowwise_rowmajor<FMT, 64, 1>(o, sf, x, smax, g, lead, st, sw);
     else if (K <= 1024)
-      launch_rowwise_rowmajor<FMT, 64, 2>(o, sf, x, smax, g, lead, st);
+      launch_rowwise_rowmajor<FMT, 64, 2>(o, sf, x, smax, g, lead, st, sw);
     else if (K <= 2048)
-      launch_rowwise_rowmajor<FMT, 64, 4>(o, sf, x, smax, g, lead, st);
+      launch_rowwise_rowmajor<FMT, 64, 4>(o, sf, x, smax, g, lead, st, sw);
     else if (K <= 4096)
-      launch_rowwise_rowmajor<FMT, 64, 8>(o, sf, x, smax, g, lead, st);
+      launch_rowwise_rowmajor<FMT, 64, 8>(o, sf, x, smax, g, lead, st, sw);
     else if (K <= 8192)
-      launch_rowwise_rowmajor<FMT, 64, 16>(o, sf, x, smax, g, lead, st);
+      launch_rowwise_rowmajor<FMT, 64, 16>(o, sf, x, smax, g, lead, st, sw);
     else
-      launch_rowwise_rowmajor<FMT, 64, 32>(o, sf, x, smax, g, lead, st);
+      launch_rowwise_rowmajor<FMT, 64, 32>(o, sf, x, smax, g, lead, st, sw);
   } else if (!swizzle && rowmajor_ok(in, K, s0, s1, sR, sK)) {  // rows too long for the register file
     dim3 grid((unsigned)ceil_div(g.Rp, 4), (unsigned)lead);
     hipLaunchKernelGGL((quantize_rowwise_longrow_kernel<FMT>), grid, dim3(256), 0, st, o, sf, x, smax, g);
