@@ -191,6 +191,39 @@ def test_mid_m_workspace_entry_matches_plain_entry():
     assert b"workspace too small" in L.ac4k_last_error()
 
 
+def test_graph_replay_of_linear_paths():
+    """Captured calls of the tile kernel, the split-K path and the fused decode path replay correctly
+    with eager work in between (no host-side state is baked into a launch)."""
+    k, n = 2048, 512
+    wq = gpu_quant(make_input((n, k), seed=3, std=0.02))
+    cases = []
+    for m, fused in ((1, True), (16, True), (128, False), (300, False)):
+        x = make_input((m, k), seed=m).cuda()
+        xs = x.clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):  # warm-up outside the capture
+            if fused:
+                ops().fused_linear(xs, *wq)
+            else:
+                ops().linear(*ops().quantize(xs, 0, 1), *wq)
+        torch.cuda.current_stream().wait_stream(side)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            d = ops().fused_linear(xs, *wq) if fused else ops().linear(*ops().quantize(xs, 0, 1), *wq)
+        cases.append((m, xs, g, d))
+    for rep in range(3):
+        for m, xs, g, d in cases:
+            x = make_input((m, k), seed=100 * rep + m)
+            xs.copy_(x.cuda())
+            g.replay()
+            torch.cuda.synchronize()
+            aq = T.quantize_nvfp4(x, 0, 1, False)
+            ref = T.linear_nvfp4(*aq, *cpu(wq))
+            torch.testing.assert_close(d.cpu(), ref, atol=ATOL, rtol=RTOL)
+        run_case(40, 96, 256, seed=rep)  # eager work between the replays
+
+
 def test_error_behaviour():
     o = ops()
     aq, bq = gpu_quant(make_input((8, 128), seed=1)), gpu_quant(make_input((16, 128), seed=2))

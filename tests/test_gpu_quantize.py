@@ -187,6 +187,26 @@ def test_nvfp4_graph_replay():
         check_nvfp4(make_input((300, 640), seed=seed), 0, 1)  # eager work between the replays
 
 
+def test_nvfp4_many_streams():
+    """More (device, stream) pairs than the library has scratch slots: the late streams take the
+    paths without scratch and every result is still exact."""
+    x = make_input((300, 640), seed=21, outliers=True)
+    big = make_input((2048, 2048), seed=22)
+    ex, eb = T.quantize_nvfp4(x, 0, 1, False), T.quantize_nvfp4(big, 0, 1, False)
+    dx, db = x.cuda(), big.cuda()
+    streams = [torch.cuda.Stream() for _ in range(40)]
+    torch.cuda.synchronize()
+    results = []
+    for st in streams:
+        with torch.cuda.stream(st):
+            results.append((ops().quantize(dx, 0, 1), ops().quantize(db, 0, 1)))
+    torch.cuda.synchronize()
+    for rx, rb in results:
+        for (out, sf, gs), (eo, es, eg) in ((rx, ex), (rb, eb)):
+            assert gs.item() == eg.item()
+            assert torch.equal(out.cpu(), eo) and torch.equal(sf.cpu().view(torch.uint8), es)
+
+
 def test_nvfp4_caller_buffers_and_negative_dims():
     x = make_input((40, 192), seed=3).cuda()
     out = torch.full((40, 96), 0xAA, dtype=torch.uint8, device="cuda")
