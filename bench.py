@@ -171,6 +171,20 @@ def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True, key=None):
             "roofline": rl}
 
 
+def vendor_gemm_yardstick(steps, warmup, n=8192):
+    """What the vendor library's dense 16-bit GEMM (torch.matmul) sustains on this box at n^3: not part
+    of the product and not a baseline of the metric (its operands are dense fp16/bf16, nothing is
+    decoded), only a measure of how far the 2.5 PFLOP/s peak is reachable at this box's clocks."""
+    res = {"workload": f"torch.matmul M=N=K={n}, dense operands"}
+    for name, dt in (("bf16", torch.bfloat16), ("fp16", torch.float16)):
+        a = torch.randn((n, n), device="cuda", dtype=dt)
+        b = torch.randn((n, n), device="cuda", dtype=dt)
+        _, ms = time_gpu(lambda: torch.matmul(a, b.t()), steps, warmup)
+        res[f"{name}_TFLOP/s"] = 2.0 * n ** 3 / (ms * 1e-3) / 1e12
+        del a, b
+    return res
+
+
 def bench_decode(ops, m, n, k, steps, warmup, check=True):
     """Fused decode-sized linear: bf16 activation in, on-the-fly NVFP4 quantize + GEMM."""
     x = make_input((m, k), seed=2, outliers=True).cuda()
@@ -271,6 +285,10 @@ def main():
             line["cpu_baseline"] = cpu_linear_baseline(8192, 8192)
             log(f"[bench] cpu linear oracle: {line['cpu_baseline']['value']:.3f} TFLOP/s")
         if args.workload == "all":
+            line["vendor_dense_gemm"] = vendor_gemm_yardstick(S, W)
+            log(f"[bench] yardstick, torch.matmul 8192^3 on already dense operands: "
+                f"{line['vendor_dense_gemm']['bf16_TFLOP/s']:.0f} TFLOP/s bf16, "
+                f"{line['vendor_dense_gemm']['fp16_TFLOP/s']:.0f} TFLOP/s fp16")
             shapes = {"cfg3_4096": bench_linear(ops, 4096, 4096, 4096, S, W, check=check)}
             for (n, k) in ((14336, 4096), (4096, 14336)):
                 for m in (16, 128, 2048, 8192):
