@@ -121,6 +121,7 @@ __global__ __launch_bounds__(AMAX_THREADS) void amax_scale_bf16_atomic_kernel(
 struct QuantGeom {
   int64_t d1, R, K, Kp, Rp;
   int64_t s0, s1, sR, sK;
+  int64_t lead0;  // first leading index of this launch (grids carry at most 65535 of them)
 };
 
 // Where a quantize kernel gets the global scale from: a device scalar (slot < 0), or the
@@ -235,7 +236,7 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
   constexpr int LPR = 8 * CPR;   // lanes per row
   constexpr int RW = 64 / LPR;   // rows per wave pass
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t lead = blockIdx.y;
+  const int64_t lead = blockIdx.y + g.lead0;
   const int64_t ngroups = ceil_div(g.Kp / 64, CPR);  // chunk groups along the reduce dim
   const int64_t k = ((int64_t)(blockIdx.x % ngroups) * LPR + (lane % LPR)) * 8;
   const int64_t row0 = (int64_t)(blockIdx.x / ngroups) * (4 * RW * ITER) + lane / LPR;
@@ -294,7 +295,7 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_generic_kernel(
   load_rcp_table(lut);
   const float alpha = load_alpha(gsrc, blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0);
   const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t chunk = blockIdx.y, lead = blockIdx.z;
+  const int64_t chunk = blockIdx.y, lead = blockIdx.z + g.lead0;
   if (r >= g.Rp) return;
   uint32_t *sfp = reinterpret_cast<uint32_t *>(sf) + (lead * (g.Kp / 64) + chunk) * g.Rp + r;
   if (r >= g.R) {
@@ -694,7 +695,7 @@ __global__ __launch_bounds__(256) void quantize_rowwise_rowmajor_kernel(
   constexpr int RPB = 256 / LPR;  // rows per block
   const int sub = threadIdx.x % LPR;
   const int64_t r = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
-  const int64_t lead = blockIdx.y;
+  const int64_t lead = blockIdx.y + g.lead0;
   const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + r * g.sR;
   uint4 v[NV];
   uint32_t m = 0;
@@ -730,7 +731,7 @@ __global__ __launch_bounds__(256) void quantize_rowwise_longrow_kernel(
   const float smax = load_scale_max<FMT>(smax_p);
   const int lane = threadIdx.x & 63;
   const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int64_t lead = blockIdx.y;
+  const int64_t lead = blockIdx.y + g.lead0;
   if (r >= g.Rp) return;
   if (r >= g.R) {
     if (lane == 0) sf[lead * g.Rp + r] = 0.0f / smax;
@@ -759,7 +760,7 @@ __global__ __launch_bounds__(256) void quantize_rowwise_generic_kernel(
     const void *__restrict__ smax_p, QuantGeom g) {
   const float smax = load_scale_max<FMT>(smax_p);
   const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t lead = blockIdx.y;
+  const int64_t lead = blockIdx.y + g.lead0;
   if (r >= g.Rp) return;
   if (r >= g.R) {
     sf[lead * g.Rp + r] = 0.0f / smax;
@@ -840,7 +841,7 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_crossmajor_kernel(
   const int kb = lane & 3, rg = lane >> 2;
   const int64_t cc = (int64_t)blockIdx.x * 4 + wave;            // 64-chunk along the reduce dim
   const int64_t row0 = (int64_t)blockIdx.y * 128 + rg * 8;      // first of the lane's eight rows
-  const int64_t lead = blockIdx.z;
+  const int64_t lead = blockIdx.z + g.lead0;
   if (cc * 64 >= g.Kp || row0 >= g.Rp) return;
   const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + row0;
   const bool rows_valid = row0 < g.R;  // R % 8 == 0: all eight or none
@@ -899,7 +900,7 @@ __global__ __launch_bounds__(256) void rowwise_crossmajor_amax_kernel(uint32_t *
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int kq = lane & 3, rg = lane >> 2;
   const int64_t row0 = (int64_t)blockIdx.y * 128 + rg * 8;
-  const int64_t lead = blockIdx.z;
+  const int64_t lead = blockIdx.z + g.lead0;
   const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + row0;
   uint4 m8 = make_uint4(0, 0, 0, 0);
   if (row0 < g.R) {
@@ -948,7 +949,7 @@ __global__ __launch_bounds__(256) void quantize_rowwise_crossmajor_kernel(
   const int kb = lane & 3, rg = lane >> 2;
   const int64_t k0 = ((int64_t)blockIdx.x * 4 + wave) * 64 + kb * 16;  // the lane's 16 output positions
   const int64_t row0 = (int64_t)blockIdx.y * 128 + rg * 8;
-  const int64_t lead = blockIdx.z;
+  const int64_t lead = blockIdx.z + g.lead0;
   if (k0 >= g.Kp || row0 >= g.R) return;
   const uint16_t *src = in + (lead / g.d1) * g.s0 + (lead % g.d1) * g.s1 + row0;
   uint4 v[16];
@@ -999,7 +1000,6 @@ static int check_geom(const void *out, const void *sf, const void *in, const voi
   AC4K_REQUIRE(d0 >= 1 && d1 >= 1 && R >= 1 && K >= 1, "sizes must be positive (d0=%lld d1=%lld R=%lld K=%lld)",
                (long long)d0, (long long)d1, (long long)R, (long long)K);
   AC4K_REQUIRE(s0 >= 0 && s1 >= 0 && sR >= 1 && sK >= 1, "strides must be positive");
-  AC4K_REQUIRE(d0 * d1 <= 65535, "product of the leading dims must be <= 65535 (got %lld)", (long long)(d0 * d1));
   return 0;
 }
 
@@ -1188,10 +1188,12 @@ static bool try_quantize_nvfp4_onepass(void *out, void *sf, float *gs, const voi
 static int launch_quantize_nvfp4(void *out, void *sf, const void *in, const GlobalScaleSrc &gsrc, int64_t d0,
                                  int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR, int64_t sK,
                                  int swizzle, hipStream_t st) {
-  QuantGeom g{d1, R, K, align_up(K, 64), align_up(R, 16), s0, s1, sR, sK};
+  QuantGeom g{d1, R, K, align_up(K, 64), align_up(R, 16), s0, s1, sR, sK, 0};
   uint8_t *o = static_cast<uint8_t *>(out), *s = static_cast<uint8_t *>(sf);
   const uint16_t *x = static_cast<const uint16_t *>(in);
-  const int64_t lead = d0 * d1;
+  const int64_t lead_all = d0 * d1;
+  for (g.lead0 = 0; g.lead0 < lead_all; g.lead0 += 65535) {
+  const int64_t lead = lead_all - g.lead0 < 65535 ? lead_all - g.lead0 : 65535;
   if (rowmajor_ok(in, K, s0, s1, sR, sK) && ceil_div(g.Kp, 64) * ceil_div(g.Rp, 16) < (1ll << 31)) {
     const int64_t chunks = g.Kp / 64;
     const bool sw = swizzle != 0;
@@ -1216,6 +1218,7 @@ static int launch_quantize_nvfp4(void *out, void *sf, const void *in, const Glob
       hipLaunchKernelGGL(quantize_nvfp4_generic_kernel<true>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
     else
       hipLaunchKernelGGL(quantize_nvfp4_generic_kernel<false>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
+  }
   }
   return 0;
 }
@@ -1282,7 +1285,7 @@ int quantize_activation_with_f16(void *out, void *sf, float *gs, const void *in,
     launch_global_scale_atomic(gs, in, M * K, max_scale, st);
     gsrc.slot = -1;
   }
-  QuantGeom g{1, M, K, K, align_up(M, 16), 0, 0, K, 1};
+  QuantGeom g{1, M, K, K, align_up(M, 16), 0, 0, K, 1, 0};
   launch_nvfp4_rowmajor<8>(static_cast<uint8_t *>(out), static_cast<uint8_t *>(sf), static_cast<const uint16_t *>(in),
                            gsrc, g, 1, st, f16out);
   return 0;
@@ -1305,10 +1308,12 @@ static int quantize_rowwise(void *out, float *sf, const void *in, const void *sm
                             int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR, int64_t sK, int swizzle,
                             hipStream_t st, const char *what) {
   if (int rc = check_geom(out, sf, in, smax, d0, d1, R, K, s0, s1, sR, sK)) return rc;
-  QuantGeom g{d1, R, K, align_up(K, 16), align_up(R, 16), s0, s1, sR, sK};
+  QuantGeom g{d1, R, K, align_up(K, 16), align_up(R, 16), s0, s1, sR, sK, 0};
   uint8_t *o = static_cast<uint8_t *>(out);
   const uint16_t *x = static_cast<const uint16_t *>(in);
-  const int64_t lead = d0 * d1;
+  const int64_t lead_all = d0 * d1;
+  for (g.lead0 = 0; g.lead0 < lead_all; g.lead0 += 65535) {
+  const int64_t lead = lead_all - g.lead0 < 65535 ? lead_all - g.lead0 : 65535;
   if (rowmajor_ok(in, K, s0, s1, sR, sK) && K <= 16384) {
     const bool sw = swizzle != 0;
     if (K <= 64)
@@ -1334,25 +1339,28 @@ static int quantize_rowwise(void *out, float *sf, const void *in, const void *sm
     hipLaunchKernelGGL((quantize_rowwise_longrow_kernel<FMT>), grid, dim3(256), 0, st, o, sf, x, smax, g);
   } else if (crossmajor_ok(in, R, s0, s1, sR, sK) && ceil_div(g.Rp, 128) <= 65535 && ceil_div(K, CM_KSPAN) <= 65535) {
     // row maxima as bf16 bit patterns in the scale array, quantize from them, then scale them in place
-    uint32_t *bits = reinterpret_cast<uint32_t *>(sf);
+    uint32_t *bits = reinterpret_cast<uint32_t *>(sf) + g.lead0 * g.Rp;  // the kernels index by absolute lead
     const int64_t nsf = lead * g.Rp;
     hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)ceil_div(nsf, 256)), dim3(256), 0, st, bits, nsf, 0u);
     hipLaunchKernelGGL(rowwise_crossmajor_amax_kernel,
                        dim3((unsigned)ceil_div(K, CM_KSPAN), (unsigned)ceil_div(g.Rp, 128), (unsigned)lead), dim3(256), 0,
-                       st, bits, x, g);
+                       st, reinterpret_cast<uint32_t *>(sf), x, g);
     dim3 grid((unsigned)ceil_div(g.Kp / 16, 16), (unsigned)ceil_div(g.Rp, 128), (unsigned)lead);
     if (swizzle)
-      hipLaunchKernelGGL((quantize_rowwise_crossmajor_kernel<FMT, true>), grid, dim3(256), 0, st, o, bits, x, smax, g);
+      hipLaunchKernelGGL((quantize_rowwise_crossmajor_kernel<FMT, true>), grid, dim3(256), 0, st, o,
+                         reinterpret_cast<const uint32_t *>(sf), x, smax, g);
     else
-      hipLaunchKernelGGL((quantize_rowwise_crossmajor_kernel<FMT, false>), grid, dim3(256), 0, st, o, bits, x, smax, g);
-    hipLaunchKernelGGL(rowwise_crossmajor_finalize_kernel<FMT>, dim3((unsigned)ceil_div(nsf, 256)), dim3(256), 0, st, sf,
-                       smax, nsf);
+      hipLaunchKernelGGL((quantize_rowwise_crossmajor_kernel<FMT, false>), grid, dim3(256), 0, st, o,
+                         reinterpret_cast<const uint32_t *>(sf), x, smax, g);
+    hipLaunchKernelGGL(rowwise_crossmajor_finalize_kernel<FMT>, dim3((unsigned)ceil_div(nsf, 256)), dim3(256), 0, st,
+                       sf + g.lead0 * g.Rp, smax, nsf);
   } else {
     dim3 grid((unsigned)ceil_div(g.Rp, 256), (unsigned)lead);
     if (swizzle)
       hipLaunchKernelGGL((quantize_rowwise_generic_kernel<FMT, true>), grid, dim3(256), 0, st, o, sf, x, smax, g);
     else
       hipLaunchKernelGGL((quantize_rowwise_generic_kernel<FMT, false>), grid, dim3(256), 0, st, o, sf, x, smax, g);
+  }
   }
   return check_launch(what);
 }

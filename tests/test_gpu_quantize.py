@@ -207,6 +207,20 @@ def test_nvfp4_many_streams():
             assert torch.equal(out.cpu(), eo) and torch.equal(sf.cpu().view(torch.uint8), es)
 
 
+def test_many_leading_indices():
+    """More than 65535 (batch-like) leading indices: the launches are issued in slices."""
+    x = make_input((300, 256, 2, 8), seed=8, outliers=True)
+    check_nvfp4(x, 2, 3)
+    check_nvfp4(x, 3, 2, True)
+    for cross, red in ((2, 3), (3, 2)):
+        out, sf = ops().quantize(x.cuda(), cross, red, precision="fp8e4m3")
+        eo, es = T.quantize_fp8(x, cross, red, None, False)
+        assert torch.equal(out.cpu().view(torch.uint8), eo) and torch.equal(sf.cpu(), es)
+        out, sf = ops().quantize(x.cuda(), cross, red, precision="int8")
+        eo, es = T.quantize_int8(x, cross, red)
+        assert torch.equal(out.cpu(), eo) and torch.equal(sf.cpu(), es)
+
+
 def test_nvfp4_caller_buffers_and_negative_dims():
     x = make_input((40, 192), seed=3).cuda()
     out = torch.full((40, 96), 0xAA, dtype=torch.uint8, device="cuda")
