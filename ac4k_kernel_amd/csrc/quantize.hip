@@ -1041,6 +1041,11 @@ namespace ac4k {
 // (device, stream) -> scratch slot.  Slots are handed out on first use and never recycled;
 // when they run out the caller gets -1 and takes the path without scratch.  A call captured into
 // a graph keeps the slot of the stream it was captured on.
+// Calls that enqueue several launches sharing a scratch slot (maxima, then their consumer) hold this
+// lock while they enqueue, so that two host threads feeding the same stream cannot interleave
+// their launches (the stream would then run a consumer against the other call's maxima).
+static std::mutex g_enqueue_mutex;
+
 static int amax_slot(hipStream_t st) {
   static std::mutex mu;
   static struct { int dev; hipStream_t st; } table[AMAX_SLOTS];
@@ -1230,6 +1235,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_global_scale_bf16(flo
   AC4K_REQUIRE(gs && (x || n == 0), "null pointer argument");
   AC4K_REQUIRE(n >= 0, "n must be non-negative");
   AC4K_REQUIRE((reinterpret_cast<uintptr_t>(x) & 1) == 0, "x must be 2-byte aligned");
+  std::lock_guard<std::mutex> lock(g_enqueue_mutex);
   launch_global_scale(gs, x, n, max_scale, (hipStream_t)stream);
   return check_launch("ac4k_global_scale_bf16");
 }
@@ -1249,6 +1255,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_quantize_nvfp4_bf16(v
                                         int64_t sK, int swizzle, float max_scale, ac4k_stream_t stream) {
   if (int rc = check_geom(out, sf, in, global_scale, d0, d1, R, K, s0, s1, sR, sK)) return rc;
   hipStream_t st = (hipStream_t)stream;
+  std::lock_guard<std::mutex> lock(g_enqueue_mutex);
   if (try_quantize_nvfp4_onepass(out, sf, global_scale, in, d0, d1, R, K, s0, s1, sR, sK, swizzle, max_scale, st))
     return check_launch("ac4k_quantize_nvfp4_bf16");
   // pass 1 leaves one maximum per block in the stream's scratch slot; the quantize kernel
@@ -1272,6 +1279,7 @@ namespace ac4k {
 int quantize_activation_with_f16(void *out, void *sf, float *gs, const void *in, int64_t M, int64_t K,
                                  float max_scale, _Float16 *f16out, hipStream_t st) {
   AC4K_REQUIRE(K % 64 == 0 && rowmajor_ok(in, K, 0, 0, K, 1), "activation must be 16-byte aligned with K %% 64 == 0");
+  std::lock_guard<std::mutex> lock(g_enqueue_mutex);
   if (M * (K / 64) <= 128 * SINGLE_WG_MAX_SEGS) {
     const OnePassGeom og{(uint32_t)(M * (K / 64)), (uint32_t)(K / 64), (uint32_t)M, (uint32_t)align_up(M, 16), 1u};
     launch_single_wg<true>(static_cast<uint32_t *>(out), static_cast<uint32_t *>(sf), static_cast<const uint4 *>(in), gs,

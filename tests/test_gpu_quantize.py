@@ -207,6 +207,34 @@ def test_nvfp4_many_streams():
             assert torch.equal(out.cpu(), eo) and torch.equal(sf.cpu().view(torch.uint8), es)
 
 
+def test_nvfp4_host_threads_share_a_stream():
+    """Several host threads quantize on the same stream at once (the C calls run without the GIL):
+    the launches of one call stay together, so every result is exact."""
+    import threading
+    shapes = [(1024, 2048), (300, 640), (4096, 1024), (8192, 8192 // 8)]
+    xs = [make_input(sh, seed=90 + i, outliers=True) for i, sh in enumerate(shapes)]
+    exp = [T.quantize_nvfp4(x, 0, 1, False) for x in xs]
+    dev = [x.cuda() for x in xs]
+    stream = torch.cuda.current_stream()
+    results = [[] for _ in xs]
+
+    def work(i):
+        with torch.cuda.stream(stream):
+            for _ in range(25):
+                results[i].append(ops().quantize(dev[i], 0, 1))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(xs))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    for i, res in enumerate(results):
+        for out, sf, gs in res:
+            assert gs.item() == exp[i][2].item()
+            assert torch.equal(out.cpu(), exp[i][0]) and torch.equal(sf.cpu().view(torch.uint8), exp[i][1])
+
+
 def test_many_leading_indices():
     """More than 65535 (batch-like) leading indices: the launches are issued in slices."""
     x = make_input((300, 256, 2, 8), seed=8, outliers=True)
