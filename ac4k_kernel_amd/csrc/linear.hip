@@ -901,6 +901,22 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
+  } else if (sizeof(typename DE::T) == 4 && (a.N % 4 == 0) && ((uintptr_t)a.D % 16 == 0)) {
+    // fp32 output: a lane holds four consecutive columns, one 16-byte store each
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      const int64_t m = m0 + i * 32 + (lane & 31);
+      if (m >= a.M) continue;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int64_t n = n0 + j * 32 + g * 8 + half * 4;
+          if (n < a.N)
+            *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.D) + m * a.N + n) =
+                make_float4(value(i, j, 4 * g), value(i, j, 4 * g + 1), value(i, j, 4 * g + 2), value(i, j, 4 * g + 3));
+        }
+    }
   } else {
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
@@ -1144,6 +1160,7 @@ struct SkinnyPlan {
 static bool skinny_plan(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
   if (M < 1 || M > 32 || K % SK_STEP != 0 || N < 1) return false;
   int ks = 1024;
+  if (const char *e = getenv("AC4K_SKINNY_KS")) ks = atoi(e);  // tuning aid
   while (ks > SK_STEP && K % ks != 0) ks >>= 1;
   p.groups = ceil_div(N, SK_ROWS);
   // short problems: use smaller slices to get enough workgroups in flight

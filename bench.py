@@ -49,11 +49,25 @@ def make_input(shape, seed=0, outliers=False, std=1.0):
     return x.to(torch.bfloat16)
 
 
+SETTLE_MS = 150.0  # see time_gpu; --settle-ms
+
+
 def time_gpu(fn, steps, warmup):
-    """-> (total ms over `steps` calls, ms per call); events on the launch stream."""
+    """-> (total ms over `steps` calls, ms per call); events on the launch stream.
+
+    `warmup` untimed calls come first.  Then the untimed calls go on until the GPU has been under
+    this load for SETTLE_MS of wall time: the clock governor of the box ramps up over the first
+    40 ms or so of sustained work (the 8192^3 linear goes from 1.2 ms for the first calls to a steady
+    0.77 ms), and a run of a few dozen steps would time the ramp, not the kernel."""
+    import time
+    t0 = time.perf_counter()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    while (time.perf_counter() - t0) * 1e3 < SETTLE_MS:
+        for _ in range(max(1, warmup)):
+            fn()
+        torch.cuda.synchronize()
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(steps):
@@ -237,11 +251,14 @@ def run_traffic(ops):
 
 
 def main():
+    global SETTLE_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all", choices=["all", "linear", "quantize", "traffic"])
+    ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
+                    help="keep the untimed warm-up going for this long (clock ramp); 0 = exactly --warmup calls")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     args = ap.parse_args()
@@ -256,7 +273,9 @@ def main():
         return run_traffic(ops)
     check = not args.no_check
     S, W = args.steps, args.warmup
-    line = {"n_gpus": 1, "steps": S, "warmup": W, "higher_is_better": True, "scaling": "weak",
+    SETTLE_MS = args.settle_ms
+    line = {"n_gpus": 1, "steps": S, "warmup": W, "warmup_settle_ms": SETTLE_MS, "higher_is_better": True,
+            "scaling": "weak",
             "vs_baseline": None, "data": "synthetic (seed 0, generated on CPU, cast to bf16)"}
     quant = None
     if args.workload in ("all", "quantize"):
