@@ -70,10 +70,11 @@ constexpr int BIAS_NONE = 3;
 
 // --- decode -------------------------------------------------------------------
 // E4M3 scale byte -> fp16x2 pattern worth scale * 2^-8 in both halves (exponent bias 7 vs 15;
-// E4M3 subnormals land on fp16 subnormals with the same ratio).  Bit 7 (sign) is dropped: the
-// block scale is unsigned.
+// E4M3 subnormals land on fp16 subnormals with the same ratio).  The scale bytes are read as
+// the signed float8_e4m3fn their tensor type says, by every linear kernel (the quantizers only
+// produce non-negative scales).
 __device__ __forceinline__ f16x2 scale_pattern(uint32_t byte) {
-  return __builtin_bit_cast(f16x2, (byte & 0x7fu) * 0x00800080u);
+  return __builtin_bit_cast(f16x2, (byte & 0x7fu) * 0x00800080u + (byte & 0x80u) * 0x01000100u);
 }
 
 // eight nibbles of `w` times the block scale -> eight fp16 (exact); the converter multiplies
@@ -515,13 +516,13 @@ struct PLayout {               // byte offsets inside one LDS stage
 // that the compiler's wait-count insertion does not see these loads: with the builtin it puts
 // s_waitcnt vmcnt(0) in front of every later LDS read, which serialises the prefetch.  The
 // kernel waits with explicit s_waitcnt vmcnt(..) before the barrier that publishes a stage.
-__device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :: "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+__device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t lds_stage, uint32_t lds_piece) {
+  asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
+               :: "s"(lds_stage), "s"(lds_piece), "v"(voff), "s"(sbase) : "memory", "scc");
 }
-__device__ __forceinline__ void dma4(const void *sbase, uint32_t voff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
-               :: "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+__device__ __forceinline__ void dma4(const void *sbase, uint32_t voff, uint32_t lds_stage, uint32_t lds_piece) {
+  asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3"
+               :: "s"(lds_stage), "s"(lds_piece), "v"(voff), "s"(sbase) : "memory", "scc");
 }
 
 template <int MI>
@@ -649,36 +650,51 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     ldsS[p2] = (uint32_t)__builtin_amdgcn_readfirstlane((isB ? PL::OFF_SFB + c * P_BN * 4 : PL::OFF_SFA + c * BM * 4) + rb * 256);
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)plds;
-  // `kt` may run past the last stage: the source is clamped (re-reading the last slice) and the
-  // destination is a stage buffer nobody reads again, which keeps the main loop free of branches
-  auto issue_piece = [&](int kt_dst, int q) {
-    const uint32_t st = lds_base + (kt_dst % P_STAGES) * PL::STAGE_BYTES;
-    const int kt = kt_dst < nkt ? kt_dst : nkt - 1;
+  // LDS destinations of this wave's transfers inside a stage (wave-uniform, loop invariant)
+  uint32_t ldsA[NDA], ldsB[NDB];
+#pragma unroll
+  for (int q = 0; q < NDA; ++q) ldsA[q] = (uint32_t)__builtin_amdgcn_readfirstlane((swave * NDA + q) * 1024);
+#pragma unroll
+  for (int q = 0; q < NDB; ++q) ldsB[q] = (uint32_t)__builtin_amdgcn_readfirstlane(PL::OFF_B + (swave * NDB + q) * 1024);
+  // Source pointers of the k-step being fetched.  They advance by one step per iteration and stop
+  // at the last step of the range: fetches past the end re-read the last slice into a stage buffer
+  // nobody reads again, which keeps the main loop free of branches.
+  struct Src {
+    const uint8_t *a, *b, *s[NS];
+  };
+  auto src_at = [&](int kt) {
+    Src p;
+    p.a = baseA + (int64_t)kt * P_ROW;
+    p.b = baseB + (int64_t)kt * P_ROW;
+#pragma unroll
+    for (int p2 = 0; p2 < NS; ++p2) p.s[p2] = baseS[p2] + kt * strideS[p2];
+    return p;
+  };
+  auto issue_piece = [&](uint32_t stage_lds, const Src &p, int q) {
     if (q < NDA) {
-      dma16(baseA + (int64_t)kt * P_ROW, offA[q], st + (swave * NDA + q) * 1024);
+      dma16(p.a, offA[q], stage_lds, ldsA[q]);
     } else if (q < NDA + NDB) {
-      const int r = q - NDA;
-      dma16(baseB + (int64_t)kt * P_ROW, offB[r], st + PL::OFF_B + (swave * NDB + r) * 1024);
+      dma16(p.b, offB[q - NDA], stage_lds, ldsB[q - NDA]);
     } else {
       const int p2 = q - NDA - NDB;
-      dma4(baseS[p2] + kt * strideS[p2], offS[p2], st + ldsS[p2]);
+      dma4(p.s[p2], offS[p2], stage_lds, ldsS[p2]);
     }
   };
-  auto issue_stage = [&](int kt) {
+  auto issue_stage = [&](uint32_t stage_lds, const Src &p) {
 #pragma unroll
-    for (int q = 0; q < NPIECES; ++q) issue_piece(kt, q);
+    for (int q = 0; q < NPIECES; ++q) issue_piece(stage_lds, p, q);
   };
-  // pieces of stage kt+2 issued in quarter `qr` (0..3) of the second half of a step
-  auto issue_quarter = [&](int kt_dst, int qr) {
+  // pieces issued in quarter `qr` (0..3) of the second half of a step
+  auto issue_quarter = [&](uint32_t stage_lds, const Src &p, int qr) {
 #pragma unroll
     for (int q = 0; q < NDA; ++q)
-      if (q * 4 / NDA == qr) issue_piece(kt_dst, q);
+      if (q * 4 / NDA == qr) issue_piece(stage_lds, p, q);
 #pragma unroll
     for (int q = 0; q < NDB; ++q)
-      if (q * 4 / NDB == qr) issue_piece(kt_dst, NDA + q);
+      if (q * 4 / NDB == qr) issue_piece(stage_lds, p, NDA + q);
 #pragma unroll
     for (int q = 0; q < NS; ++q)
-      if (q * 4 / NS == qr) issue_piece(kt_dst, NDA + NDB + q);
+      if (q * 4 / NS == qr) issue_piece(stage_lds, p, NDA + NDB + q);
   };
 
   f32x16 acc[MI][4];
@@ -692,14 +708,14 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   // fragment addresses inside a stage (bytes)
   const int fa_off = (wm * (32 * MI) + (lane & 31)) * P_ROW + half * 16;
   const int fb_off = PL::OFF_B + (wn * 128 + (lane & 31)) * P_ROW + half * 16;
-  const int sa_off = PL::OFF_SFA + (wm * (32 * MI) + (lane & 31)) * 4;
-  const int sb_off = PL::OFF_SFB + (wn * 128 + (lane & 31)) * 4;
-  const int sh = half * 16;  // a lane needs the two scale bytes of its half of the chunk
+  // a lane needs the two scale bytes of its half of the chunk: blocks 2*half, 2*half+1
+  const int sa_off = PL::OFF_SFA + (wm * (32 * MI) + (lane & 31)) * 4 + half * 2;
+  const int sb_off = PL::OFF_SFB + (wn * 128 + (lane & 31)) * 4 + half * 2;
 
   uint4 PA[2][MI], PB[2][4];  // packed fragments of a 64-chunk, double buffered by chunk parity
   f16x2 SA[2][MI], SB[2][4];  // their two block scales (blocks 2*half, 2*half+1) as fp16
-  auto load_chunk = [&](int kt, int c) {
-    const char *st = plds + (kt % P_STAGES) * PL::STAGE_BYTES;
+  auto load_chunk = [&](uint32_t stage_off, int c) {
+    const char *st = plds + stage_off;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if (i < MI) PA[c][i] = *reinterpret_cast<const uint4 *>(st + fa_off + c * 32 + i * 32 * P_ROW);
@@ -708,11 +724,11 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if (i < MI) {
-        uint32_t wa = *reinterpret_cast<const uint32_t *>(st + sa_off + c * (BM * 4) + i * 128);
-        SA[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((wa >> sh) & 0x7f7fu, 1.0f, false);  // scales are unsigned e4m3
+        const uint32_t wa = *reinterpret_cast<const uint16_t *>(st + sa_off + c * (BM * 4) + i * 128);
+        SA[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wa, 1.0f, false);
       }
-      uint32_t wb = *reinterpret_cast<const uint32_t *>(st + sb_off + c * (P_BN * 4) + i * 128);
-      SB[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((wb >> sh) & 0x7f7fu, 1.0f, false);
+      const uint32_t wb = *reinterpret_cast<const uint16_t *>(st + sb_off + c * (P_BN * 4) + i * 128);
+      SB[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wb, 1.0f, false);
     }
   };
 
@@ -754,8 +770,9 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   using I3 = std::integral_constant<int, 3>;
 
   // prologue: stages 0 and 1 in flight, stage 0 visible, chunk 0 fragments and first decode
-  issue_stage(0);
-  if (nkt > 1) issue_stage(1);
+  const int last = nkt - 1;
+  issue_stage(lds_base, src_at(0));
+  if (nkt > 1) issue_stage(lds_base + PL::STAGE_BYTES, src_at(1));
   if (nkt > 1) {
     static_assert(NPIECES == 12 || NPIECES == 9, "wait count below is spelled out per variant");
     if constexpr (NPIECES == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
@@ -767,13 +784,17 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   load_chunk(0, 0);
   decode(D[0], 0, I0{});
 
+  // loop-carried, wave-uniform: LDS offsets of the stages holding k-steps kt, kt+1 and of the one
+  // being filled with kt+2 (rotating), and the source pointers of k-step min(kt+2, last)
+  uint32_t st_cur = 0, st_nxt = PL::STAGE_BYTES, st_dma = 2 * PL::STAGE_BYTES;
+  Src src = src_at(last < 2 ? last : 2);
 #ifdef AC4K_LINEAR_TIMELINE
   const uint64_t tl_c0 = __builtin_readcyclecounter();
 #endif
   AC4K_LTL(1, wall_clock64());
   for (int kt = 0; kt < nkt; ++kt) {
     // chunk 0: sub-steps 0..3 (fragments of chunk 1 are fetched meanwhile)
-    load_chunk(kt, 1);
+    load_chunk(st_cur, 1);
     decode(D[1], 0, I1{});
     mfma16(D[0]);
     interleave();
@@ -791,23 +812,34 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     __syncthreads();
     // chunk 1: sub-steps 4..7 (chunk 0 of the next stage is fetched meanwhile); the DMA of stage
     // kt+2 is spread over these sub-steps
+    const uint32_t dma_lds = lds_base + st_dma;
     decode(D[1], 1, I1{});
-    issue_quarter(kt + 2, 0);
+    issue_quarter(dma_lds, src, 0);
     mfma16(D[0]);
     interleave();
-    load_chunk(kt + 1, 0);  // past the end this reads a stale stage; the result is never used
+    load_chunk(st_nxt, 0);  // past the end this reads a stale stage; the result is never used
     decode(D[0], 1, I2{});
-    issue_quarter(kt + 2, 1);
+    issue_quarter(dma_lds, src, 1);
     mfma16(D[1]);
     interleave();
     decode(D[1], 1, I3{});
-    issue_quarter(kt + 2, 2);
+    issue_quarter(dma_lds, src, 2);
     mfma16(D[0]);
     interleave();
     decode(D[0], 0, I0{});  // first sub-step of the next stage (unused after the last step)
-    issue_quarter(kt + 2, 3);
+    issue_quarter(dma_lds, src, 3);
     mfma16(D[1]);
     interleave();
+    // rotate the stages; advance the sources unless they already sit on the last k-step
+    const uint32_t freed = st_cur;
+    st_cur = st_nxt;
+    st_nxt = st_dma;
+    st_dma = freed;
+    const bool adv = kt + 3 <= last;
+    src.a += adv ? P_ROW : 0;
+    src.b += adv ? P_ROW : 0;
+#pragma unroll
+    for (int p2 = 0; p2 < NS; ++p2) src.s[p2] += adv ? strideS[p2] : 0;
   }
   AC4K_LTL(2, wall_clock64());
 #ifdef AC4K_LINEAR_TIMELINE
@@ -1068,8 +1100,8 @@ __global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) 
       f16x2 sc[2][2];  // [chunk][block pair] -> scales of blocks (0,1) and (2,3) of each 64-chunk
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
-        sc[c][0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(S[t][c] & 0x7f7f7f7fu, 1.0f, false);
-        sc[c][1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(S[t][c] & 0x7f7f7f7fu, 1.0f, true);
+        sc[c][0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(S[t][c], 1.0f, false);
+        sc[c][1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(S[t][c], 1.0f, true);
       }
 #pragma unroll
       for (int q = 0; q < 4; ++q) {       // 16-byte word q: elements [32q, 32q+32) of the lane's 128
@@ -1145,7 +1177,7 @@ __global__ __launch_bounds__(256) void decode_activation_kernel(_Float16 *__rest
   if (i >= M * (K >> 3)) return;
   const int64_t m = i / (K >> 3), k = (i % (K >> 3)) * 8;
   const uint32_t w = *reinterpret_cast<const uint32_t *>(A + m * (K >> 1) + (k >> 1));
-  const uint32_t code = A_sf[(((k >> 6) * Mp + m) << 2) + ((k >> 4) & 3)] & 0x7fu;
+  const uint32_t code = A_sf[(((k >> 6) * Mp + m) << 2) + ((k >> 4) & 3)];
   const f16x2 sc2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(code, 1.0f, false);
   const f16x8 d = decode_dword<false>(w, sc2);
   *reinterpret_cast<f16x8 *>(ahat + m * K + k) = d;
