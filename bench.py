@@ -135,18 +135,22 @@ def bench_quantize(ops, shape, precision, steps, warmup, outliers, check=True, n
             "roofline": roofline("hbm", gbs, key), "rotating_buffers": nbuf}
 
 
-def cpu_quantize_baseline(shape, outliers):
+def cpu_quantize_baseline(shape, outliers, budget_s=10.0):
+    """The torch oracle on the host cores: whole quantizes of one tensor, repeated for about
+    `budget_s` seconds (at least three), median time."""
     from oracle import nvfp4_oracle as T
     x = make_input(shape, seed=0, outliers=outliers)
     T.quantize_nvfp4(x[:256], 0, 1)
-    ts = []
-    for _ in range(3):
+    ts, t_begin = [], time.perf_counter()
+    while len(ts) < 3 or time.perf_counter() - t_begin < budget_s:
         t0 = time.perf_counter()
         T.quantize_nvfp4(x, 0, 1)
         ts.append(time.perf_counter() - t0)
-    t = sorted(ts)[1]
+    t = sorted(ts)[len(ts) // 2]
     return {"value": quant_bytes(shape, "nvfp4") / t / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
-            "kind": "port", "sample": f"full nvfp4 quantize of one {shape[0]}x{shape[1]} bf16 tensor, median of 3"}
+            "kind": "port",
+            "sample": f"full nvfp4 quantize of one {shape[0]}x{shape[1]} bf16 tensor, median of {len(ts)} runs "
+                      f"({time.perf_counter() - t_begin:.0f} s)"}
 
 
 # --------------------------------------------------------------------------- linear
@@ -217,8 +221,9 @@ def bench_decode(ops, m, n, k, steps, warmup, check=True):
             "roofline": roofline("hbm", gbs)}
 
 
-def cpu_linear_baseline(n, k, rows=256):
-    """fp32 dequantize-then-matmul of the oracle on `rows` rows of the 8192^3 problem."""
+def cpu_linear_baseline(n, k, rows=4096):
+    """fp32 dequantize-then-matmul of the oracle on `rows` rows of the 8192^3 problem (the weight
+    operand in full): about ten seconds of host work."""
     from oracle import nvfp4_oracle as T
     a, b = make_input((rows, k), seed=0), make_input((n, k), seed=1)
     aq, bq = T.quantize_nvfp4(a, 0, 1), T.quantize_nvfp4(b, 0, 1)
@@ -227,7 +232,8 @@ def cpu_linear_baseline(n, k, rows=256):
     t = time.perf_counter() - t0
     return {"value": 2.0 * rows * n * k / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
             "kind": "port",
-            "sample": f"oracle fp32 dequantize + torch.matmul of M={rows} rows of the N={n} K={k} problem, 1 run"}
+            "sample": f"oracle fp32 dequantize + torch.matmul of M={rows} rows of the N={n} K={k} problem, "
+                      f"1 run ({t:.1f} s)"}
 
 
 def run_traffic(ops):
@@ -289,7 +295,7 @@ def main():
             log(f"[bench] {k_}: {v['ms'] * 1e3:.1f} us  {v['GB/s']:.0f} GB/s  "
                 f"({100 * v['roofline']['frac']:.1f}% of HBM peak)  bit-exact={v['bit_exact_vs_oracle']}")
         if not args.no_cpu_baseline:
-            quant["cpu_baseline"] = cpu_quantize_baseline((4096, 4096), False)
+            quant["cpu_baseline"] = cpu_quantize_baseline((8192, 4096), True)
             log(f"[bench] cpu quantize oracle: {quant['cpu_baseline']['value']:.2f} GB/s on "
                 f"{quant['cpu_baseline']['cores']} threads")
     if args.workload in ("all", "linear"):
