@@ -110,6 +110,28 @@ def test_large_shapes(m, n, k, wstd):
     torch.testing.assert_close(d, full, atol=ATOL, rtol=RTOL)
 
 
+@pytest.mark.parametrize("m,n,k", [(4096, 4096, 4096), (128, 4096, 14336), (8, 28672, 8192), (2048, 4096, 14336)])
+def test_size_independent_properties(m, n, k):
+    """At full BASELINE sizes, with fp32 output so that nothing is rounded after the accumulation:
+    (1) the result is linear in the global scale, bit for bit for a power of two;
+    (2) an output row depends only on its own activation row: permuting the rows of the packed
+        activation (and of its scales) permutes the output rows, bit for bit, wherever the rows land
+        in the tiling."""
+    aq = gpu_quant(make_input((m, k), seed=4))
+    bq = gpu_quant(make_input((n, k), seed=5, std=0.02))
+    d1 = ops().linear(*aq, *bq, out=torch.empty((m, n), dtype=torch.float32, device="cuda"))
+    d2 = ops().linear(aq[0], aq[1], aq[2] * 4.0, *bq, out=torch.empty((m, n), dtype=torch.float32, device="cuda"))
+    assert torch.equal(d2, d1 * 4.0)
+    perm = torch.randperm(m, generator=torch.Generator().manual_seed(m)).cuda()
+    mp = aq[1].shape[1]
+    sf_perm = aq[1].clone()
+    sf_perm[:, :m] = aq[1][:, perm]
+    assert mp >= m
+    d3 = ops().linear(aq[0][perm].contiguous(), sf_perm, aq[2], *bq,
+                      out=torch.empty((m, n), dtype=torch.float32, device="cuda"))
+    assert torch.equal(d3, d1[perm])
+
+
 @pytest.mark.parametrize("m", [1, 8, 32])
 def test_fused_skinny_equals_composition(m):
     n, k = 1024, 2048
