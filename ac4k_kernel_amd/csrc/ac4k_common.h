@@ -14,10 +14,6 @@ namespace ac4k {
 int set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 int check_launch(const char *what);  // hipGetLastError() -> status
 
-// quantize.hip: nvfp4-quantize a contiguous activation and also emit its fp16 dequantization
-int quantize_activation_with_f16(void *out, void *sf, float *gs, const void *in, int64_t M, int64_t K,
-                                 float max_scale, _Float16 *f16out, hipStream_t st);
-
 #define AC4K_REQUIRE(cond, ...)                      \
   do {                                               \
     if (!(cond)) return ::ac4k::set_error(__VA_ARGS__); \

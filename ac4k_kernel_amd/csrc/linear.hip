@@ -13,6 +13,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "ac4k_common.h"
@@ -965,17 +966,26 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   AC4K_LTL(3, wall_clock64());
 }
 
+// Raises a kernel's dynamic LDS limit once per (kernel instantiation, device): the attribute belongs
+// to the device the call is made on.
+template <typename Kernel>
+static int allow_dynamic_lds(Kernel *kern, std::atomic<uint32_t> &done_mask, int bytes) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  const uint32_t bit = 1u << (dev & 31);
+  if (done_mask.load(std::memory_order_relaxed) & bit) return 0;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return set_error("hipFuncSetAttribute(LDS=%d): %s", bytes, hipGetErrorString(e));
+  done_mask.fetch_or(bit, std::memory_order_relaxed);
+  return 0;
+}
+
 template <int D_DT, int BIAS_DT, int MI>
 static int launch_tile256p_mi(const LinearArgs &a, const SplitK &sk, hipStream_t st) {
   auto *kern = linear_nvfp4_tile256p_kernel<D_DT, BIAS_DT, MI>;
   using PL = PLayout<64 * MI>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, PL::LDS_BYTES);
-    if (e != hipSuccess) return set_error("hipFuncSetAttribute(LDS=%d): %s", PL::LDS_BYTES, hipGetErrorString(e));
-    attr_set = true;
-  }
+  static std::atomic<uint32_t> lds_ok{0};
+  if (int rc = allow_dynamic_lds(kern, lds_ok, PL::LDS_BYTES)) return rc;
   const int64_t ntiles = ceil_div(a.M, 64 * MI) * ceil_div(a.N, P_BN);
   hipLaunchKernelGGL(kern, dim3((unsigned)ntiles, (unsigned)sk.splits), dim3(256), PL::LDS_BYTES, st, a, sk);
   return 0;
@@ -1006,13 +1016,8 @@ static LinearKernel forced_kernel() {  // benchmarking aid: AC4K_LINEAR_KERNEL=t
 template <int D_DT, int BIAS_DT>
 static int launch_tile256(const LinearArgs &a, hipStream_t st) {
   auto *kern = linear_nvfp4_tile256_kernel<D_DT, BIAS_DT>;
-  static bool attr_set = false;  // per instantiation; the attribute is idempotent
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, L_LDS_BYTES);
-    if (e != hipSuccess) return set_error("hipFuncSetAttribute(LDS=%d): %s", L_LDS_BYTES, hipGetErrorString(e));
-    attr_set = true;
-  }
+  static std::atomic<uint32_t> lds_ok{0};
+  if (int rc = allow_dynamic_lds(kern, lds_ok, L_LDS_BYTES)) return rc;
   const int64_t ntiles = ceil_div(a.M, L_BM) * ceil_div(a.N, L_BN);
   hipLaunchKernelGGL(kern, dim3((unsigned)ntiles), dim3(256), L_LDS_BYTES, st, a);
   return 0;
@@ -1021,11 +1026,11 @@ static int launch_tile256(const LinearArgs &a, hipStream_t st) {
 // ===========================================================================
 // Decode-sized linear (1 <= M <= 32): bound by streaming the weights once.
 //
-// The activation arrives as its exact fp16 dequantization Ahat [M, K] (without the global
-// scale).  A workgroup (4 waves) owns 128 weight rows and one K-slice; every wave one 32-row
-// tile.  Lane (row r, half h) streams 64 contiguous bytes of its weight row per 256-k step
+// A workgroup (4 waves) owns 128 weight rows and one K-slice; every wave one 32-row tile.  It
+// first decodes its slice of the packed activation to fp16 (exact, without the global scale)
+// into LDS, shared by the four waves.  Lane (row r, half h) streams 64 contiguous bytes of its weight row per 256-k step
 // (elements [128h, 128h+128) of the step) and decodes them dword by dword into MFMA operands;
-// the activation slice sits in LDS (shared by the four waves).  The MFMA is issued as
+// The MFMA is issued as
 // D^T = W . Ahat^T so a lane ends up with 4 consecutive n for one m.  K-slices of one row
 // group meet through fp32 partial tiles in a caller-provided workspace; a small second kernel
 // adds them in slice order (deterministic), applies gsA*gsB and the bias, converts and stores.
@@ -1035,7 +1040,9 @@ static int launch_tile256(const LinearArgs &a, hipStream_t st) {
 // ===========================================================================
 struct SkinnyArgs {
   void *D;
-  const _Float16 *Ahat;
+  const uint8_t *Aq;         // packed activation [M, K/2] and its scale bytes [K/64, Mp, 4]
+  const uint8_t *A_sf;
+  int64_t Mp;
   const uint8_t *B;
   const uint32_t *B_sf;
   const float *A_gs, *B_gs;
@@ -1077,14 +1084,17 @@ __global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) 
       S[t][1] = sp[(int64_t)(t * 4 + 1) * a.Np];
     }
   }
-  // activation slice -> LDS
+  // activation slice -> LDS as its exact fp16 dequantization (without the global scale)
   {
-    const int vec_per_row = a.ks_len / 8;  // 16-byte vectors per row
+    const int vec_per_row = a.ks_len / 8;  // 16-byte vectors (8 elements) per row
     const int total = (int)a.M * vec_per_row;
     for (int i = tid; i < total; i += 256) {
       const int m = i / vec_per_row, v = i % vec_per_row;
-      *reinterpret_cast<uint4 *>(slds + m * pitch + v * 16) =
-          *reinterpret_cast<const uint4 *>(a.Ahat + (int64_t)m * a.K + kbeg + v * 8);
+      const int64_t k = kbeg + v * 8;
+      const uint32_t w = *reinterpret_cast<const uint32_t *>(a.Aq + (int64_t)m * (a.K >> 1) + (k >> 1));
+      const uint32_t code = a.A_sf[(((k >> 6) * a.Mp + m) << 2) + ((k >> 4) & 3)];
+      const f16x8 d = decode_dword<false>(w, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(code, 1.0f, false));
+      *reinterpret_cast<f16x8 *>(slds + m * pitch + v * 16) = d;
     }
   }
   __syncthreads();
@@ -1168,24 +1178,9 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(SkinnyArgs a) {
   static_cast<typename Elem<D_DT>::T *>(a.D)[i] = Elem<D_DT>::cvt(v);
 }
 
-// packed activation -> exact fp16 dequantization (without the global scale), one dword per thread
-__global__ __launch_bounds__(256) void decode_activation_kernel(_Float16 *__restrict__ ahat,
-                                                                const uint8_t *__restrict__ A,
-                                                                const uint8_t *__restrict__ A_sf, int64_t M, int64_t K,
-                                                                int64_t Mp) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // dword index
-  if (i >= M * (K >> 3)) return;
-  const int64_t m = i / (K >> 3), k = (i % (K >> 3)) * 8;
-  const uint32_t w = *reinterpret_cast<const uint32_t *>(A + m * (K >> 1) + (k >> 1));
-  const uint32_t code = A_sf[(((k >> 6) * Mp + m) << 2) + ((k >> 4) & 3)];
-  const f16x2 sc2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(code, 1.0f, false);
-  const f16x8 d = decode_dword<false>(w, sc2);
-  *reinterpret_cast<f16x8 *>(ahat + m * K + k) = d;
-}
-
 struct SkinnyPlan {
   int ks_len, split_k;
-  int64_t ahat_bytes, partial_bytes, groups;
+  int64_t partial_bytes, groups;
   int lds_bytes;
 };
 
@@ -1199,7 +1194,6 @@ static bool skinny_plan(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
   while (ks > SK_STEP && p.groups * (K / ks) < 768) ks >>= 1;
   p.ks_len = ks;
   p.split_k = (int)(K / ks);
-  p.ahat_bytes = align_up(M * K * 2, 256);
   p.partial_bytes = p.split_k > 1 ? (int64_t)p.split_k * M * N * 4 : 0;
   p.lds_bytes = (int)M * (ks * 2 + 16);
   return true;
@@ -1208,13 +1202,8 @@ static bool skinny_plan(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
 template <int D_DT, int BIAS_DT>
 static int launch_skinny(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_t st) {
   auto *kern = linear_nvfp4_skinny_kernel<D_DT, BIAS_DT>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 32 * (1024 * 2 + 16));
-    if (e != hipSuccess) return set_error("hipFuncSetAttribute: %s", hipGetErrorString(e));
-    attr_set = true;
-  }
+  static std::atomic<uint32_t> lds_ok{0};
+  if (int rc = allow_dynamic_lds(kern, lds_ok, 32 * (1024 * 2 + 16))) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)p.split_k, (unsigned)p.groups), dim3(256), p.lds_bytes, st, a);
   if (p.split_k > 1)
     hipLaunchKernelGGL((skinny_reduce_kernel<D_DT, BIAS_DT>), dim3((unsigned)ceil_div(a.M * a.N, 256)), dim3(256), 0, st, a);
@@ -1359,7 +1348,7 @@ static int launch_mid(const LinearArgs &a, const MidPlan &p, float *partial, hip
   const SplitK sk{partial, p.splits};
   const int rc = a.M <= 128 ? launch_tile256p_mi<D_DT, BIAS_DT, 2>(a, sk, st) : launch_tile256p_mi<D_DT, BIAS_DT, 4>(a, sk, st);
   if (rc) return rc;
-  SkinnyArgs r{a.D, nullptr, nullptr, nullptr, a.A_gs, a.B_gs, a.bias, partial, a.M, a.N, a.K, a.Np, 0, p.splits};
+  SkinnyArgs r{a.D, nullptr, nullptr, 0, nullptr, nullptr, a.A_gs, a.B_gs, a.bias, partial, a.M, a.N, a.K, a.Np, 0, p.splits};
   hipLaunchKernelGGL((skinny_reduce_kernel<D_DT, BIAS_DT>), dim3((unsigned)ceil_div(a.M * a.N, 256)), dim3(256), 0, st, r);
   return 0;
 }
@@ -1385,18 +1374,20 @@ static int dispatch_mid(const LinearArgs &a, const MidPlan &p, float *partial, i
   return set_error("d must be bfloat16, half or float (dtype tag %d)", d_dtype);
 }
 
-// shared tail of the two decode-sized entry points: Ahat is in the workspace already
-static int run_skinny(void *D, int d_dtype, const float *A_gs, const void *B, const void *B_sf, const float *B_gs,
-                      const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, const SkinnyPlan &p,
-                      void *workspace, hipStream_t st) {
+// shared tail of the two decode-sized entry points: packed activation in, partial sums in the workspace
+static int run_skinny(void *D, int d_dtype, const void *Aq, const void *A_sf, const float *A_gs, const void *B,
+                      const void *B_sf, const float *B_gs, const void *bias, int bias_dtype, int64_t M, int64_t N,
+                      int64_t K, const SkinnyPlan &p, void *workspace, hipStream_t st) {
   SkinnyArgs a{D,
-               static_cast<const _Float16 *>(workspace),
+               static_cast<const uint8_t *>(Aq),
+               static_cast<const uint8_t *>(A_sf),
+               align_up(M, 16),
                static_cast<const uint8_t *>(B),
                static_cast<const uint32_t *>(B_sf),
                A_gs,
                B_gs,
                bias,
-               reinterpret_cast<float *>(static_cast<char *>(workspace) + p.ahat_bytes),
+               static_cast<float *>(workspace),
                M,
                N,
                K,
@@ -1410,8 +1401,7 @@ static int check_skinny(const SkinnyPlan &p, bool ok, const void *B, void *works
   AC4K_REQUIRE(ok, "no workspace-assisted path for this shape (ac4k_linear_nvfp4_skinny_workspace_bytes returns 0)");
   AC4K_REQUIRE(((uintptr_t)B & 15) == 0, "weights must be 16-byte aligned");
   AC4K_REQUIRE(workspace && ((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
-  AC4K_REQUIRE(workspace_bytes >= p.ahat_bytes + p.partial_bytes, "workspace too small: %lld bytes needed",
-               (long long)(p.ahat_bytes + p.partial_bytes));
+  AC4K_REQUIRE(workspace_bytes >= p.partial_bytes, "workspace too small: %lld bytes needed", (long long)p.partial_bytes);
   return 0;
 }
 
@@ -1419,7 +1409,7 @@ static int check_skinny(const SkinnyPlan &p, bool ok, const void *B, void *works
 
 extern "C" __attribute__((visibility("default"))) int64_t ac4k_linear_nvfp4_skinny_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   SkinnyPlan p;
-  if (skinny_plan(M, N, K, p)) return p.ahat_bytes + p.partial_bytes;
+  if (skinny_plan(M, N, K, p)) return p.partial_bytes > 0 ? p.partial_bytes : 256;  // non-zero selects this path
   MidPlan mp;
   if (mid_plan(M, N, K, mp)) return mp.partial_bytes;
   return 0;
@@ -1446,11 +1436,8 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_skinny(v
   SkinnyPlan p;
   const bool ok = skinny_plan(M, N, K, p);
   if (int rc = check_skinny(p, ok, B, workspace, workspace_bytes)) return rc;
-  const int64_t dwords = M * (K >> 3);
-  hipLaunchKernelGGL(decode_activation_kernel, dim3((unsigned)ceil_div(dwords, 256)), dim3(256), 0, st,
-                     static_cast<_Float16 *>(workspace), static_cast<const uint8_t *>(A),
-                     static_cast<const uint8_t *>(A_sf), M, K, align_up(M, 16));
-  if (int rc = run_skinny(D, d_dtype, A_gs, B, B_sf, B_gs, bias, bias_dtype, M, N, K, p, workspace, st))
+  AC4K_REQUIRE(((uintptr_t)A & 3) == 0, "A must be 4-byte aligned");
+  if (int rc = run_skinny(D, d_dtype, A, A_sf, A_gs, B, B_sf, B_gs, bias, bias_dtype, M, N, K, p, workspace, st))
     return rc;
   return check_launch("ac4k_linear_nvfp4_skinny");
 }
@@ -1465,9 +1452,10 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_fused_bf
   const bool ok = skinny_plan(M, N, K, p);
   if (int rc = check_skinny(p, ok, B, workspace, workspace_bytes)) return rc;
   hipStream_t st = (hipStream_t)stream;
-  if (int rc = quantize_activation_with_f16(X_q, X_sf, X_gs, X, M, K, 2688.0f, static_cast<_Float16 *>(workspace), st))
-    return rc;
-  if (int rc = run_skinny(D, d_dtype, X_gs, B, B_sf, B_gs, bias, bias_dtype, M, N, K, p, workspace, st))
+  AC4K_REQUIRE(K % 64 == 0 && ((uintptr_t)X & 15) == 0, "activation must be 16-byte aligned with K %% 64 == 0");
+  if (int rc = ac4k_quantize_nvfp4_bf16(X_q, X_sf, X_gs, X, 1, 1, M, K, 0, 0, K, 1, 0, 2688.0f, stream)) return rc;
+  if (int rc = run_skinny(D, d_dtype, X_q, X_sf, X_gs, B, B_sf, B_gs, bias, bias_dtype, M, N, K, p, workspace,
+                          st))
     return rc;
   return check_launch("ac4k_linear_nvfp4_fused_bf16");
 }

@@ -224,12 +224,10 @@ __device__ __forceinline__ uint4 swizzle_fp8_pair(uint4 v, int lane) {
 // chunk's first lane with three DPP row shifts and stored as one dword.
 //   CPR  = 64-element chunks per wave row (8*CPR lanes per row, 8/CPR rows per wave pass)
 //   ITER = wave passes per workgroup (independent loads in flight per lane)
-//   EMIT = also write the dequantized block values e2m1 * fp32(sf) as fp16 (exact) to `f16out`
-//          [rows, K] (2-D inputs only): the decode-sized linear consumes them directly
-template <int CPR, int ITER, bool EMIT, bool SWIZZLE>
+template <int CPR, int ITER, bool SWIZZLE>
 __global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
     uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in, GlobalScaleSrc gsrc,
-    QuantGeom g, _Float16 *__restrict__ f16out) {
+    QuantGeom g) {
   __shared__ float lut[128];
   load_rcp_table(lut);
   const float alpha = load_alpha(gsrc, blockIdx.x == 0 && blockIdx.y == 0);
@@ -268,19 +266,6 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
       st_stream_u1(out + (lead * g.R + r) * (g.Kp / 2) + k / 2, packed);
     if ((lane & 7) == 0 && r < g.Rp)
       reinterpret_cast<uint32_t *>(sf)[(lead * (g.Kp / 64) + k / 64) * g.Rp + r] = sfw;
-    if constexpr (EMIT) {
-      if (r < g.R) {
-        const f16x2 sc2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(code, 1.0f, false);
-        const f16x2 sc = {sc2.x, sc2.x};
-        f16x2 d0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 0) * sc;
-        f16x2 d1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 1) * sc;
-        f16x2 d2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 2) * sc;
-        f16x2 d3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 3) * sc;
-        *reinterpret_cast<uint4 *>(f16out + r * g.Kp + k) =
-            make_uint4(__builtin_bit_cast(uint32_t, d0), __builtin_bit_cast(uint32_t, d1),
-                       __builtin_bit_cast(uint32_t, d2), __builtin_bit_cast(uint32_t, d3));
-      }
-    }
   }
 }
 
@@ -569,12 +554,11 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
 // ---------------------------------------------------------------------------
 // Tiny dense tensors (at most NV * 1024 vectors of 8 elements): one workgroup holds everything in
 // registers, so global scale and quantize are one launch with an ordinary
-// workgroup barrier in between.  EMIT also writes the dequantized block values e2m1 * fp32(sf) as
-// fp16 (exact) to f16out [rows, K] for the decode-sized linear.
-template <int NV, bool EMIT>
+// workgroup barrier in between.
+template <int NV>
 __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_single_wg_kernel(
     uint32_t *__restrict__ out, uint32_t *__restrict__ sf, const uint4 *__restrict__ in, float *__restrict__ gs_out,
-    OnePassGeom g, float max_scale, _Float16 *__restrict__ f16out) {
+    OnePassGeom g, float max_scale) {
   __shared__ float lut[128];
   __shared__ uint32_t red[OP_THREADS / 64];
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -615,17 +599,6 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_single_wg_kernel(
         const uint32_t ch = lv >> 3, row = ch / g.ncc, cc = ch - row * g.ncc;
         const uint32_t l = g.lead > 1 ? row / g.R : 0u, r = row - l * g.R;
         sf[((uint64_t)l * g.ncc + cc) * g.Rp + r] = sfw;
-      }
-      if constexpr (EMIT) {
-        const f16x2 sc2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(code, 1.0f, false);
-        const f16x2 sc = {sc2.x, sc2.x};
-        const f16x2 d0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 0) * sc;
-        const f16x2 d1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 1) * sc;
-        const f16x2 d2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 2) * sc;
-        const f16x2 d3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 3) * sc;
-        reinterpret_cast<uint4 *>(f16out)[lv] =
-            make_uint4(__builtin_bit_cast(uint32_t, d0), __builtin_bit_cast(uint32_t, d1),
-                       __builtin_bit_cast(uint32_t, d2), __builtin_bit_cast(uint32_t, d3));
       }
     }
   }
@@ -1016,20 +989,14 @@ static bool crossmajor_ok(const void *in, int64_t R, int64_t s0, int64_t s1, int
 
 template <int CPR>
 static void launch_nvfp4_rowmajor(uint8_t *out, uint8_t *sf, const uint16_t *in, const GlobalScaleSrc &gs,
-                                  const QuantGeom &g, int64_t lead, hipStream_t st, _Float16 *f16out = nullptr,
-                                  bool swizzle = false) {
+                                  const QuantGeom &g, int64_t lead, hipStream_t st, bool swizzle) {
   constexpr int ITER = 4;
   constexpr int ROWS = 4 * (8 / CPR) * ITER;
   dim3 grid((unsigned)(ceil_div(g.Kp / 64, CPR) * ceil_div(g.Rp, ROWS)), (unsigned)lead);
-  if (f16out)
-    hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER, true, false>), grid, dim3(256), 0, st, out, sf, in, gs,
-                       g, f16out);
-  else if (swizzle)
-    hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER, false, true>), grid, dim3(256), 0, st, out, sf, in, gs,
-                       g, f16out);
+  if (swizzle)
+    hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER, true>), grid, dim3(256), 0, st, out, sf, in, gs, g);
   else
-    hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER, false, false>), grid, dim3(256), 0, st, out, sf, in,
-                       gs, g, f16out);
+    hipLaunchKernelGGL((quantize_nvfp4_rowmajor_kernel<CPR, ITER, false>), grid, dim3(256), 0, st, out, sf, in, gs, g);
 }
 
 }  // namespace ac4k
@@ -1137,19 +1104,13 @@ static void launch_onepass(uint32_t *out, uint32_t *sf, const uint4 *in, float *
 // 16 KB segments the two-launch paths are faster.
 constexpr int SINGLE_WG_MAX_SEGS = 2;
 
-template <bool EMIT>
 static void launch_single_wg(uint32_t *out, uint32_t *sf, const uint4 *in, float *gs, const OnePassGeom &g,
-                             float max_scale, _Float16 *f16out, hipStream_t st) {
-  const int64_t segs = ceil_div((int64_t)g.total_chunks, 128);  // 1024-vector segments
-#define AC4K_SINGLE_WG(NV)                                                                                       \
-  hipLaunchKernelGGL((quantize_nvfp4_single_wg_kernel<NV, EMIT>), dim3(1), dim3(OP_THREADS), 0, st, out, sf, in, \
-                     gs, g, max_scale, f16out)
+                             float max_scale, hipStream_t st) {
   static_assert(SINGLE_WG_MAX_SEGS == 2, "instantiations below");
-  if (segs <= 1)
-    AC4K_SINGLE_WG(1);
+  if (g.total_chunks <= 128)  // one 1024-vector segment
+    hipLaunchKernelGGL(quantize_nvfp4_single_wg_kernel<1>, dim3(1), dim3(OP_THREADS), 0, st, out, sf, in, gs, g, max_scale);
   else
-    AC4K_SINGLE_WG(2);
-#undef AC4K_SINGLE_WG
+    hipLaunchKernelGGL(quantize_nvfp4_single_wg_kernel<2>, dim3(1), dim3(OP_THREADS), 0, st, out, sf, in, gs, g, max_scale);
 }
 
 // Global scale + nvfp4 quantize of a dense [lead, R, K] tensor in one pass over the input, when
@@ -1168,8 +1129,8 @@ static bool try_quantize_nvfp4_onepass(void *out, void *sf, float *gs, const voi
   if (nwg < 8 || chunks > (int64_t)nwg * 128 * OP_MAX_NV) return false;
   const OnePassGeom g{(uint32_t)chunks, (uint32_t)(K / 64), (uint32_t)R, (uint32_t)align_up(R, 16), (uint32_t)lead};
   if (chunks <= 128 * SINGLE_WG_MAX_SEGS) {  // tiny: one workgroup, one launch, no grid wait
-    launch_single_wg<false>(static_cast<uint32_t *>(out), static_cast<uint32_t *>(sf), static_cast<const uint4 *>(in), gs,
-                            g, max_scale, nullptr, st);
+    launch_single_wg(static_cast<uint32_t *>(out), static_cast<uint32_t *>(sf), static_cast<const uint4 *>(in), gs, g,
+                     max_scale, st);
     return true;
   }
   const int slot = amax_slot(st);
@@ -1203,13 +1164,13 @@ static int launch_quantize_nvfp4(void *out, void *sf, const void *in, const Glob
     const int64_t chunks = g.Kp / 64;
     const bool sw = swizzle != 0;
     if (chunks >= 8)
-      launch_nvfp4_rowmajor<8>(o, s, x, gsrc, g, lead, st, nullptr, sw);
+      launch_nvfp4_rowmajor<8>(o, s, x, gsrc, g, lead, st, sw);
     else if (chunks >= 3)
-      launch_nvfp4_rowmajor<4>(o, s, x, gsrc, g, lead, st, nullptr, sw);
+      launch_nvfp4_rowmajor<4>(o, s, x, gsrc, g, lead, st, sw);
     else if (chunks == 2)
-      launch_nvfp4_rowmajor<2>(o, s, x, gsrc, g, lead, st, nullptr, sw);
+      launch_nvfp4_rowmajor<2>(o, s, x, gsrc, g, lead, st, sw);
     else
-      launch_nvfp4_rowmajor<1>(o, s, x, gsrc, g, lead, st, nullptr, sw);
+      launch_nvfp4_rowmajor<1>(o, s, x, gsrc, g, lead, st, sw);
   } else if (crossmajor_ok(in, R, s0, s1, sR, sK) && ceil_div(g.Rp, 128) <= 65535) {
     dim3 grid((unsigned)ceil_div(g.Kp / 64, 4), (unsigned)ceil_div(g.Rp, 128), (unsigned)lead);
     if (swizzle)
@@ -1272,32 +1233,6 @@ extern "C" __attribute__((visibility("default"))) int ac4k_quantize_nvfp4_bf16(v
 }
 
 namespace ac4k {
-
-// Internal: quantize a contiguous 2-D activation X [M, K] (K % 64 == 0, 16-byte aligned) like
-// ac4k_quantize_nvfp4_bf16 and also emit its exact fp16 dequantization (without the global
-// scale) to f16out [M, K].  Two launches.
-int quantize_activation_with_f16(void *out, void *sf, float *gs, const void *in, int64_t M, int64_t K,
-                                 float max_scale, _Float16 *f16out, hipStream_t st) {
-  AC4K_REQUIRE(K % 64 == 0 && rowmajor_ok(in, K, 0, 0, K, 1), "activation must be 16-byte aligned with K %% 64 == 0");
-  std::lock_guard<std::mutex> lock(g_enqueue_mutex);
-  if (M * (K / 64) <= 128 * SINGLE_WG_MAX_SEGS) {
-    const OnePassGeom og{(uint32_t)(M * (K / 64)), (uint32_t)(K / 64), (uint32_t)M, (uint32_t)align_up(M, 16), 1u};
-    launch_single_wg<true>(static_cast<uint32_t *>(out), static_cast<uint32_t *>(sf), static_cast<const uint4 *>(in), gs,
-                           og, max_scale, f16out, st);
-    return 0;
-  }
-  int slot = -1;
-  const int npart = launch_amax_partials(in, M * K, st, &slot);
-  GlobalScaleSrc gsrc{gs, slot, npart, max_scale};
-  if (npart == 0) {
-    launch_global_scale_atomic(gs, in, M * K, max_scale, st);
-    gsrc.slot = -1;
-  }
-  QuantGeom g{1, M, K, K, align_up(M, 16), 0, 0, K, 1, 0};
-  launch_nvfp4_rowmajor<8>(static_cast<uint8_t *>(out), static_cast<uint8_t *>(sf), static_cast<const uint16_t *>(in),
-                           gsrc, g, 1, st, f16out);
-  return 0;
-}
 
 template <RowFmt FMT, int LPR, int NV>
 static void launch_rowwise_rowmajor(uint8_t *out, float *sf, const uint16_t *in, const void *smax,

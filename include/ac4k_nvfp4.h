@@ -102,7 +102,7 @@ int ac4k_linear_nvfp4(void *D, int d_dtype, const void *A, const void *A_sf, con
  * (lib/cuda/sm120/linear_nvfp4.cu:753-901; the reference runs every shape through its one
  * 128x128 tile kernel).  Two families:
  *   - decode-sized, 1 <= M <= 32 and K % 256 == 0: a weight-streaming split-K kernel; the
- *     workspace receives the fp16 activation and the fp32 partial sums of the K-slices;
+ *     workspace receives the fp32 partial sums of the K-slices;
  *   - 32 < M with too few output tiles to fill the GPU and K % 128 == 0: split-K over the tile
  *     kernel; the workspace receives the fp32 partial sums.
  * `workspace` = ac4k_linear_nvfp4_skinny_workspace_bytes(M,N,K) bytes of device memory, 256-byte
@@ -117,7 +117,7 @@ int ac4k_linear_nvfp4_skinny(void *D, int d_dtype, const void *A, const void *A_
 /* Fused decode-sized linear: quantize(X,0,1) followed by linear(...) in one call.  No single
  * reference function: it equals the composition the reference's tests make
  * (test/test_linear_bench.py:128-137) — the activation bytes, scales and global scale it
- * produces are those of ac4k_quantize_nvfp4_bf16, and they are returned:
+ * produces are those of ac4k_quantize_nvfp4_bf16 (it is that call), and they are returned:
  * X bf16 [M,K] contiguous -> X_q [M,K/2], X_sf [K/64,align_up(M,16),4], X_gs (1 float).
  * workspace as for ac4k_linear_nvfp4_skinny. */
 int ac4k_linear_nvfp4_fused_bf16(void *D, int d_dtype, const void *X, void *X_q, void *X_sf,
