@@ -167,7 +167,7 @@ def linear_bytes(m, n, k):
     return (m + n) * k // 2 + ((m + 15) // 16 * 16 + (n + 15) // 16 * 16) * k // 16 + m * n * 2 + 8
 
 
-def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True, key=None):
+def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True, key=None, with_quantize=False):
     a, b = make_input((m, k), seed=0), make_input((n, k), seed=1, std=wstd)
     aq, bq = ops.quantize(a.cuda(), 0, 1), ops.quantize(b.cuda(), 0, 1)
     out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
@@ -180,13 +180,18 @@ def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True, key=None):
         ok = bool(torch.all((got.float() - ref.float()).abs() <= 1e-2 + 1e-2 * ref.float().abs()).item())
         del ref
     total, ms = time_gpu(lambda: ops.linear(*aq, *bq, out=out), steps, warmup)
+    ms_with_quantize = None
+    if with_quantize:  # the activation quantized inside the timed region, the weights not
+        xa = a.cuda()
+        _, ms_with_quantize = time_gpu(lambda: ops.linear(*ops.quantize(xa, 0, 1), *bq, out=out), steps, warmup)
+        del xa
     tflops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
     gbs = linear_bytes(m, n, k) / (ms * 1e-3) / 1e9
     t_flops, t_bytes = 2.0 * m * n * k / (MFMA_PEAK_TFLOPS * 1e12), linear_bytes(m, n, k) / (HBM_PEAK_GBS * 1e9)
     rl = roofline("mfma", tflops, key) if t_flops >= t_bytes else roofline("hbm", gbs, key)
     return {"workload": f"NVFP4 linear M={m} N={n} K={k}, bf16 out, operands pre-quantized", "ms": ms,
             "total_ms": total, "TFLOP/s": tflops, "GB/s": gbs, "within_1e-2_of_fp32_dequant_matmul": ok,
-            "roofline": rl}
+            "roofline": rl, "ms_with_activation_quantize": ms_with_quantize}
 
 
 def vendor_gemm_yardstick(steps, warmup, n=8192):
@@ -317,11 +322,14 @@ def main():
             shapes = {"cfg3_4096": bench_linear(ops, 4096, 4096, 4096, S, W, check=check)}
             for (n, k) in ((14336, 4096), (4096, 14336)):
                 for m in (16, 128, 2048, 8192):
-                    shapes[f"cfg4_M{m}_N{n}_K{k}"] = bench_linear(ops, m, n, k, S, W, wstd=0.02, check=check)
+                    shapes[f"cfg4_M{m}_N{n}_K{k}"] = bench_linear(ops, m, n, k, S, W, wstd=0.02, check=check,
+                                                                  with_quantize=True)
             for k_, v in shapes.items():
+                wq_ = v["ms_with_activation_quantize"]
                 log(f"[bench] {k_}: {v['ms'] * 1e3:.1f} us  {v['TFLOP/s']:.1f} TFLOP/s  {v['GB/s']:.0f} GB/s  "
                     f"{100 * v['roofline']['frac']:.1f}% of {v['roofline']['bound']} peak  "
-                    f"ok={v['within_1e-2_of_fp32_dequant_matmul']}")
+                    f"ok={v['within_1e-2_of_fp32_dequant_matmul']}"
+                    + ("" if wq_ is None else f"  with activation quantize {wq_ * 1e3:.1f} us"))
             line["linear_shapes"] = shapes
             dec = {f"cfg5_M{m}": bench_decode(ops, m, 28672, 8192, S, W, check) for m in (1, 8, 32)}
             for k_, v in dec.items():
