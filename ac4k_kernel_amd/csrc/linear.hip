@@ -856,7 +856,7 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   // ---- epilogue.  The MFMAs were issued with the operands swapped, so acc[i][j] holds the
   // TRANSPOSED 32x32 block: lane l, element e <-> n = j*32 + (e>>2)*8 + (l>>5)*4 + (e&3),
   // m = i*32 + (l&31): four consecutive n per lane.
-  const int64_t m0 = tm * BM + wm * (32 * MI), n0 = tn * P_BN + wn * 128;
+  const int64_t m0 = tm * BM + (swave >> 1) * (32 * MI), n0 = tn * P_BN + (swave & 1) * 128;
   if (sk.partial) {  // split-K: raw fp32 sums of this K range; the reduce kernel scales and converts
     float *pp = sk.partial + (int64_t)blockIdx.y * a.M * a.N;
     const bool v4 = (a.N & 3) == 0;
@@ -882,85 +882,116 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     AC4K_LTL(3, wall_clock64());
     return;
   }
-  // 2-byte outputs are staged through LDS (free now) so that every lane stores 16 bytes and a
-  // wave store covers whole 256-byte row segments.
+  // Outputs are staged through LDS (the operand stages are free now), one wave-private block of
+  // RP rows x 128 columns at a time, so that every lane stores 16 bytes and a wave store covers
+  // whole row segments (256 bytes of a 2-byte output, 512 bytes of fp32).  The bias of the tile's
+  // 256 columns sits behind the staging blocks as fp32.
   const float scale = (*a.A_gs) * (*a.B_gs);
   using DE = Elem<D_DT>;
-  typename DE::T *Dp = static_cast<typename DE::T *>(a.D);
-  float bias4[4][4][4];  // [j][g][e&3]
+  using DT = typename DE::T;
+  DT *Dp = static_cast<DT *>(a.D);
+  constexpr int S = sizeof(DT);
+  constexpr int RP = S == 2 ? 64 : 32;      // rows per staging pass
+  constexpr int PITCH = 128 * S + 16;       // bytes per staged row, 16 bytes of padding
+  constexpr int STG_BYTES = 4 * RP * PITCH;
+  static_assert(STG_BYTES + P_BN * 4 <= PL::LDS_BYTES, "epilogue staging and bias must fit in LDS");
+  // the last iterations' LDS-DMA fetches (into a stage nobody reads) must have landed before the
+  // stages are reused, and every wave must be done reading them
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  const float *bias_s = reinterpret_cast<const float *>(plds + STG_BYTES) + wn * 128 + half * 4;
   if constexpr (BIAS_DT != BIAS_NONE) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int g = 0; g < 4; ++g)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int64_t n = n0 + j * 32 + g * 8 + half * 4 + q;
-          bias4[j][g][q] = n < a.N ? Elem<BIAS_DT>::load(a.bias, n) : 0.0f;
-        }
+    const int64_t n = tn * P_BN + tid;
+    reinterpret_cast<float *>(plds + STG_BYTES)[tid] = n < a.N ? Elem<BIAS_DT>::load(a.bias, n) : 0.0f;
+    __syncthreads();
   }
-  auto value = [&](int i, int j, int e) {
-    float v = acc[i][j][e] * scale;
-    if constexpr (BIAS_DT != BIAS_NONE) v += bias4[j][e >> 2][e & 3];
+  // the four outputs acc[i][j][4g .. 4g+3] of a lane, scaled, plus their bias b
+  auto value4 = [&](int i, int j, int g, const float4 &b) {
+    float4 v = make_float4(acc[i][j][4 * g] * scale, acc[i][j][4 * g + 1] * scale, acc[i][j][4 * g + 2] * scale,
+                           acc[i][j][4 * g + 3] * scale);
+    if constexpr (BIAS_DT != BIAS_NONE) {
+      v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+    }
     return v;
   };
-  const bool vec_ok = sizeof(typename DE::T) == 2 && (a.N % 8 == 0) && ((uintptr_t)a.D % 16 == 0);
+  // bias of column block j: four 16-byte LDS reads in one go (one wait), kept for the rows of a pass
+  auto bias_of = [&](int j, float4 (&b)[4]) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      b[g] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      if constexpr (BIAS_DT != BIAS_NONE) b[g] = *reinterpret_cast<const float4 *>(bias_s + j * 32 + g * 8);
+    }
+  };
+  const bool vec_ok = (a.N % (16 / S) == 0) && ((uintptr_t)a.D % 16 == 0);
   if (vec_ok) {
-    constexpr int PITCH = 272;  // bytes per staged row: 128 outputs + 16 bytes of padding
-    static_assert(4 * 64 * PITCH <= PL::LDS_BYTES, "epilogue staging must fit in LDS");
-    __syncthreads();            // every wave is done reading the operand stages
-    char *stg = plds + wave * (64 * PITCH);
+    char *stg = plds + wave * (RP * PITCH);
+    constexpr int CPR = 128 * S / 16;  // 16-byte pieces per staged row
+    constexpr int RS = 64 / CPR;       // rows covered by one wave store
+    const int lrow = lane / CPR, lq = lane % CPR;
+    const int64_t row_bytes = a.N * S;
+    const uint32_t lane_off = (uint32_t)(lrow * row_bytes) + lq * 16;
+    char *out0 = reinterpret_cast<char *>(Dp) + (m0 * a.N + n0) * S;  // wave-uniform
+    const bool interior = m0 + 32 * MI <= a.M && n0 + 128 <= a.N;
+    const bool col_ok = n0 + lq * (16 / S) < a.N;
+    const int64_t rl = a.M - m0 - lrow;
+    const int rows_left = rl > 32 * MI ? 32 * MI : (int)rl;  // rows of the block below this lane's first one
 #pragma unroll
-    for (int p = 0; p < MI / 2; ++p) {
+    for (int p = 0; p < 32 * MI / RP; ++p) {
+      asm volatile("" ::: "memory");  // keeps the bias reads of one pass from being merged with the next one's
 #pragma unroll
-      for (int ii = 0; ii < 2; ++ii) {
-        const int i = 2 * p + ii;
+      for (int j = 0; j < 4; ++j) {
+        float4 b[4];
+        bias_of(j, b);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int ii = 0; ii < RP / 32; ++ii) {
+          const int i = p * (RP / 32) + ii;
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            const uint2 w = make_uint2(DE::cvt2(value(i, j, g * 4), value(i, j, g * 4 + 1)),
-                                       DE::cvt2(value(i, j, g * 4 + 2), value(i, j, g * 4 + 3)));
-            *reinterpret_cast<uint2 *>(stg + (ii * 32 + (lane & 31)) * PITCH + (j * 32 + g * 8 + half * 4) * 2) = w;
+            const float4 v = value4(i, j, g, b[g]);
+            char *dst = stg + (ii * 32 + (lane & 31)) * PITCH + (j * 32 + g * 8 + half * 4) * S;
+            if constexpr (S == 2) *reinterpret_cast<uint2 *>(dst) = make_uint2(DE::cvt2(v.x, v.y), DE::cvt2(v.z, v.w));
+            else *reinterpret_cast<float4 *>(dst) = v;
           }
+        }
       }
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the staging region is private to the wave
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the staging block is private to the wave
+      // pass `it` stores rows it*RS .. it*RS+RS-1 of the block: a wave-uniform base that advances by
+      // RS rows, plus a fixed 32-bit lane offset; the bounds checks are per lane only on edge tiles
+      const char *src = stg + lrow * PITCH + lq * 16;
+      char *rowp = out0 + (int64_t)p * RP * row_bytes;
+      if (interior) {
 #pragma unroll
-      for (int it = 0; it < 16; ++it) {
-        const int id = it * 64 + lane, row = id >> 4, q = id & 15;
-        const uint4 v = *reinterpret_cast<const uint4 *>(stg + row * PITCH + q * 16);
-        const int64_t m = m0 + p * 64 + row, n = n0 + q * 8;
-        if (m < a.M && n < a.N) *reinterpret_cast<uint4 *>(Dp + m * a.N + n) = v;
+        for (int it = 0; it < RP / RS; ++it)
+          *reinterpret_cast<uint4 *>(rowp + it * RS * row_bytes + lane_off) =
+              *reinterpret_cast<const uint4 *>(src + it * RS * PITCH);
+      } else {
+#pragma unroll
+        for (int it = 0; it < RP / RS; ++it) {
+          const uint4 v = *reinterpret_cast<const uint4 *>(src + it * RS * PITCH);
+          if (col_ok && p * RP + it * RS < rows_left) *reinterpret_cast<uint4 *>(rowp + it * RS * row_bytes + lane_off) = v;
+        }
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
-  } else if (sizeof(typename DE::T) == 4 && (a.N % 4 == 0) && ((uintptr_t)a.D % 16 == 0)) {
-    // fp32 output: a lane holds four consecutive columns, one 16-byte store each
-#pragma unroll
-    for (int i = 0; i < MI; ++i) {
-      const int64_t m = m0 + i * 32 + (lane & 31);
-      if (m >= a.M) continue;
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int64_t n = n0 + j * 32 + g * 8 + half * 4;
-          if (n < a.N)
-            *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.D) + m * a.N + n) =
-                make_float4(value(i, j, 4 * g), value(i, j, 4 * g + 1), value(i, j, 4 * g + 2), value(i, j, 4 * g + 3));
-        }
-    }
   } else {
 #pragma unroll
-    for (int i = 0; i < MI; ++i) {
-      const int64_t m = m0 + i * 32 + (lane & 31);
+    for (int j = 0; j < 4; ++j) {
+      float4 b[4];
+      bias_of(j, b);
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int i = 0; i < MI; ++i) {
+        const int64_t m = m0 + i * 32 + (lane & 31);
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int64_t n = n0 + j * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
-          if (m < a.M && n < a.N) Dp[m * a.N + n] = DE::cvt(value(i, j, e));
+        for (int g = 0; g < 4; ++g) {
+          const float4 v = value4(i, j, g, b[g]);
+          const float ve[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int64_t n = n0 + j * 32 + g * 8 + half * 4 + q;
+            if (m < a.M && n < a.N) Dp[m * a.N + n] = DE::cvt(ve[q]);
+          }
         }
+      }
     }
   }
   AC4K_LTL(3, wall_clock64());
@@ -1231,8 +1262,10 @@ static int dispatch_skinny(const SkinnyArgs &a, const SkinnyPlan &p, int d_dtype
 }
 
 // shapes the packed-LDS kernel takes: whole 128-k stages, 16-byte aligned rows, 32-bit lane offsets
+// (256 operand rows in the loop, 4 output rows of up to 4-byte elements in the epilogue)
 static bool packed_kernel_ok(const LinearArgs &a) {
-  return a.K % P_BK == 0 && (((uintptr_t)a.A | (uintptr_t)a.B) & 15) == 0 && (a.K >> 1) * 256 < (1ll << 31);
+  return a.K % P_BK == 0 && (((uintptr_t)a.A | (uintptr_t)a.B) & 15) == 0 && (a.K >> 1) * 256 < (1ll << 31) &&
+         a.N < (1ll << 27);
 }
 
 template <int D_DT, int BIAS_DT>

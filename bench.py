@@ -130,9 +130,27 @@ def bench_quantize(ops, shape, precision, steps, warmup, outliers, check=True, n
     _, ms = time_gpu(step, steps, warmup)
     nbytes = quant_bytes(shape, precision)
     gbs = nbytes / (ms * 1e-3) / 1e9
-    return {"workload": f"quantize {precision} {shape[0]}x{shape[1]} bf16" + (" outliers" if outliers else ""),
-            "ms": ms, "bytes": nbytes, "GB/s": gbs, "bit_exact_vs_oracle": ok,
-            "roofline": roofline("hbm", gbs, key), "rotating_buffers": nbuf}
+    r = {"workload": f"quantize {precision} {shape[0]}x{shape[1]} bf16" + (" outliers" if outliers else ""),
+         "ms": ms, "bytes": nbytes, "GB/s": gbs, "bit_exact_vs_oracle": ok,
+         "roofline": roofline("hbm", gbs, key), "rotating_buffers": nbuf}
+    if precision == "nvfp4":  # the quantize kernel alone, its global scale already on the device
+        from ac4k_kernel_amd import _rocm_ops
+        gss = [ops.quantize(x, 0, 1)[2] for x in xs]
+
+        def kernel_only():
+            j = i[0] % nbuf
+            i[0] += 1
+            _rocm_ops.quantize_nvfp4(outs[j][0], outs[j][1], xs[j], gss[j], 0, 1, False)
+
+        i[0] = 0
+        kernel_only()
+        same = torch.equal(outs[0][0], res[0]) and torch.equal(outs[0][1].view(torch.uint8), res[1].view(torch.uint8))
+        i[0] = 0
+        _, kms = time_gpu(kernel_only, steps, warmup)
+        r["global_scale_given"] = {"ms": kms, "GB/s": (nbytes - 4) / (kms * 1e-3) / 1e9,
+                                   "frac_of_hbm_peak": (nbytes - 4) / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                   "equals_whole_op_output": same}
+    return r
 
 
 def cpu_quantize_baseline(shape, outliers, budget_s=10.0):
@@ -226,6 +244,46 @@ def bench_decode(ops, m, n, k, steps, warmup, check=True):
             "roofline": roofline("hbm", gbs)}
 
 
+def bench_quantize_layouts(ops, steps, warmup):
+    """Quantizer layouts beyond (cross 0, reduce 1): the two calls of the reference's bandwidth test
+    (test/test_quantize_bandwidth.py:37-38, shape (1, 75600, 40, 128)) for nvfp4 and fp8, and the
+    swizzled row-major case.  Bytes = input + output + scales, the input counted once."""
+    res = {}
+    g = torch.Generator(device="cpu").manual_seed(4)
+    x = torch.randn((1, 75600, 40, 128), generator=g, dtype=torch.float32).to(torch.bfloat16).cuda()
+    y = make_input((8192, 4096), seed=0, outliers=True).cuda()
+    cases = (("attn_cross1_reduce3", x, 1, 3, False), ("attn_cross3_reduce1_swizzle", x, 3, 1, True),
+             ("rowmajor_8192x4096_swizzle", y, 0, 1, True))
+    for name, t, cross, red, swz in cases:
+        for prec in ("nvfp4", "fp8e4m3"):
+            r = ops.quantize(t, cross, red, precision=prec, swizzle=swz)
+            o, sf = r[0], r[1]
+            _, ms = time_gpu(lambda: ops.quantize(t, cross, red, precision=prec, swizzle=swz, output=o, sf=sf),
+                             steps, warmup)
+            nbytes = t.nbytes + o.nbytes + sf.nbytes
+            res[f"{name}_{prec}"] = {"shape": list(t.shape), "cross_dim": cross, "reduce_dim": red, "swizzle": swz,
+                                     "ms": ms, "GB/s": nbytes / (ms * 1e-3) / 1e9}
+            del r, o, sf
+    return res
+
+
+def bench_linear_epilogues(ops, steps, warmup, n=8192):
+    """Output dtype x bias matrix of the linear (test/test_linear_bench.py:178-205) at n^3."""
+    a, b = make_input((n, n), seed=0).cuda(), make_input((n, n), seed=1).cuda()
+    aq, bq = ops.quantize(a, 0, 1), ops.quantize(b, 0, 1)
+    del a, b
+    res = {}
+    for od in (torch.bfloat16, torch.float16, torch.float32):
+        for bd in (None, torch.bfloat16, torch.float32):
+            out = torch.empty((n, n), dtype=od, device="cuda")
+            bias = None if bd is None else torch.randn((1, n), device="cuda").to(bd)
+            _, ms = time_gpu(lambda: ops.linear(*aq, *bq, bias=bias, out=out), steps, warmup)
+            name = f"out_{str(od).split('.')[-1]}_bias_{'none' if bd is None else str(bd).split('.')[-1]}"
+            res[name] = {"ms": ms, "TFLOP/s": 2.0 * n ** 3 / (ms * 1e-3) / 1e12}
+            del out
+    return res
+
+
 def cpu_linear_baseline(n, k, rows=4096):
     """fp32 dequantize-then-matmul of the oracle on `rows` rows of the 8192^3 problem (the weight
     operand in full): about ten seconds of host work."""
@@ -298,7 +356,9 @@ def main():
         }
         for k_, v in quant.items():
             log(f"[bench] {k_}: {v['ms'] * 1e3:.1f} us  {v['GB/s']:.0f} GB/s  "
-                f"({100 * v['roofline']['frac']:.1f}% of HBM peak)  bit-exact={v['bit_exact_vs_oracle']}")
+                f"({100 * v['roofline']['frac']:.1f}% of HBM peak)  bit-exact={v['bit_exact_vs_oracle']}"
+                + (f"  kernel alone with the global scale given: {v['global_scale_given']['ms'] * 1e3:.1f} us "
+                   f"({100 * v['global_scale_given']['frac_of_hbm_peak']:.1f}%)" if "global_scale_given" in v else ""))
         if not args.no_cpu_baseline:
             quant["cpu_baseline"] = cpu_quantize_baseline((8192, 4096), True)
             log(f"[bench] cpu quantize oracle: {quant['cpu_baseline']['value']:.2f} GB/s on "
@@ -336,6 +396,14 @@ def main():
                 log(f"[bench] {k_}: {v['ms'] * 1e3:.1f} us  {v['GB/s']:.0f} GB/s "
                     f"({100 * v['roofline']['frac']:.1f}% of HBM peak)  ok={v['equals_quantize_then_linear_within_1e-2']}")
             line["decode"] = dec
+            lay = bench_quantize_layouts(ops, S, W)
+            for k_, v in lay.items():
+                log(f"[bench] quantize layout {k_}: {v['ms'] * 1e3:.1f} us  {v['GB/s']:.0f} GB/s")
+            line["quantize_layouts"] = lay
+            epi = bench_linear_epilogues(ops, S, W)
+            log("[bench] linear 8192^3 by output/bias dtype, TFLOP/s: "
+                + ", ".join(f"{k_} {v['TFLOP/s']:.0f}" for k_, v in epi.items()))
+            line["linear_epilogues"] = epi
         if quant is not None:
             line["quantize"] = quant
     else:
