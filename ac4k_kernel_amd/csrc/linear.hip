@@ -499,18 +499,22 @@ __device__ __forceinline__ void decode_half_block(_Float16 *tile, int row, int h
 // Requires K % 128 == 0 and 16-byte aligned operands.
 // ===========================================================================
 constexpr int P_BK = 128;     // k per stage (two 64-chunks)
-constexpr int P_STAGES = 3;
 constexpr int P_ROW = 64;     // packed bytes per row per stage: [chunk][half] x 16 B
-constexpr int P_BN = 256;
 
-template <int BM>
-struct PLayout {               // byte offsets inside one LDS stage
+template <int BM, int BN, int PS>
+struct PLayout {               // byte offsets inside one LDS stage; PS stages
   static constexpr int OFF_B = BM * P_ROW;                 // B rows follow the A rows
-  static constexpr int OFF_SFA = OFF_B + P_BN * P_ROW;     // scale dwords: [chunk][BM rows]
-  static constexpr int OFF_SFB = OFF_SFA + 2 * BM * 4;     // [chunk][256 rows]
-  static constexpr int STAGE_BYTES = OFF_SFB + 2 * P_BN * 4;
-  static constexpr int LDS_BYTES = P_STAGES * STAGE_BYTES;
+  static constexpr int OFF_SFA = OFF_B + BN * P_ROW;       // scale dwords: [chunk][BM rows]
+  static constexpr int OFF_SFB = OFF_SFA + 2 * BM * 4;     // [chunk][BN rows]
+  static constexpr int STAGE_BYTES = OFF_SFB + 2 * BN * 4;
+  static constexpr int LDS_BYTES = PS * STAGE_BYTES;
+  static_assert(LDS_BYTES <= 160 * 1024, "stages must fit in the CU's LDS");
 };
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
 
 // LDS-DMA: global_load_lds with a scalar 64-bit base, a 32-bit lane offset and the LDS
 // destination of lane 0 in M0 (lane l lands at M0 + size * l).  Issued through inline asm so
@@ -526,9 +530,9 @@ __device__ __forceinline__ void dma4(const void *sbase, uint32_t voff, uint32_t 
                :: "s"(lds_stage), "s"(lds_piece), "v"(voff), "s"(sbase) : "memory", "scc");
 }
 
-template <int MI>
+template <int MI, int NJ>
 struct DecFrags {
-  f16x8 a[MI], b[4];
+  f16x8 a[MI], b[NJ];
 };
 
 // dword `w` (8 nibbles) times block scale `sc` (both halves of `sc2` hold candidates, HI picks)
@@ -565,21 +569,147 @@ struct SplitK {
   int splits;
 };
 
-// MI = 32-row fragments per wave along M: 4 (BM = 256) or 2 (BM = 128).
-template <int D_DT, int BIAS_DT, int MI>
+// Epilogue of the packed-LDS tile kernel: the accumulators of one wave, (32*MI) x (32*NJ) outputs, to
+// `out` (row stride N).  acc[i][j] holds the TRANSPOSED 32x32 block (the MFMAs are issued with the
+// operands swapped): lane l, element e <-> n = j*32 + (e>>2)*8 + (l>>5)*4 + (e&3), m = i*32 + (l&31),
+// i.e. four consecutive n per lane.  RAW stores the fp32 sums as they are (split-K partials);
+// otherwise out = cvt(acc * scale + bias).  Outputs are staged through LDS (`lds`, free at this
+// point), one wave-private block of RP rows at a time, so that every lane stores 16 bytes and a
+// wave store covers whole row segments; the bias of the tile's columns sits behind the staging
+// blocks as fp32.  Callers have passed a workgroup barrier after their last read of `lds`.
+template <int OUT_DT, int BIAS_DT, bool RAW, int MI, int NJ, int LDS_BYTES>
+__device__ __forceinline__ void store_tile(const f32x16 (&acc)[MI][NJ], char *lds, void *out, const void *bias,
+                                           float scale, int64_t M, int64_t N, int64_t m0, int64_t n0,
+                                           int64_t tile_n0) {
+  using DE = Elem<OUT_DT>;
+  using DT = typename DE::T;
+  DT *Dp = static_cast<DT *>(out);
+  constexpr int S = sizeof(DT);
+  constexpr int WN = 32 * NJ;               // columns per wave
+  constexpr int RP = S == 2 ? 64 : 32;      // rows per staging pass
+  constexpr int PITCH = WN * S + 16;        // bytes per staged row, 16 bytes of padding
+  constexpr int STG_BYTES = 4 * RP * PITCH;
+  static_assert(STG_BYTES + 2 * WN * 4 <= LDS_BYTES, "epilogue staging and bias must fit in LDS");
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, wn = wave & 1;
+  const float *bias_s = reinterpret_cast<const float *>(lds + STG_BYTES) + wn * WN + half * 4;
+  if constexpr (BIAS_DT != BIAS_NONE) {
+    if (tid < 2 * WN) {
+      const int64_t n = tile_n0 + tid;
+      reinterpret_cast<float *>(lds + STG_BYTES)[tid] = n < N ? Elem<BIAS_DT>::load(bias, n) : 0.0f;
+    }
+    __syncthreads();
+  }
+  // the four outputs acc[i][j][4g .. 4g+3] of a lane, scaled, plus their bias b
+  auto value4 = [&](int i, int j, int g, const float4 &b) {
+    float4 v = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+    if constexpr (!RAW) {
+      v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
+    }
+    if constexpr (BIAS_DT != BIAS_NONE) {
+      v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+    }
+    return v;
+  };
+  // bias of column block j: four 16-byte LDS reads in one go (one wait), kept for the rows of a pass
+  auto bias_of = [&](int j, float4 (&b)[4]) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      b[g] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      if constexpr (BIAS_DT != BIAS_NONE) b[g] = *reinterpret_cast<const float4 *>(bias_s + j * 32 + g * 8);
+    }
+  };
+  const bool vec_ok = (N % (16 / S) == 0) && ((uintptr_t)out % 16 == 0);
+  if (vec_ok) {
+    char *stg = lds + wave * (RP * PITCH);
+    constexpr int CPR = WN * S / 16;   // 16-byte pieces per staged row
+    constexpr int RS = 64 / CPR;       // rows covered by one wave store
+    const int lrow = lane / CPR, lq = lane % CPR;
+    const int64_t row_bytes = N * S;
+    const uint32_t lane_off = (uint32_t)(lrow * row_bytes) + lq * 16;
+    char *out0 = reinterpret_cast<char *>(Dp) + (m0 * N + n0) * S;  // wave-uniform
+    const bool interior = m0 + 32 * MI <= M && n0 + WN <= N;
+    const bool col_ok = n0 + lq * (16 / S) < N;
+    const int64_t rl = M - m0 - lrow;
+    const int rows_left = rl > 32 * MI ? 32 * MI : (int)rl;  // rows of the block below this lane's first one
+#pragma unroll
+    for (int p = 0; p < 32 * MI / RP; ++p) {
+      asm volatile("" ::: "memory");  // keeps the bias reads of one pass from being merged with the next one's
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        float4 b[4];
+        bias_of(j, b);
+#pragma unroll
+        for (int ii = 0; ii < RP / 32; ++ii) {
+          const int i = p * (RP / 32) + ii;
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const float4 v = value4(i, j, g, b[g]);
+            char *dst = stg + (ii * 32 + (lane & 31)) * PITCH + (j * 32 + g * 8 + half * 4) * S;
+            if constexpr (S == 2) *reinterpret_cast<uint2 *>(dst) = make_uint2(DE::cvt2(v.x, v.y), DE::cvt2(v.z, v.w));
+            else *reinterpret_cast<float4 *>(dst) = v;
+          }
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the staging block is private to the wave
+      // pass `it` stores rows it*RS .. it*RS+RS-1 of the block: a wave-uniform base that advances by
+      // RS rows, plus a fixed 32-bit lane offset; the bounds checks are per lane only on edge tiles
+      const char *src = stg + lrow * PITCH + lq * 16;
+      char *rowp = out0 + (int64_t)p * RP * row_bytes;
+      if (interior) {
+#pragma unroll
+        for (int it = 0; it < RP / RS; ++it)
+          *reinterpret_cast<uint4 *>(rowp + it * RS * row_bytes + lane_off) =
+              *reinterpret_cast<const uint4 *>(src + it * RS * PITCH);
+      } else {
+#pragma unroll
+        for (int it = 0; it < RP / RS; ++it) {
+          const uint4 v = *reinterpret_cast<const uint4 *>(src + it * RS * PITCH);
+          if (col_ok && p * RP + it * RS < rows_left) *reinterpret_cast<uint4 *>(rowp + it * RS * row_bytes + lane_off) = v;
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      float4 b[4];
+      bias_of(j, b);
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        const int64_t m = m0 + i * 32 + (lane & 31);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const float4 v = value4(i, j, g, b[g]);
+          const float ve[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int64_t n = n0 + j * 32 + g * 8 + half * 4 + q;
+            if (m < M && n < N) Dp[m * N + n] = DE::cvt(ve[q]);
+          }
+        }
+      }
+    }
+  }
+}
+
+// MI = 32-row fragments per wave along M: 4 (BM = 256) or 2 (BM = 128);
+// NJ = 32-column fragments per wave along N: 4 (BN = 256), 2 (BN = 128) or 1 (BN = 64);
+// PS = LDS stages: PS - 1 k-steps are in flight ahead of the one being multiplied, which a small
+// tile needs because its k-step is much shorter than the memory latency.
+template <int D_DT, int BIAS_DT, int MI, int NJ, int PS>
 __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArgs a, SplitK sk) {
   extern __shared__ __attribute__((aligned(16))) char plds[];
   AC4K_LTL(0, wall_clock64());
-  constexpr int BM = 64 * MI;              // two waves along M
-  using PL = PLayout<BM>;
+  constexpr int BM = 64 * MI, BN = 64 * NJ;  // two waves along M, two along N
+  using PL = PLayout<BM, BN, PS>;
   constexpr int NDA = BM / 4 / 16;         // 16-row A transfers per wave per stage
-  constexpr int NDB = P_BN / 4 / 16;       // 16-row B transfers per wave per stage
+  constexpr int NDB = BN / 4 / 16;         // 16-row B transfers per wave per stage
   constexpr int NSA = 2 * (BM / 64);       // scale transfers of A per stage: chunks x 64-row blocks
-  constexpr int NS = (NSA + 8) / 4;        // scale transfers per wave
+  constexpr int NSB = 2 * (BN / 64);
+  constexpr int NS = (NSA + NSB + 3) / 4;  // scale transfers per wave (a remainder repeats the last one)
   constexpr int NPIECES = NDA + NDB + NS;
-  static_assert((NSA + 8) % 4 == 0, "scale transfers must split evenly over the waves");
 
-  const int64_t tiles_m = ceil_div(a.M, BM), tiles_n = ceil_div(a.N, P_BN);
+  const int64_t tiles_m = ceil_div(a.M, BM), tiles_n = ceil_div(a.N, BN);
   const int64_t ntiles = tiles_m * tiles_n;
   int64_t pid = blockIdx.x;
   {  // contiguous run of tiles per XCD (workgroups are dealt round-robin to the 8 XCDs)
@@ -618,7 +748,7 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
 #pragma unroll
   for (int q = 0; q < NDB; ++q) {
     int64_t rb = (swave * NDB + q) * 16 + (lane >> 2);
-    rb = tn * P_BN + rb < a.N ? rb : a.N - 1 - tn * P_BN;
+    rb = tn * BN + rb < a.N ? rb : a.N - 1 - tn * BN;
     offB[q] = (uint32_t)(rb * kb + (lane & 3) * 16);
   }
   auto uniform_ptr = [](const void *p) {  // pin a wave-uniform pointer to scalar registers
@@ -627,28 +757,29 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
   };
   const uint8_t *baseA = uniform_ptr(a.A + tm * BM * kb + (int64_t)kt0 * P_ROW);
-  const uint8_t *baseB = uniform_ptr(a.B + tn * P_BN * kb + (int64_t)kt0 * P_ROW);
-  // scale transfers: piece g = swave * NS + p.  g < NSA: operand A, chunk g / (BM/64), 64-row block
-  // g % (BM/64); otherwise operand B, chunk (g-NSA) / 4, block (g-NSA) % 4.  Source base, bytes
-  // per stage and LDS offset are wave-uniform and fixed, computed here so that the loop body
-  // stays free of branches.
+  const uint8_t *baseB = uniform_ptr(a.B + tn * BN * kb + (int64_t)kt0 * P_ROW);
+  // scale transfers: piece g = swave * NS + p (past the last piece: the last piece again, which
+  // lands the same bytes in the same place).  g < NSA: operand A, chunk g / (BM/64), 64-row block
+  // g % (BM/64); otherwise operand B, chunk (g-NSA) / (BN/64), block (g-NSA) % (BN/64).  Source
+  // base, bytes per stage and LDS offset are wave-uniform and fixed, computed here so that the
+  // loop body stays free of branches.
   const uint8_t *sfA8 = uniform_ptr(a.A_sf), *sfB8 = uniform_ptr(a.B_sf);
   uint32_t offS[NS], ldsS[NS];
   const uint8_t *baseS[NS];
   int64_t strideS[NS];
 #pragma unroll
   for (int p2 = 0; p2 < NS; ++p2) {
-    const int gq = swave * NS + p2;
+    const int gq = swave * NS + p2 < NSA + NSB ? swave * NS + p2 : NSA + NSB - 1;
     const bool isB = gq >= NSA;
-    const int gl = isB ? gq - NSA : gq, nb = isB ? 4 : BM / 64;
+    const int gl = isB ? gq - NSA : gq, nb = isB ? BN / 64 : BM / 64;
     const int c = gl / nb, rb = gl % nb;
     const int64_t rows = isB ? a.Np : a.Mp;
-    int64_t sr = (isB ? tn * P_BN : tm * BM) + rb * 64 + lane;
+    int64_t sr = (isB ? tn * BN : tm * BM) + rb * 64 + lane;
     sr = sr < rows ? sr : rows - 1;
     offS[p2] = (uint32_t)sr * 4u;  // byte offset inside a scale plane
     strideS[p2] = 2 * rows * 4;    // two planes (chunks) per stage
     baseS[p2] = uniform_ptr((isB ? sfB8 : sfA8) + c * rows * 4 + kt0 * strideS[p2]);
-    ldsS[p2] = (uint32_t)__builtin_amdgcn_readfirstlane((isB ? PL::OFF_SFB + c * P_BN * 4 : PL::OFF_SFA + c * BM * 4) + rb * 256);
+    ldsS[p2] = (uint32_t)__builtin_amdgcn_readfirstlane((isB ? PL::OFF_SFB + c * BN * 4 : PL::OFF_SFA + c * BM * 4) + rb * 256);
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)plds;
   // LDS destinations of this wave's transfers inside a stage (wave-uniform, loop invariant)
@@ -698,29 +829,29 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
       if (q * 4 / NS == qr) issue_piece(stage_lds, p, NDA + NDB + q);
   };
 
-  f32x16 acc[MI][4];
+  f32x16 acc[MI][NJ];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   // fragment addresses inside a stage (bytes)
   const int fa_off = (wm * (32 * MI) + (lane & 31)) * P_ROW + half * 16;
-  const int fb_off = PL::OFF_B + (wn * 128 + (lane & 31)) * P_ROW + half * 16;
+  const int fb_off = PL::OFF_B + (wn * (32 * NJ) + (lane & 31)) * P_ROW + half * 16;
   // a lane needs the two scale bytes of its half of the chunk: blocks 2*half, 2*half+1
   const int sa_off = PL::OFF_SFA + (wm * (32 * MI) + (lane & 31)) * 4 + half * 2;
-  const int sb_off = PL::OFF_SFB + (wn * 128 + (lane & 31)) * 4 + half * 2;
+  const int sb_off = PL::OFF_SFB + (wn * (32 * NJ) + (lane & 31)) * 4 + half * 2;
 
-  uint4 PA[2][MI], PB[2][4];  // packed fragments of a 64-chunk, double buffered by chunk parity
-  f16x2 SA[2][MI], SB[2][4];  // their two block scales (blocks 2*half, 2*half+1) as fp16
+  uint4 PA[2][MI], PB[2][NJ];  // packed fragments of a 64-chunk, double buffered by chunk parity
+  f16x2 SA[2][MI], SB[2][NJ];  // their two block scales (blocks 2*half, 2*half+1) as fp16
   auto load_chunk = [&](uint32_t stage_off, int c) {
     const char *st = plds + stage_off;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if (i < MI) PA[c][i] = *reinterpret_cast<const uint4 *>(st + fa_off + c * 32 + i * 32 * P_ROW);
-      PB[c][i] = *reinterpret_cast<const uint4 *>(st + fb_off + c * 32 + i * 32 * P_ROW);
+      if (i < NJ) PB[c][i] = *reinterpret_cast<const uint4 *>(st + fb_off + c * 32 + i * 32 * P_ROW);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -728,40 +859,36 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
         const uint32_t wa = *reinterpret_cast<const uint16_t *>(st + sa_off + c * (BM * 4) + i * 128);
         SA[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wa, 1.0f, false);
       }
-      const uint32_t wb = *reinterpret_cast<const uint16_t *>(st + sb_off + c * (P_BN * 4) + i * 128);
-      SB[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wb, 1.0f, false);
+      if (i < NJ) {
+        const uint32_t wb = *reinterpret_cast<const uint16_t *>(st + sb_off + c * (BN * 4) + i * 128);
+        SB[c][i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wb, 1.0f, false);
+      }
     }
   };
 
-  DecFrags<MI> D[2];
-  auto decode = [&](DecFrags<MI> &d, int c, auto S) {
+  DecFrags<MI, NJ> D[2];
+  auto decode = [&](DecFrags<MI, NJ> &d, int c, auto S) {
     constexpr int s = decltype(S)::value;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if (i < MI) d.a[i] = decode_dword<(s >= 2)>(dword_of<s>(PA[c][i]), SA[c][i]);
-      d.b[i] = decode_dword<(s >= 2)>(dword_of<s>(PB[c][i]), SB[c][i]);
+      if (i < NJ) d.b[i] = decode_dword<(s >= 2)>(dword_of<s>(PB[c][i]), SB[c][i]);
     }
   };
-  auto mfma16 = [&](const DecFrags<MI> &d) {
+  auto mfma16 = [&](const DecFrags<MI, NJ> &d) {
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < NJ; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(d.b[j], d.a[i], acc[i][j], 0, 0, 0);  // D^T block
   };
   auto interleave = [&]() {  // the decode of the next sub-step rides in the shadow of the MFMAs
-    if constexpr (MI == 4) {
+    constexpr int NMFMA = MI * NJ, NVALU = 8 * (MI + NJ);
+    constexpr int PER = (NVALU + NMFMA - 1) / NMFMA;  // 4 for 4x4, 6 for 2x4 and 4x2, 8 for 2x2, ...
 #pragma unroll
-      for (int g = 0; g < 16; ++g) {  // 16 x (1 MFMA, 4 VALU)
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-      }
-    } else {
-#pragma unroll
-      for (int g = 0; g < 8; ++g) {  // 8 x (1 MFMA, 6 VALU)
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
-      }
+    for (int g = 0; g < NMFMA; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, PER, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -770,25 +897,22 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   using I2 = std::integral_constant<int, 2>;
   using I3 = std::integral_constant<int, 3>;
 
-  // prologue: stages 0 and 1 in flight, stage 0 visible, chunk 0 fragments and first decode
+  // prologue: stages 0 .. PS-2 in flight (past the last k-step: the last one again), stage 0
+  // visible, chunk 0 fragments and first decode
+  static_assert(PS >= 3 && (PS - 2) * NPIECES <= 63, "the wait counts below must fit the 6-bit counter");
   const int last = nkt - 1;
-  issue_stage(lds_base, src_at(0));
-  if (nkt > 1) issue_stage(lds_base + PL::STAGE_BYTES, src_at(1));
-  if (nkt > 1) {
-    static_assert(NPIECES == 12 || NPIECES == 9, "wait count below is spelled out per variant");
-    if constexpr (NPIECES == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
-  } else {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  }
+#pragma unroll
+  for (int d = 0; d < PS - 1; ++d) issue_stage(lds_base + d * PL::STAGE_BYTES, src_at(d < last ? d : last));
+  wait_vmcnt<(PS - 2) * NPIECES>();  // everything of stage 0 has landed, later stages may be in flight
   __syncthreads();
   load_chunk(0, 0);
   decode(D[0], 0, I0{});
 
   // loop-carried, wave-uniform: LDS offsets of the stages holding k-steps kt, kt+1 and of the one
-  // being filled with kt+2 (rotating), and the source pointers of k-step min(kt+2, last)
-  uint32_t st_cur = 0, st_nxt = PL::STAGE_BYTES, st_dma = 2 * PL::STAGE_BYTES;
-  Src src = src_at(last < 2 ? last : 2);
+  // being filled with kt+PS-1 (a ring of PS), and the source pointers of k-step min(kt+PS-1, last)
+  uint32_t st_cur = 0, st_nxt = PL::STAGE_BYTES, st_dma = (PS - 1) * PL::STAGE_BYTES;
+  auto ring_next = [](uint32_t o) { return o + PL::STAGE_BYTES == (uint32_t)PL::LDS_BYTES ? 0u : o + PL::STAGE_BYTES; };
+  Src src = src_at(last < PS - 1 ? last : PS - 1);
 #ifdef AC4K_LINEAR_TIMELINE
   const uint64_t tl_c0 = __builtin_readcyclecounter();
 #endif
@@ -808,11 +932,12 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     decode(D[0], 1, I0{});
     mfma16(D[1]);
     interleave();
-    // stage kt+1 must be complete (own DMA done, then everybody's); stage kt-1 is free after this
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // stage kt+1 must be complete (own DMA done, then everybody's; stages kt+2 .. kt+PS-2 may still
+    // be in flight); stage kt-1 is free after this
+    wait_vmcnt<(PS - 3) * NPIECES>();
     __syncthreads();
     // chunk 1: sub-steps 4..7 (chunk 0 of the next stage is fetched meanwhile); the DMA of stage
-    // kt+2 is spread over these sub-steps
+    // kt+PS-1 is spread over these sub-steps
     const uint32_t dma_lds = lds_base + st_dma;
     decode(D[1], 1, I1{});
     issue_quarter(dma_lds, src, 0);
@@ -832,11 +957,10 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     mfma16(D[1]);
     interleave();
     // rotate the stages; advance the sources unless they already sit on the last k-step
-    const uint32_t freed = st_cur;
     st_cur = st_nxt;
-    st_nxt = st_dma;
-    st_dma = freed;
-    const bool adv = kt + 3 <= last;
+    st_nxt = ring_next(st_nxt);
+    st_dma = ring_next(st_dma);
+    const bool adv = kt + PS <= last;
     src.a += adv ? P_ROW : 0;
     src.b += adv ? P_ROW : 0;
 #pragma unroll
@@ -856,143 +980,17 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   // ---- epilogue.  The MFMAs were issued with the operands swapped, so acc[i][j] holds the
   // TRANSPOSED 32x32 block: lane l, element e <-> n = j*32 + (e>>2)*8 + (l>>5)*4 + (e&3),
   // m = i*32 + (l&31): four consecutive n per lane.
-  const int64_t m0 = tm * BM + (swave >> 1) * (32 * MI), n0 = tn * P_BN + (swave & 1) * 128;
-  if (sk.partial) {  // split-K: raw fp32 sums of this K range; the reduce kernel scales and converts
-    float *pp = sk.partial + (int64_t)blockIdx.y * a.M * a.N;
-    const bool v4 = (a.N & 3) == 0;
-#pragma unroll
-    for (int i = 0; i < MI; ++i) {
-      const int64_t m = m0 + i * 32 + (lane & 31);
-      if (m >= a.M) continue;
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int64_t n = n0 + j * 32 + g * 8 + half * 4;
-          if (v4 && n + 3 < a.N) {
-            *reinterpret_cast<float4 *>(pp + m * a.N + n) =
-                make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
-          } else {
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-              if (n + q < a.N) pp[m * a.N + n + q] = acc[i][j][4 * g + q];
-          }
-        }
-    }
-    AC4K_LTL(3, wall_clock64());
-    return;
-  }
-  // Outputs are staged through LDS (the operand stages are free now), one wave-private block of
-  // RP rows x 128 columns at a time, so that every lane stores 16 bytes and a wave store covers
-  // whole row segments (256 bytes of a 2-byte output, 512 bytes of fp32).  The bias of the tile's
-  // 256 columns sits behind the staging blocks as fp32.
-  const float scale = (*a.A_gs) * (*a.B_gs);
-  using DE = Elem<D_DT>;
-  using DT = typename DE::T;
-  DT *Dp = static_cast<DT *>(a.D);
-  constexpr int S = sizeof(DT);
-  constexpr int RP = S == 2 ? 64 : 32;      // rows per staging pass
-  constexpr int PITCH = 128 * S + 16;       // bytes per staged row, 16 bytes of padding
-  constexpr int STG_BYTES = 4 * RP * PITCH;
-  static_assert(STG_BYTES + P_BN * 4 <= PL::LDS_BYTES, "epilogue staging and bias must fit in LDS");
+  const int64_t m0 = tm * BM + (swave >> 1) * (32 * MI), n0 = tn * BN + (swave & 1) * (32 * NJ);
   // the last iterations' LDS-DMA fetches (into a stage nobody reads) must have landed before the
   // stages are reused, and every wave must be done reading them
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  const float *bias_s = reinterpret_cast<const float *>(plds + STG_BYTES) + wn * 128 + half * 4;
-  if constexpr (BIAS_DT != BIAS_NONE) {
-    const int64_t n = tn * P_BN + tid;
-    reinterpret_cast<float *>(plds + STG_BYTES)[tid] = n < a.N ? Elem<BIAS_DT>::load(a.bias, n) : 0.0f;
-    __syncthreads();
-  }
-  // the four outputs acc[i][j][4g .. 4g+3] of a lane, scaled, plus their bias b
-  auto value4 = [&](int i, int j, int g, const float4 &b) {
-    float4 v = make_float4(acc[i][j][4 * g] * scale, acc[i][j][4 * g + 1] * scale, acc[i][j][4 * g + 2] * scale,
-                           acc[i][j][4 * g + 3] * scale);
-    if constexpr (BIAS_DT != BIAS_NONE) {
-      v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
-    }
-    return v;
-  };
-  // bias of column block j: four 16-byte LDS reads in one go (one wait), kept for the rows of a pass
-  auto bias_of = [&](int j, float4 (&b)[4]) {
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      b[g] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-      if constexpr (BIAS_DT != BIAS_NONE) b[g] = *reinterpret_cast<const float4 *>(bias_s + j * 32 + g * 8);
-    }
-  };
-  const bool vec_ok = (a.N % (16 / S) == 0) && ((uintptr_t)a.D % 16 == 0);
-  if (vec_ok) {
-    char *stg = plds + wave * (RP * PITCH);
-    constexpr int CPR = 128 * S / 16;  // 16-byte pieces per staged row
-    constexpr int RS = 64 / CPR;       // rows covered by one wave store
-    const int lrow = lane / CPR, lq = lane % CPR;
-    const int64_t row_bytes = a.N * S;
-    const uint32_t lane_off = (uint32_t)(lrow * row_bytes) + lq * 16;
-    char *out0 = reinterpret_cast<char *>(Dp) + (m0 * a.N + n0) * S;  // wave-uniform
-    const bool interior = m0 + 32 * MI <= a.M && n0 + 128 <= a.N;
-    const bool col_ok = n0 + lq * (16 / S) < a.N;
-    const int64_t rl = a.M - m0 - lrow;
-    const int rows_left = rl > 32 * MI ? 32 * MI : (int)rl;  // rows of the block below this lane's first one
-#pragma unroll
-    for (int p = 0; p < 32 * MI / RP; ++p) {
-      asm volatile("" ::: "memory");  // keeps the bias reads of one pass from being merged with the next one's
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float4 b[4];
-        bias_of(j, b);
-#pragma unroll
-        for (int ii = 0; ii < RP / 32; ++ii) {
-          const int i = p * (RP / 32) + ii;
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const float4 v = value4(i, j, g, b[g]);
-            char *dst = stg + (ii * 32 + (lane & 31)) * PITCH + (j * 32 + g * 8 + half * 4) * S;
-            if constexpr (S == 2) *reinterpret_cast<uint2 *>(dst) = make_uint2(DE::cvt2(v.x, v.y), DE::cvt2(v.z, v.w));
-            else *reinterpret_cast<float4 *>(dst) = v;
-          }
-        }
-      }
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the staging block is private to the wave
-      // pass `it` stores rows it*RS .. it*RS+RS-1 of the block: a wave-uniform base that advances by
-      // RS rows, plus a fixed 32-bit lane offset; the bounds checks are per lane only on edge tiles
-      const char *src = stg + lrow * PITCH + lq * 16;
-      char *rowp = out0 + (int64_t)p * RP * row_bytes;
-      if (interior) {
-#pragma unroll
-        for (int it = 0; it < RP / RS; ++it)
-          *reinterpret_cast<uint4 *>(rowp + it * RS * row_bytes + lane_off) =
-              *reinterpret_cast<const uint4 *>(src + it * RS * PITCH);
-      } else {
-#pragma unroll
-        for (int it = 0; it < RP / RS; ++it) {
-          const uint4 v = *reinterpret_cast<const uint4 *>(src + it * RS * PITCH);
-          if (col_ok && p * RP + it * RS < rows_left) *reinterpret_cast<uint4 *>(rowp + it * RS * row_bytes + lane_off) = v;
-        }
-      }
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    }
+  if (sk.partial) {  // split-K: raw fp32 sums of this K range; the reduce kernel scales and converts
+    store_tile<AC4K_DTYPE_FP32, BIAS_NONE, true, MI, NJ, PL::LDS_BYTES>(
+        acc, plds, sk.partial + (int64_t)blockIdx.y * a.M * a.N, nullptr, 1.0f, a.M, a.N, m0, n0, tn * BN);
   } else {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float4 b[4];
-      bias_of(j, b);
-#pragma unroll
-      for (int i = 0; i < MI; ++i) {
-        const int64_t m = m0 + i * 32 + (lane & 31);
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const float4 v = value4(i, j, g, b[g]);
-          const float ve[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int64_t n = n0 + j * 32 + g * 8 + half * 4 + q;
-            if (m < a.M && n < a.N) Dp[m * a.N + n] = DE::cvt(ve[q]);
-          }
-        }
-      }
-    }
+    store_tile<D_DT, BIAS_DT, false, MI, NJ, PL::LDS_BYTES>(acc, plds, a.D, a.bias, (*a.A_gs) * (*a.B_gs), a.M, a.N,
+                                                           m0, n0, tn * BN);
   }
   AC4K_LTL(3, wall_clock64());
 }
@@ -1011,22 +1009,82 @@ static int allow_dynamic_lds(Kernel *kern, std::atomic<uint32_t> &done_mask, int
   return 0;
 }
 
-template <int D_DT, int BIAS_DT, int MI>
-static int launch_tile256p_mi(const LinearArgs &a, const SplitK &sk, hipStream_t st) {
-  auto *kern = linear_nvfp4_tile256p_kernel<D_DT, BIAS_DT, MI>;
-  using PL = PLayout<64 * MI>;
+// LDS stages per tile shape: enough k-steps in flight to cover the memory latency
+constexpr int tile_stages(int mi, int nj) { return mi * nj >= 16 ? 3 : mi * nj >= 8 ? 4 : mi * nj >= 4 ? 6 : 8; }
+
+template <int D_DT, int BIAS_DT, int MI, int NJ>
+static int launch_tile_p(const LinearArgs &a, const SplitK &sk, hipStream_t st) {
+  constexpr int PS = tile_stages(MI, NJ);
+  auto *kern = linear_nvfp4_tile256p_kernel<D_DT, BIAS_DT, MI, NJ, PS>;
+  using PL = PLayout<64 * MI, 64 * NJ, PS>;
   static std::atomic<uint32_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, lds_ok, PL::LDS_BYTES)) return rc;
-  const int64_t ntiles = ceil_div(a.M, 64 * MI) * ceil_div(a.N, P_BN);
+  const int64_t ntiles = ceil_div(a.M, 64 * MI) * ceil_div(a.N, 64 * NJ);
   hipLaunchKernelGGL(kern, dim3((unsigned)ntiles, (unsigned)sk.splits), dim3(256), PL::LDS_BYTES, st, a, sk);
   return 0;
 }
 
-// the packed-LDS kernel with the tile height that suits M; no split-K (one K range, output to D)
+// Tile shape and K split of the packed-LDS kernel for one problem.
+struct TilePlan {
+  int mi, nj;              // tile = (64 mi) x (64 nj)
+  int splits;              // K ranges per tile; > 1 needs `partial_bytes` of fp32 scratch
+  int64_t partial_bytes;
+};
+
+// Picks the tile and the split by a rough cost model in microseconds on 256 CUs: rounds of
+// workgroups x stages per range x time per 128-k stage of that tile, a fixed prologue/epilogue,
+// and for more than one range the partial sums written and read back at about 4.5 TB/s plus the
+// second launch.  Big problems (192 or more of the largest tiles) take the largest tile as is.
+// The time per stage is a fit to measured loops of the five tile shapes: per 16-k sub-step about
+// 14 cycles per MFMA plus 5 per decode instruction, 400 cycles per stage on top, at 2.1 GHz.
+static TilePlan tile_plan(int64_t M, int64_t N, int64_t K, bool allow_split) {
+  TilePlan best{M <= 128 ? 2 : 4, 4, 1, 0};
+  if (const char *e = getenv("AC4K_TILE_PLAN")) {  // tuning aid: "mi,nj,splits"
+    int mi = 0, nj = 0, sp = 0;
+    if (sscanf(e, "%d,%d,%d", &mi, &nj, &sp) == 3 && (mi == 2 || mi == 4) && (nj == 1 || nj == 2 || nj == 4) &&
+        !(mi == 4 && nj == 1) && sp >= 1 && sp <= K / P_BK && (sp == 1 || allow_split))
+      return TilePlan{mi, nj, sp, sp > 1 ? (int64_t)sp * M * N * 4 : 0};
+  }
+  const int64_t stages = K / P_BK;
+  if (ceil_div(M, 64 * best.mi) * ceil_div(N, 256) >= 192) return best;
+  double best_t = 0.0;
+  bool first = true;
+  for (int mi = 2; mi <= 4; mi += 2) {
+    if (mi == 4 && M <= 128) continue;
+    for (int nj = 4; nj >= 1; nj >>= 1) {
+      if (mi == 4 && nj == 1) continue;  // not instantiated
+      if (nj < 4 && N < 64 * nj * 2) continue;
+      const int nm = mi * nj, nv = 8 * (mi + nj);
+      const double stage_us = (8.0 * (14.0 * nm + 5.0 * nv) + 400.0) / 2100.0;
+      const double fixed_us = 5.0 + 0.1 * nm;
+      const int64_t tiles = ceil_div(M, 64 * mi) * ceil_div(N, 64 * nj);
+      for (int64_t sp = 1; sp <= 32 && (sp == 1 || (allow_split && sp * 2 <= stages)); ++sp) {
+        const double rounds = (double)ceil_div(tiles * sp, 256);
+        double t = rounds * (double)ceil_div(stages, sp) * stage_us + fixed_us;
+        if (sp > 1) t += (double)sp * (double)(M * N) * 8.0 / 4.5e6 + 2.5;
+        if (first || t < best_t) {
+          first = false;
+          best_t = t;
+          best = TilePlan{mi, nj, (int)sp, sp > 1 ? sp * M * N * 4 : 0};
+        }
+      }
+    }
+  }
+  return best;
+}
+
+template <int D_DT, int BIAS_DT>
+static int launch_tile_plan(const LinearArgs &a, const TilePlan &p, const SplitK &sk, hipStream_t st) {
+  if (p.mi == 4) return p.nj == 4 ? launch_tile_p<D_DT, BIAS_DT, 4, 4>(a, sk, st) : launch_tile_p<D_DT, BIAS_DT, 4, 2>(a, sk, st);
+  if (p.nj == 4) return launch_tile_p<D_DT, BIAS_DT, 2, 4>(a, sk, st);
+  return p.nj == 2 ? launch_tile_p<D_DT, BIAS_DT, 2, 2>(a, sk, st) : launch_tile_p<D_DT, BIAS_DT, 2, 1>(a, sk, st);
+}
+
+// the packed-LDS kernel with the tile that suits the shape; no split-K (one K range, output to D)
 template <int D_DT, int BIAS_DT>
 static int launch_tile256p(const LinearArgs &a, hipStream_t st) {
   const SplitK one{nullptr, 1};
-  return a.M <= 128 ? launch_tile256p_mi<D_DT, BIAS_DT, 2>(a, one, st) : launch_tile256p_mi<D_DT, BIAS_DT, 4>(a, one, st);
+  return launch_tile_plan<D_DT, BIAS_DT>(a, tile_plan(a.M, a.N, a.K, false), one, st);
 }
 
 constexpr int L_LDS_BYTES = 2 * 2 * L_TILE_HALVES * (int)sizeof(_Float16);  // 128 KiB
@@ -1115,17 +1173,38 @@ __global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) 
       S[t][1] = sp[(int64_t)(t * 4 + 1) * a.Np];
     }
   }
-  // activation slice -> LDS as its exact fp16 dequantization (without the global scale)
+  // activation slice -> LDS as its exact fp16 dequantization (without the global scale).  A thread
+  // takes 32 elements (16 packed bytes, two 16-blocks) at a time; every load of the slice is issued
+  // before the first decode, so the slice costs one memory latency whatever M is.
   {
-    const int vec_per_row = a.ks_len / 8;  // 16-byte vectors (8 elements) per row
+    constexpr int MAX_IT = 32 * (1024 / 32) / 256;  // M <= 32, slices of at most 1024 k
+    const int vec_per_row = a.ks_len / 32;
     const int total = (int)a.M * vec_per_row;
-    for (int i = tid; i < total; i += 256) {
-      const int m = i / vec_per_row, v = i % vec_per_row;
-      const int64_t k = kbeg + v * 8;
-      const uint32_t w = *reinterpret_cast<const uint32_t *>(a.Aq + (int64_t)m * (a.K >> 1) + (k >> 1));
-      const uint32_t code = a.A_sf[(((k >> 6) * a.Mp + m) << 2) + ((k >> 4) & 3)];
-      const f16x8 d = decode_dword<false>(w, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(code, 1.0f, false));
-      *reinterpret_cast<f16x8 *>(slds + m * pitch + v * 16) = d;
+    uint4 aw[MAX_IT];
+    uint32_t ac[MAX_IT];
+#pragma unroll
+    for (int it = 0; it < MAX_IT; ++it) {
+      const int i = it * 256 + tid;
+      if (i < total) {
+        const int m = i / vec_per_row, v = i % vec_per_row;
+        const int64_t k = kbeg + v * 32;
+        aw[it] = *reinterpret_cast<const uint4 *>(a.Aq + (int64_t)m * (a.K >> 1) + (k >> 1));
+        // scale bytes of blocks (k/16) % 4 and the next one: k % 32 == 0, so an aligned pair
+        ac[it] = *reinterpret_cast<const uint16_t *>(a.A_sf + (((k >> 6) * a.Mp + m) << 2) + ((k >> 4) & 3));
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < MAX_IT; ++it) {
+      const int i = it * 256 + tid;
+      if (i < total) {
+        const int m = i / vec_per_row, v = i % vec_per_row;
+        const f16x2 sc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(ac[it], 1.0f, false);
+        f16x8 *dst = reinterpret_cast<f16x8 *>(slds + m * pitch + v * 64);
+        dst[0] = decode_dword<false>(aw[it].x, sc);
+        dst[1] = decode_dword<false>(aw[it].y, sc);
+        dst[2] = decode_dword<true>(aw[it].z, sc);
+        dst[3] = decode_dword<true>(aw[it].w, sc);
+      }
     }
   }
   __syncthreads();
@@ -1196,17 +1275,69 @@ __global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) 
   }
 }
 
-// D[m, n] = cvt( (sum over K-slices of partial[s][m][n]) * gsA*gsB + bias[n] ), slices added in order
-template <int D_DT, int BIAS_DT>
+// D[m, n] = cvt( (sum over K-slices of partial[s][m][n]) * gsA*gsB + bias[n] ), slices added in order.
+// V outputs per thread (V = 4: 16-byte loads; needs N % 4 == 0); the loads of eight slices are in
+// flight together, the additions stay in slice order.
+template <int D_DT, int BIAS_DT, int V>
 __global__ __launch_bounds__(256) void skinny_reduce_kernel(SkinnyArgs a) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
   const int64_t total = a.M * a.N;
   if (i >= total) return;
-  float v = 0.0f;
-  for (int sidx = 0; sidx < a.split_k; ++sidx) v += a.partial[(int64_t)sidx * total + i];
-  v *= (*a.A_gs) * (*a.B_gs);
-  if constexpr (BIAS_DT != BIAS_NONE) v += Elem<BIAS_DT>::load(a.bias, i % a.N);
-  static_cast<typename Elem<D_DT>::T *>(a.D)[i] = Elem<D_DT>::cvt(v);
+  float v[V];
+#pragma unroll
+  for (int q = 0; q < V; ++q) v[q] = 0.0f;
+  const float *p = a.partial + i;
+  int sidx = 0;
+  for (; sidx + 8 <= a.split_k; sidx += 8) {
+    float t[8][V];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if constexpr (V == 4) {
+        const float4 f = *reinterpret_cast<const float4 *>(p + (int64_t)(sidx + u) * total);
+        t[u][0] = f.x; t[u][1] = f.y; t[u][2] = f.z; t[u][3] = f.w;
+      } else {
+        t[u][0] = p[(int64_t)(sidx + u) * total];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int q = 0; q < V; ++q) v[q] += t[u][q];
+  }
+  for (; sidx < a.split_k; ++sidx) {
+    if constexpr (V == 4) {
+      const float4 f = *reinterpret_cast<const float4 *>(p + (int64_t)sidx * total);
+      v[0] += f.x; v[1] += f.y; v[2] += f.z; v[3] += f.w;
+    } else {
+      v[0] += p[(int64_t)sidx * total];
+    }
+  }
+  const float scale = (*a.A_gs) * (*a.B_gs);
+  using DE = Elem<D_DT>;
+  typename DE::T *D = static_cast<typename DE::T *>(a.D);
+  const int64_t n = i % a.N;  // V consecutive outputs share a row (N % V == 0)
+#pragma unroll
+  for (int q = 0; q < V; ++q) {
+    v[q] *= scale;
+    if constexpr (BIAS_DT != BIAS_NONE) v[q] += Elem<BIAS_DT>::load(a.bias, n + q);
+  }
+  if constexpr (V == 4 && sizeof(typename DE::T) == 2) {
+    *reinterpret_cast<uint2 *>(D + i) = make_uint2(DE::cvt2(v[0], v[1]), DE::cvt2(v[2], v[3]));
+  } else if constexpr (V == 4) {
+    *reinterpret_cast<float4 *>(D + i) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+    D[i] = DE::cvt(v[0]);
+  }
+}
+
+template <int D_DT, int BIAS_DT>
+static void launch_reduce(const SkinnyArgs &a, hipStream_t st) {
+  const int64_t total = a.M * a.N;
+  const bool v4 = a.N % 4 == 0 && ((uintptr_t)a.D & 15) == 0 && ((uintptr_t)a.partial & 15) == 0;
+  if (v4)
+    hipLaunchKernelGGL((skinny_reduce_kernel<D_DT, BIAS_DT, 4>), dim3((unsigned)ceil_div(total / 4, 256)), dim3(256), 0, st, a);
+  else
+    hipLaunchKernelGGL((skinny_reduce_kernel<D_DT, BIAS_DT, 1>), dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, a);
 }
 
 struct SkinnyPlan {
@@ -1236,8 +1367,7 @@ static int launch_skinny(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_t s
   static std::atomic<uint32_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, lds_ok, 32 * (1024 * 2 + 16))) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)p.split_k, (unsigned)p.groups), dim3(256), p.lds_bytes, st, a);
-  if (p.split_k > 1)
-    hipLaunchKernelGGL((skinny_reduce_kernel<D_DT, BIAS_DT>), dim3((unsigned)ceil_div(a.M * a.N, 256)), dim3(256), 0, st, a);
+  if (p.split_k > 1) launch_reduce<D_DT, BIAS_DT>(a, st);
   return 0;
 }
 
@@ -1344,50 +1474,25 @@ namespace ac4k {
 // Split-K for problems with too few output tiles to fill the GPU (32 < M, few tiles, long K):
 // the packed-LDS kernel runs `splits` K ranges per tile into fp32 partial buffers in the
 // workspace and skinny_reduce_kernel adds them.
-struct MidPlan {
-  int splits;
-  int64_t partial_bytes;
-};
-
-static bool mid_plan(int64_t M, int64_t N, int64_t K, MidPlan &p) {
-  if (M <= 32 || N < 128 || K % P_BK != 0 || (K >> 1) * 256 >= (1ll << 31)) return false;
-  const bool small = M <= 128;
-  const int64_t tiles = ceil_div(M, small ? 128 : 256) * ceil_div(N, P_BN);
-  const int64_t stages = K / P_BK;
-  if (tiles >= 192) return false;
-  // Rough cost in microseconds of running `s` K ranges per tile on 256 CUs: rounds of
-  // workgroups x stages per range x time per stage, fixed prologue/epilogue, and for s > 1 the
-  // partial sums written and read back at about 3 TB/s plus the second launch.
-  const double stage_us = small ? 1.45 : 2.9;
-  double best = 0.0;
-  int64_t best_s = 1;
-  for (int64_t s = 1; s <= 32 && s * 2 <= stages; ++s) {
-    const double rounds = (double)ceil_div(tiles * s, 256);
-    double t = rounds * (double)ceil_div(stages, s) * stage_us + 6.0;
-    if (s > 1) t += (double)s * (double)(M * N) * 8.0 / 3.0e6 + 4.0;
-    if (s == 1 || t < best) {
-      best = t;
-      best_s = s;
-    }
-  }
-  if (best_s < 2) return false;
-  p.splits = (int)best_s;
-  p.partial_bytes = best_s * M * N * 4;
-  return true;
+// shapes the workspace entry point splits along K: the packed-LDS kernel's shapes for which the
+// plan wants more than one K range
+static bool mid_plan(int64_t M, int64_t N, int64_t K, TilePlan &p) {
+  if (M <= 32 || N < 128 || K % P_BK != 0 || (K >> 1) * 256 >= (1ll << 31) || N >= (1ll << 27)) return false;
+  p = tile_plan(M, N, K, true);
+  return p.splits > 1;
 }
 
 template <int D_DT, int BIAS_DT>
-static int launch_mid(const LinearArgs &a, const MidPlan &p, float *partial, hipStream_t st) {
+static int launch_mid(const LinearArgs &a, const TilePlan &p, float *partial, hipStream_t st) {
   const SplitK sk{partial, p.splits};
-  const int rc = a.M <= 128 ? launch_tile256p_mi<D_DT, BIAS_DT, 2>(a, sk, st) : launch_tile256p_mi<D_DT, BIAS_DT, 4>(a, sk, st);
-  if (rc) return rc;
+  if (int rc = launch_tile_plan<D_DT, BIAS_DT>(a, p, sk, st)) return rc;
   SkinnyArgs r{a.D, nullptr, nullptr, 0, nullptr, nullptr, a.A_gs, a.B_gs, a.bias, partial, a.M, a.N, a.K, a.Np, 0, p.splits};
-  hipLaunchKernelGGL((skinny_reduce_kernel<D_DT, BIAS_DT>), dim3((unsigned)ceil_div(a.M * a.N, 256)), dim3(256), 0, st, r);
+  launch_reduce<D_DT, BIAS_DT>(r, st);
   return 0;
 }
 
 template <int D_DT>
-static int dispatch_mid_bias(const LinearArgs &a, const MidPlan &p, float *partial, int bias_dtype, hipStream_t st) {
+static int dispatch_mid_bias(const LinearArgs &a, const TilePlan &p, float *partial, int bias_dtype, hipStream_t st) {
   if (!a.bias) return launch_mid<D_DT, BIAS_NONE>(a, p, partial, st);
   switch (bias_dtype) {
     case AC4K_DTYPE_BF16: return launch_mid<D_DT, AC4K_DTYPE_BF16>(a, p, partial, st);
@@ -1397,7 +1502,7 @@ static int dispatch_mid_bias(const LinearArgs &a, const MidPlan &p, float *parti
   return set_error("bias must be bfloat16, half or float (dtype tag %d)", bias_dtype);
 }
 
-static int dispatch_mid(const LinearArgs &a, const MidPlan &p, float *partial, int d_dtype, int bias_dtype,
+static int dispatch_mid(const LinearArgs &a, const TilePlan &p, float *partial, int d_dtype, int bias_dtype,
                         hipStream_t st) {
   switch (d_dtype) {
     case AC4K_DTYPE_BF16: return dispatch_mid_bias<AC4K_DTYPE_BF16>(a, p, partial, bias_dtype, st);
@@ -1443,7 +1548,7 @@ static int check_skinny(const SkinnyPlan &p, bool ok, const void *B, void *works
 extern "C" __attribute__((visibility("default"))) int64_t ac4k_linear_nvfp4_skinny_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   SkinnyPlan p;
   if (skinny_plan(M, N, K, p)) return p.partial_bytes > 0 ? p.partial_bytes : 256;  // non-zero selects this path
-  MidPlan mp;
+  TilePlan mp;
   if (mid_plan(M, N, K, mp)) return mp.partial_bytes;
   return 0;
 }
@@ -1454,7 +1559,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_skinny(v
                                         int64_t workspace_bytes, ac4k_stream_t stream) {
   AC4K_REQUIRE(D && A && A_sf && A_gs && B && B_sf && B_gs, "null pointer argument");
   hipStream_t st = (hipStream_t)stream;
-  MidPlan mp;
+  TilePlan mp;
   if (M > 32 && mid_plan(M, N, K, mp)) {  // few tiles, long K: split-K over the tile kernel
     AC4K_REQUIRE((((uintptr_t)A | (uintptr_t)B) & 15) == 0, "A and B must be 16-byte aligned");
     AC4K_REQUIRE(workspace && ((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
@@ -1469,7 +1574,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_skinny(v
   SkinnyPlan p;
   const bool ok = skinny_plan(M, N, K, p);
   if (int rc = check_skinny(p, ok, B, workspace, workspace_bytes)) return rc;
-  AC4K_REQUIRE(((uintptr_t)A & 3) == 0, "A must be 4-byte aligned");
+  AC4K_REQUIRE(((uintptr_t)A & 15) == 0, "A must be 16-byte aligned");
   if (int rc = run_skinny(D, d_dtype, A, A_sf, A_gs, B, B_sf, B_gs, bias, bias_dtype, M, N, K, p, workspace, st))
     return rc;
   return check_launch("ac4k_linear_nvfp4_skinny");

@@ -191,6 +191,23 @@ def test_mid_m_shapes(m, n, k):
         run_case(m, n, k, bias_dtype=torch.bfloat16, o_dtype=torch.float32, seed=m + k + 2, wstd=0.02)
 
 
+# every tile shape of the packed-LDS kernel (64*mi rows x 64*nj columns, its own LDS stage depth),
+# alone and split along K, forced through the library's tuning variable; ragged M and N included
+TILE_PLANS = [(2, 1, 1), (2, 2, 1), (2, 4, 1), (4, 2, 1), (4, 4, 1), (2, 1, 3), (2, 2, 2), (2, 4, 5), (4, 2, 2), (4, 4, 4)]
+
+
+@pytest.mark.parametrize("mi,nj,splits", TILE_PLANS)
+def test_tile_plans(mi, nj, splits, monkeypatch):
+    monkeypatch.setenv("AC4K_TILE_PLAN", f"{mi},{nj},{splits}")
+    for (m, n, k) in [(64 * mi, 128 * nj, 1280), (64 * mi + 37, 64 * nj * 3 - 10, 1536), (33, 136, 2048)]:
+        run_case(m, n, k, seed=mi * 100 + nj * 10 + splits, wstd=0.02)
+        run_case(m, n, k, bias_dtype=torch.bfloat16, o_dtype=torch.float32, seed=m + n, wstd=0.02)
+        run_case(m, n, k, bias_dtype=torch.float32, o_dtype=torch.float16, seed=m + n + 1, wstd=0.02)
+    # K of one and of two stages: shorter than the stage ring
+    run_case(96, 256, 128, seed=3)
+    run_case(96, 256, 256, bias_dtype=torch.float16, seed=4)
+
+
 def test_mid_m_workspace_entry_matches_plain_entry():
     """The workspace-assisted entry point and ac4k_linear_nvfp4 compute the same contract; with fp32
     output they agree to accumulation-order noise."""
