@@ -552,57 +552,55 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Tiny dense tensors (at most NV * 1024 vectors of 8 elements): one workgroup holds everything in
-// registers, so global scale and quantize are one launch with an ordinary
-// workgroup barrier in between.
-template <int NV>
-__global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_single_wg_kernel(
+// Small dense tensors (at most NSEG segments of 1024 16-byte vectors, 16 KB each): one launch, no
+// grid wait.  Workgroup b quantizes segment b; for the global scale every workgroup reads the
+// whole tensor itself (all loads in flight at once; after the first workgroup they are cache hits),
+// so nothing has to be exchanged between workgroups.
+template <int NSEG>
+__global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_small_kernel(
     uint32_t *__restrict__ out, uint32_t *__restrict__ sf, const uint4 *__restrict__ in, float *__restrict__ gs_out,
     OnePassGeom g, float max_scale) {
   __shared__ float lut[128];
   __shared__ uint32_t red[OP_THREADS / 64];
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t nvec = g.total_chunks * 8;
-  uint4 v[NV];
+  const uint32_t lv = blockIdx.x * OP_THREADS + tid;  // this lane's vector of the workgroup's own segment
+  uint4 own = make_uint4(0, 0, 0, 0);
+  if (lv < nvec) own = in[lv];
+  uint4 v[NSEG];
 #pragma unroll
-  for (int j = 0; j < NV; ++j) {
-    const uint32_t lv = j * OP_THREADS + tid;
+  for (int j = 0; j < NSEG; ++j) {
+    const uint32_t ov = j * OP_THREADS + tid;
     v[j] = make_uint4(0, 0, 0, 0);
-    if (lv < nvec) v[j] = in[lv];
+    if (ov < nvec) v[j] = in[ov];
   }
   if (tid < 128) lut[tid] = g_rcp_e4m3.v[tid];
-  uint32_t bm[NV], m = 0;
+  uint32_t m = 0;
 #pragma unroll
-  for (int j = 0; j < NV; ++j) {
-    bm[j] = absmax_bf16x8(v[j]);
-    bm[j] = umax32(bm[j], dpp_u32<DPP_QUAD_XOR1>(bm[j]));
-    m = umax32(m, bm[j]);
-  }
+  for (int j = 0; j < NSEG; ++j) m = umax32(m, absmax_bf16x8(v[j]));
   m = group_umax<64>(m);
   if (lane == 0) red[wave] = m;
   __syncthreads();
   const uint32_t gm = group_umax<16>(red[lane & 15]);
   const float gs = bf16_bits_to_f32(gm) / max_scale;
-  if (tid == 0) *gs_out = gs;
+  if (blockIdx.x == 0 && tid == 0) *gs_out = gs;
   const float alpha = 1.0f / gs;
-#pragma unroll
-  for (int j = 0; j < NV; ++j) {
-    const uint32_t lv = j * OP_THREADS + tid;
-    uint32_t code;
-    const float o = nvfp4_block_scale(bf16_bits_to_f32(bm[j]), alpha, lut, code);
-    const uint32_t packed = nvfp4_pack8(v[j], o);
-    const uint32_t sfw = code | (dpp_u32<DPP_ROW_SHL(2)>(code) << 8) | (dpp_u32<DPP_ROW_SHL(4)>(code) << 16) |
-                         (dpp_u32<DPP_ROW_SHL(6)>(code) << 24);
-    if (lv < nvec) {
-      out[lv] = packed;
-      if ((lane & 7) == 0) {
-        const uint32_t ch = lv >> 3, row = ch / g.ncc, cc = ch - row * g.ncc;
-        const uint32_t l = g.lead > 1 ? row / g.R : 0u, r = row - l * g.R;
-        sf[((uint64_t)l * g.ncc + cc) * g.Rp + r] = sfw;
-      }
+  uint32_t bm = absmax_bf16x8(own);
+  bm = umax32(bm, dpp_u32<DPP_QUAD_XOR1>(bm));
+  uint32_t code;
+  const float o = nvfp4_block_scale(bf16_bits_to_f32(bm), alpha, lut, code);
+  const uint32_t packed = nvfp4_pack8(own, o);
+  const uint32_t sfw = code | (dpp_u32<DPP_ROW_SHL(2)>(code) << 8) | (dpp_u32<DPP_ROW_SHL(4)>(code) << 16) |
+                       (dpp_u32<DPP_ROW_SHL(6)>(code) << 24);
+  if (lv < nvec) {
+    out[lv] = packed;
+    if ((lane & 7) == 0) {
+      const uint32_t ch = lv >> 3, row = ch / g.ncc, cc = ch - row * g.ncc;
+      const uint32_t l = g.lead > 1 ? row / g.R : 0u, r = row - l * g.R;
+      sf[((uint64_t)l * g.ncc + cc) * g.Rp + r] = sfw;
     }
   }
-  if (g.Rp > g.R) {  // zero scales of the pad rows R..Rp-1
+  if (g.Rp > g.R && blockIdx.x == 0) {  // zero scales of the pad rows R..Rp-1
     const uint32_t pad = g.Rp - g.R, npad = g.lead * g.ncc * pad;
     for (uint32_t i = tid; i < npad; i += OP_THREADS) sf[(uint64_t)(i / pad) * g.Rp + g.R + i % pad] = 0u;
   }
@@ -1100,17 +1098,19 @@ static void launch_onepass(uint32_t *out, uint32_t *sf, const uint4 *in, float *
                      g, slot, max_scale, ticks);
 }
 
-// One workgroup streams at a few tens of GB/s, so this only pays for tensors of a few KB: above two
-// 16 KB segments the two-launch paths are faster.
-constexpr int SINGLE_WG_MAX_SEGS = 2;
+// Up to 16 segments (256 KB) every workgroup can afford to read the whole tensor for its maximum:
+// one launch of a few microseconds, against two launches and a grid wait.
+constexpr int SMALL_MAX_SEGS = 16;
 
-static void launch_single_wg(uint32_t *out, uint32_t *sf, const uint4 *in, float *gs, const OnePassGeom &g,
-                             float max_scale, hipStream_t st) {
-  static_assert(SINGLE_WG_MAX_SEGS == 2, "instantiations below");
-  if (g.total_chunks <= 128)  // one 1024-vector segment
-    hipLaunchKernelGGL(quantize_nvfp4_single_wg_kernel<1>, dim3(1), dim3(OP_THREADS), 0, st, out, sf, in, gs, g, max_scale);
-  else
-    hipLaunchKernelGGL(quantize_nvfp4_single_wg_kernel<2>, dim3(1), dim3(OP_THREADS), 0, st, out, sf, in, gs, g, max_scale);
+static void launch_small(uint32_t *out, uint32_t *sf, const uint4 *in, float *gs, const OnePassGeom &g,
+                         float max_scale, hipStream_t st) {
+  const unsigned nseg = (unsigned)ceil_div((int64_t)g.total_chunks, 128);
+  const dim3 grid(nseg), block(OP_THREADS);
+  if (nseg <= 1) hipLaunchKernelGGL(quantize_nvfp4_small_kernel<1>, grid, block, 0, st, out, sf, in, gs, g, max_scale);
+  else if (nseg <= 2) hipLaunchKernelGGL(quantize_nvfp4_small_kernel<2>, grid, block, 0, st, out, sf, in, gs, g, max_scale);
+  else if (nseg <= 4) hipLaunchKernelGGL(quantize_nvfp4_small_kernel<4>, grid, block, 0, st, out, sf, in, gs, g, max_scale);
+  else if (nseg <= 8) hipLaunchKernelGGL(quantize_nvfp4_small_kernel<8>, grid, block, 0, st, out, sf, in, gs, g, max_scale);
+  else hipLaunchKernelGGL(quantize_nvfp4_small_kernel<16>, grid, block, 0, st, out, sf, in, gs, g, max_scale);
 }
 
 // Global scale + nvfp4 quantize of a dense [lead, R, K] tensor in one pass over the input, when
@@ -1128,9 +1128,9 @@ static bool try_quantize_nvfp4_onepass(void *out, void *sf, float *gs, const voi
   if (nwg > OP_MAX_WGS) nwg = OP_MAX_WGS;
   if (nwg < 8 || chunks > (int64_t)nwg * 128 * OP_MAX_NV) return false;
   const OnePassGeom g{(uint32_t)chunks, (uint32_t)(K / 64), (uint32_t)R, (uint32_t)align_up(R, 16), (uint32_t)lead};
-  if (chunks <= 128 * SINGLE_WG_MAX_SEGS) {  // tiny: one workgroup, one launch, no grid wait
-    launch_single_wg(static_cast<uint32_t *>(out), static_cast<uint32_t *>(sf), static_cast<const uint4 *>(in), gs, g,
-                     max_scale, st);
+  if (chunks <= 128 * SMALL_MAX_SEGS) {  // small: one launch, no grid wait
+    launch_small(static_cast<uint32_t *>(out), static_cast<uint32_t *>(sf), static_cast<const uint4 *>(in), gs, g,
+                 max_scale, st);
     return true;
   }
   const int slot = amax_slot(st);
