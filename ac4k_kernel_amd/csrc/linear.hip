@@ -879,8 +879,12 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-      for (int j = 0; j < NJ; ++j)
+      for (int jj = 0; jj < NJ; ++jj) {
+        // boustrophedon order: every MFMA shares one operand with the one before it (measured 0.6 %
+        // faster than row by row on the power-limited 8192^3 problem: less operand switching)
+        const int j = (i & 1) ? NJ - 1 - jj : jj;
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(d.b[j], d.a[i], acc[i][j], 0, 0, 0);  // D^T block
+      }
   };
   auto interleave = [&]() {  // the decode of the next sub-step rides in the shadow of the MFMAs
     constexpr int NMFMA = MI * NJ, NVALU = 8 * (MI + NJ);
