@@ -64,13 +64,14 @@ int ac4k_quantize_nvfp4(void *out, void *sf, const void *in, const float *global
 
 /* The nvfp4 branch of Ac4kQuantizeOp.forward in one call
  * (python/ac4k_kernel/ops/quant.py:187-242): *global_scale = max|in| / max_scale over the whole
- * (contiguous) input, then ac4k_quantize_nvfp4 with it.  Two launches, nothing to initialise, no host synchronisation. */
+ * (contiguous) input, then ac4k_quantize_nvfp4 with it.  One launch for dense tensors of up to
+ * 256 KB, else two; nothing to initialise, no host synchronisation. */
 int ac4k_quantize_nvfp4_bf16(void *out, void *sf, float *global_scale, const void *in, int64_t d0,
                              int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
                              int64_t sK, int swizzle, float max_scale, ac4k_stream_t stream);
 
-/* Tuning knob of ac4k_quantize_nvfp4_bf16 (no counterpart in the reference).  Dense tensors of up to
- * 64 MiB are quantized in one pass over the input by a kernel whose workgroups wait for each other;
+/* Tuning knob of ac4k_quantize_nvfp4_bf16 (no counterpart in the reference).  Dense tensors between
+ * 256 KB and 64 MiB are quantized in one pass over the input by a kernel whose workgroups wait for each other;
  * the wait is bounded by this many microseconds (default 200), after which the workgroups that gave
  * up are redone by a second launch that is always enqueued behind the first.  0 sends every workgroup
  * down that second path (used by the tests); a negative value selects the two-kernel quantizer. */
@@ -102,9 +103,10 @@ int ac4k_linear_nvfp4(void *D, int d_dtype, const void *A, const void *A_sf, con
  * (lib/cuda/sm120/linear_nvfp4.cu:753-901; the reference runs every shape through its one
  * 128x128 tile kernel).  Two families:
  *   - decode-sized, 1 <= M <= 32 and K % 256 == 0: a weight-streaming split-K kernel; the
- *     workspace receives the fp32 partial sums of the K-slices;
+ *     workspace receives the fp32 partial sums of the K-slices; A and B 16-byte aligned;
  *   - 32 < M with too few output tiles to fill the GPU and K % 128 == 0: split-K over the tile
- *     kernel; the workspace receives the fp32 partial sums.
+ *     kernel (tile shape and number of K ranges chosen by a cost model); the workspace receives
+ *     the fp32 partial sums; A and B 16-byte aligned.
  * `workspace` = ac4k_linear_nvfp4_skinny_workspace_bytes(M,N,K) bytes of device memory, 256-byte
  * aligned, contents irrelevant.  The size function returns 0 for shapes that gain nothing from
  * scratch; those go to ac4k_linear_nvfp4. */
