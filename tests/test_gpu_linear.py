@@ -132,18 +132,36 @@ def test_size_independent_properties(m, n, k):
     assert torch.equal(d3, d1[perm])
 
 
-@pytest.mark.parametrize("m", [1, 8, 32])
-def test_fused_skinny_equals_composition(m):
-    n, k = 1024, 2048
+# K = 256 is one K slice (no reduce kernel), 14336 is 28 of them; N = 130 leaves a ragged row group.
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8, 32])
+@pytest.mark.parametrize("n,k", [(1024, 2048), (130, 256), (384, 14336)])
+def test_fused_skinny_equals_composition(m, n, k):
     x = make_input((m, k), seed=m, outliers=True).cuda()
     wq = gpu_quant(make_input((n, k), seed=50, std=0.02))
-    d, (xq, xsf, xgs) = ops().fused_linear(x, *wq, return_quantized=True)
+    bias = make_input((1, n), seed=7).to(torch.float32).cuda()
+    d, (xq, xsf, xgs) = ops().fused_linear(x, *wq, bias=bias, return_quantized=True)
     eq, esf, egs = T.quantize_nvfp4(x.cpu(), 0, 1)
     assert torch.equal(xq.cpu(), eq) and torch.equal(xsf.cpu().view(torch.uint8), esf) and xgs.item() == egs.item()
-    ref = T.linear_nvfp4(eq, esf, egs, *cpu(wq))
+    ref = T.linear_nvfp4(eq, esf, egs, *cpu(wq), bias=bias.cpu())
     torch.testing.assert_close(d.cpu(), ref, atol=ATOL, rtol=RTOL)
-    comp = ops().linear(*ops().quantize(x, 0, 1), *wq)
-    torch.testing.assert_close(d, comp, atol=ATOL, rtol=RTOL)
+    comp = ops().linear(*ops().quantize(x, 0, 1), *wq, bias=bias)
+    assert torch.equal(d, comp)  # same packed activation, same kernel arithmetic, same slice order
+
+
+def test_fused_skinny_edge_activations():
+    """Blocks of zeros, a negative zero, one huge outlier and a whole row of zeros through the fused
+    entry point: bytes, scales and global scale equal the oracle's."""
+    n, k = 256, 1024
+    x = make_input((3, k), seed=9)
+    x[0, 64:96] = 0.0
+    x[0, 70] = -0.0
+    x[1, :] = 0.0
+    x[2, 5] = 3000.0
+    wq = gpu_quant(make_input((n, k), seed=52, std=0.02))
+    d, (xq, xsf, xgs) = ops().fused_linear(x.cuda(), *wq, return_quantized=True)
+    eq, esf, egs = T.quantize_nvfp4(x, 0, 1)
+    assert torch.equal(xq.cpu(), eq) and torch.equal(xsf.cpu().view(torch.uint8), esf) and xgs.item() == egs.item()
+    torch.testing.assert_close(d.cpu(), T.linear_nvfp4(eq, esf, egs, *cpu(wq)), atol=ATOL, rtol=RTOL)
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 256, 256), (7, 300, 512), (16, 130, 768), (32, 1000, 1024), (32, 64, 4096),
