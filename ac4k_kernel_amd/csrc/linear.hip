@@ -8,7 +8,7 @@
 // gfx950's scaled MFMA takes power-of-two scales per 32 elements, not E4M3 per 16, so the
 // packed tiles are decoded on the fly: v_cvt_scalef32_pk_f16_fp4 expands two nibbles to two
 // fp16 values and one v_pk_mul_f16 applies the E4M3 block scale.  e2m1 * e4m3 has at most
-// 5 significant bits and lies in [2^-10, 2688], so the fp16 product is exact; the MFMA
+// 6 significant bits and lies in [2^-10, 2688], so the fp16 product is exact; the MFMA
 // (v_mfma_f32_32x32x16_f16, same rate as bf16) accumulates in fp32.
 #include <stdlib.h>
 #include <string.h>
@@ -480,20 +480,21 @@ __device__ __forceinline__ void decode_half_block(_Float16 *tile, int row, int h
 
 
 // ===========================================================================
-// BM x 256 tile (BM = 256 or 128), packed operands in LDS, decode after the fragment load.
+// (64 MI) x (64 NJ) tile, packed operands in LDS, decode after the fragment load.
 //
 // The packed A/B slices and their scale dwords go from global memory straight into LDS with
-// LDS-DMA loads (global_load_lds: no VGPR staging, no LDS store instruction), three stages of
-// 128 k each.  A wave (4 waves, 2x2, (BM/2)x128 each) reads for every 32-row fragment ONE
+// LDS-DMA loads (global_load_lds: no VGPR staging, no LDS store instruction), PS stages of
+// 128 k each.  A wave (4 waves, 2x2, (32 MI) x (32 NJ) each) reads for every 32-row fragment ONE
 // 16-byte word per lane per 64-chunk: lane (row r, half h) owns elements [32h, 32h+32) of the
 // chunk; dword s of that word feeds MFMA sub-step s.  The same k-slot assignment is used for A
 // and B, so the permutation of k inside a chunk cancels in the dot product.  Decode per dword:
 // 4 x v_cvt_scalef32_pk_f16_fp4 + 4 x v_pk_mul_f16 by the block scale (E4M3 -> fp16 with
 // v_cvt_scalef32_pk_f16_fp8, splat through op_sel); the decode of a sub-step is interleaved with
-// the MFMAs of the previous one.  A single wave issues roughly one VALU instruction per six
-// cycles, so the 4.6 VALU per MFMA of the 256-row tile stretch a 32-cycle MFMA slot to about 41
-// cycles; that, not LDS or HBM, bounds the loop.  There is one workgroup barrier per 128 k,
-// placed in the middle of the step so that the next stage is readable before the current one ends.
+// the MFMAs of the previous one.  A single wave per SIMD is bound by instruction issue: the
+// 4 decode instructions per MFMA of the 256x256 tile stretch a 32-cycle MFMA slot to about 38
+// cycles, the smaller tiles (more decode per MFMA) are decode-bound outright; that, not LDS or
+// HBM, bounds the loop.  There is one workgroup barrier per 128 k, placed in the middle of the
+// step so that the next stage is readable before the current one ends.
 // Split-K: blockIdx.y selects a contiguous range of stages; with more than one range the
 // accumulators go to an fp32 partial buffer and a second kernel adds the ranges.
 // Requires K % 128 == 0 and 16-byte aligned operands.
