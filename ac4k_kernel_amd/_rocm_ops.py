@@ -22,19 +22,21 @@ __version__ = _L.ac4k_version().decode()
 _DTYPE_TAG = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 
 
-def _check(cond: bool, msg: str) -> None:
+def _check(cond: bool, msg: str, *args) -> None:
+    """RuntimeError(msg.format(*args)) unless cond; the message is only built on failure."""
     if not cond:
-        raise RuntimeError(msg)
+        raise RuntimeError(msg.format(*args) if args else msg)
 
 
-def _check_tensor(t, dtype, name: str) -> None:
+def _check_tensor(t, dtype, name: str, suffix: str = "") -> None:
     # one combined test on the hot path; the individual messages are only built on failure
     if isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dtype and t.is_contiguous():
         return
-    _check(isinstance(t, torch.Tensor), f"{name} must be a tensor")
-    _check(t.is_cuda, f"{name} must be a CUDA tensor")
-    _check(t.is_contiguous(), f"{name} must be contiguous")
-    _check(t.dtype == dtype, f"Inconsistency of Tensor type: {name} must be {dtype}")
+    name += suffix
+    _check(isinstance(t, torch.Tensor), "{} must be a tensor", name)
+    _check(t.is_cuda, "{} must be a CUDA tensor", name)
+    _check(t.is_contiguous(), "{} must be contiguous", name)
+    _check(t.dtype == dtype, "Inconsistency of Tensor type: {} must be {}", name, dtype)
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -131,14 +133,14 @@ def quantize_int8(out, sf, inp, scale_max, cross_dim: int, reduce_dim: int) -> N
 
 
 def _check_linear_operand(x, x_sf, x_gs, rows, name):
-    _check(x.dim() == 2, f"{name} must be a 2d matrix")
+    _check(x.dim() == 2, "{} must be a 2d matrix", name)
     _check_tensor(x, torch.uint8, name)
     K = x.size(1) * 2
-    _check(x_sf.dim() == 3, f"scale_{name} must be a 3d matrix")
-    _check_tensor(x_sf, torch.float8_e4m3fn, f"scale_{name}")
-    _check(list(x_sf.shape) == [(K + 63) // 64, _align_up(rows, 16), 4], f"scale_{name} has an invalid shape")
-    _check_tensor(x_gs, torch.float32, f"global_scale_{name}")
-    _check(x_gs.dim() == 0, f"{name}_global_scale must be a scalar")
+    _check(x_sf.dim() == 3, "scale_{} must be a 3d matrix", name)
+    _check_tensor(x_sf, torch.float8_e4m3fn, "scale_", name)
+    _check(x_sf.shape == ((K + 63) // 64, _align_up(rows, 16), 4), "scale_{} has an invalid shape", name)
+    _check_tensor(x_gs, torch.float32, "global_scale_", name)
+    _check(x_gs.dim() == 0, "{}_global_scale must be a scalar", name)
     return K
 
 
@@ -157,7 +159,7 @@ def _bias_args(bias, N):
     _check(bias.is_cuda and bias.is_contiguous(), "bias must be contiguous")
     _check(bias.dim() == 2, "bias must be a 2d matrix")
     _check(bias.size(0) == 1, "bias shape[0] must be 1")
-    _check(bias.size(1) == N, f"bias shape[1] must be {N}")
+    _check(bias.size(1) == N, "bias shape[1] must be {}", N)
     return bias.data_ptr(), _DTYPE_TAG[bias.dtype]
 
 
@@ -169,11 +171,11 @@ def linear_nvfp4(D, A, A_sf, A_global_scale, B, B_sf, B_global_scale, bias=None)
     _check(D.dtype in _DTYPE_TAG, "d must be bfloat16, half or float")
     _check(D.is_cuda and D.is_contiguous(), "d must be contiguous")
     M, N = D.shape
-    _check(A.dim() == 2 and A.size(0) == M, f"A size(0) must be {M}")
+    _check(A.dim() == 2 and A.size(0) == M, "A size(0) must be {}", M)
     K = _check_linear_operand(A, A_sf, A_global_scale, M, "a")
-    _check(K % 16 == 0, f"A size(1)*2 must be multiple of 16 but see {K}")
+    _check(K % 16 == 0, "A size(1)*2 must be multiple of 16 but see {}", K)
     _check(B.dim() == 2 and B.size(1) == A.size(1), "B size(1) must equal A size(1)")
-    _check(B.size(0) == N, f"B size(0) must be {N}")
+    _check(B.size(0) == N, "B size(0) must be {}", N)
     _check_linear_operand(B, B_sf, B_global_scale, N, "b")
     bias_ptr, bias_tag = _bias_args(bias, N)
     if M == 0 or N == 0:
@@ -199,7 +201,7 @@ def linear_nvfp4_fused(D, X, X_q, X_sf, X_global_scale, B, B_sf, B_global_scale,
     _check(D.is_cuda and D.is_contiguous(), "d must be contiguous")
     M, N = D.shape
     _check_tensor(X, torch.bfloat16, "x")
-    _check(X.dim() == 2 and X.size(0) == M, f"x must be [{M}, K]")
+    _check(X.dim() == 2 and X.size(0) == M, "x must be [{}, K]", M)
     _check(1 <= M <= 32, "the fused linear takes 1 <= M <= 32")
     K = X.size(1)
     _check(K % 64 == 0, "K must be a multiple of 64")
