@@ -197,19 +197,32 @@ def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True, key=None, wi
         got = out[rows]
         ok = bool(torch.all((got.float() - ref.float()).abs() <= 1e-2 + 1e-2 * ref.float().abs()).item())
         del ref
-    total, ms = time_gpu(lambda: ops.linear(*aq, *bq, out=out), steps, warmup)
+    # memory-bound shapes rotate over enough copies of the weight operand to exceed the 256 MB
+    # memory-side cache, so that the weights really come from HBM (as distinct layers' weights would)
+    t_flops0, t_bytes0 = 2.0 * m * n * k / (MFMA_PEAK_TFLOPS * 1e12), linear_bytes(m, n, k) / (HBM_PEAK_GBS * 1e9)
+    wbytes = bq[0].nbytes + bq[1].nbytes
+    ncopy = 1 if t_flops0 >= t_bytes0 else max(2, min(12, -(-320_000_000 // wbytes)))
+    bqs = [bq] + [tuple(t.clone() for t in bq) for _ in range(ncopy - 1)]
+    turn = [0]
+
+    def weights():
+        turn[0] += 1
+        return bqs[turn[0] % ncopy]
+
+    total, ms = time_gpu(lambda: ops.linear(*aq, *weights(), out=out), steps, warmup)
     ms_with_quantize = None
     if with_quantize:  # the activation quantized inside the timed region, the weights not
         xa = a.cuda()
-        _, ms_with_quantize = time_gpu(lambda: ops.linear(*ops.quantize(xa, 0, 1), *bq, out=out), steps, warmup)
+        _, ms_with_quantize = time_gpu(lambda: ops.linear(*ops.quantize(xa, 0, 1), *weights(), out=out), steps, warmup)
         del xa
+    del bqs
     tflops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
     gbs = linear_bytes(m, n, k) / (ms * 1e-3) / 1e9
     t_flops, t_bytes = 2.0 * m * n * k / (MFMA_PEAK_TFLOPS * 1e12), linear_bytes(m, n, k) / (HBM_PEAK_GBS * 1e9)
     rl = roofline("mfma", tflops, key) if t_flops >= t_bytes else roofline("hbm", gbs, key)
     return {"workload": f"NVFP4 linear M={m} N={n} K={k}, bf16 out, operands pre-quantized", "ms": ms,
             "total_ms": total, "TFLOP/s": tflops, "GB/s": gbs, "within_1e-2_of_fp32_dequant_matmul": ok,
-            "roofline": rl, "ms_with_activation_quantize": ms_with_quantize}
+            "roofline": rl, "ms_with_activation_quantize": ms_with_quantize, "rotating_weight_copies": ncopy}
 
 
 def vendor_gemm_yardstick(steps, warmup, n=8192):
@@ -226,22 +239,31 @@ def vendor_gemm_yardstick(steps, warmup, n=8192):
     return res
 
 
-def bench_decode(ops, m, n, k, steps, warmup, check=True):
-    """Fused decode-sized linear: bf16 activation in, on-the-fly NVFP4 quantize + GEMM."""
+def bench_decode(ops, m, n, k, steps, warmup, check=True, ncopy=3):
+    """Fused decode-sized linear: bf16 activation in, on-the-fly NVFP4 quantize + GEMM.  The calls
+    rotate over `ncopy` copies of the weights (3 x 132 MB: more than the 256 MB memory-side cache holds),
+    so that the weights are streamed from HBM."""
     x = make_input((m, k), seed=2, outliers=True).cuda()
     wq = ops.quantize(make_input((n, k), seed=3, std=0.02).cuda(), 0, 1)
+    wqs = [wq] + [tuple(t.clone() for t in wq) for _ in range(ncopy - 1)]
     out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
     ops.fused_linear(x, *wq, out=out)
     ok = None
     if check:
         ref = ops.linear(*ops.quantize(x, 0, 1), *wq)
         ok = bool(torch.all((out.float() - ref.float()).abs() <= 1e-2 + 1e-2 * ref.float().abs()).item())
-    _, ms = time_gpu(lambda: ops.fused_linear(x, *wq, out=out), steps, warmup)
+    turn = [0]
+
+    def step():
+        turn[0] += 1
+        ops.fused_linear(x, *wqs[turn[0] % ncopy], out=out)
+
+    _, ms = time_gpu(step, steps, warmup)
     nbytes = n * k // 2 + n * k // 16 + 2 * m * k + 2 * m * n
     gbs = nbytes / (ms * 1e-3) / 1e9
     return {"workload": f"fused decode linear M={m} N={n} K={k} (bf16 activation quantized on the fly)", "ms": ms,
             "bytes": nbytes, "GB/s": gbs, "equals_quantize_then_linear_within_1e-2": ok,
-            "roofline": roofline("hbm", gbs)}
+            "roofline": roofline("hbm", gbs), "rotating_weight_copies": ncopy}
 
 
 def bench_quantize_layouts(ops, steps, warmup):
