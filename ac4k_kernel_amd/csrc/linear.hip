@@ -1162,6 +1162,27 @@ __global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) 
   const int nsteps = a.ks_len / SK_STEP;  // 1..4
   const int pitch = a.ks_len * 2 + 16;    // LDS row pitch in bytes (16 bytes of padding: no bank conflicts)
 
+  // activation slice -> LDS as its exact fp16 dequantization (without the global scale).  A thread
+  // takes 32 elements (16 packed bytes, two 16-blocks) at a time; every load of the slice is issued
+  // before the first decode, so the slice costs one memory latency whatever M is.
+  // (the activation loads go out before the weight stream: the memory counter is in order, so loads
+  // issued behind the stream could only be waited for together with all of it)
+  constexpr int MAX_IT = 32 * (1024 / 32) / 256;  // M <= 32, slices of at most 1024 k
+  const int vec_per_row = a.ks_len / 32;
+  const int total = (int)a.M * vec_per_row;
+  uint4 aw[MAX_IT];
+  uint32_t ac[MAX_IT];
+#pragma unroll
+  for (int it = 0; it < MAX_IT; ++it) {
+    const int i = it * 256 + tid;
+    if (i < total) {
+      const int m = i / vec_per_row, v = i % vec_per_row;
+      const int64_t k = kbeg + v * 32;
+      aw[it] = *reinterpret_cast<const uint4 *>(a.Aq + (int64_t)m * (a.K >> 1) + (k >> 1));
+      // scale bytes of blocks (k/16) % 4 and the next one: k % 32 == 0, so an aligned pair
+      ac[it] = *reinterpret_cast<const uint16_t *>(a.A_sf + (((k >> 6) * a.Mp + m) << 2) + ((k >> 4) & 3));
+    }
+  }
   // weight stream of this lane: all steps of the slice are requested up front
   int64_t wrow = n0 + r;
   wrow = wrow < a.N ? wrow : a.N - 1;  // rows past N feed outputs that are never stored
@@ -1178,38 +1199,18 @@ __global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) 
       S[t][1] = sp[(int64_t)(t * 4 + 1) * a.Np];
     }
   }
-  // activation slice -> LDS as its exact fp16 dequantization (without the global scale).  A thread
-  // takes 32 elements (16 packed bytes, two 16-blocks) at a time; every load of the slice is issued
-  // before the first decode, so the slice costs one memory latency whatever M is.
-  {
-    constexpr int MAX_IT = 32 * (1024 / 32) / 256;  // M <= 32, slices of at most 1024 k
-    const int vec_per_row = a.ks_len / 32;
-    const int total = (int)a.M * vec_per_row;
-    uint4 aw[MAX_IT];
-    uint32_t ac[MAX_IT];
+  // decode of the activation slice, in the shadow of the weight loads
 #pragma unroll
-    for (int it = 0; it < MAX_IT; ++it) {
-      const int i = it * 256 + tid;
-      if (i < total) {
-        const int m = i / vec_per_row, v = i % vec_per_row;
-        const int64_t k = kbeg + v * 32;
-        aw[it] = *reinterpret_cast<const uint4 *>(a.Aq + (int64_t)m * (a.K >> 1) + (k >> 1));
-        // scale bytes of blocks (k/16) % 4 and the next one: k % 32 == 0, so an aligned pair
-        ac[it] = *reinterpret_cast<const uint16_t *>(a.A_sf + (((k >> 6) * a.Mp + m) << 2) + ((k >> 4) & 3));
-      }
-    }
-#pragma unroll
-    for (int it = 0; it < MAX_IT; ++it) {
-      const int i = it * 256 + tid;
-      if (i < total) {
-        const int m = i / vec_per_row, v = i % vec_per_row;
-        const f16x2 sc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(ac[it], 1.0f, false);
-        f16x8 *dst = reinterpret_cast<f16x8 *>(slds + m * pitch + v * 64);
-        dst[0] = decode_dword<false>(aw[it].x, sc);
-        dst[1] = decode_dword<false>(aw[it].y, sc);
-        dst[2] = decode_dword<true>(aw[it].z, sc);
-        dst[3] = decode_dword<true>(aw[it].w, sc);
-      }
+  for (int it = 0; it < MAX_IT; ++it) {
+    const int i = it * 256 + tid;
+    if (i < total) {
+      const int m = i / vec_per_row, v = i % vec_per_row;
+      const f16x2 sc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(ac[it], 1.0f, false);
+      f16x8 *dst = reinterpret_cast<f16x8 *>(slds + m * pitch + v * 64);
+      dst[0] = decode_dword<false>(aw[it].x, sc);
+      dst[1] = decode_dword<false>(aw[it].y, sc);
+      dst[2] = decode_dword<true>(aw[it].z, sc);
+      dst[3] = decode_dword<true>(aw[it].w, sc);
     }
   }
   __syncthreads();
