@@ -148,6 +148,28 @@ def test_fused_skinny_equals_composition(m, n, k):
     assert torch.equal(d, comp)  # same packed activation, same kernel arithmetic, same slice order
 
 
+def test_more_than_2_to_31_outputs():
+    """An output of 2.15e9 elements: element offsets past 32 bits in the epilogue.  Sampled rows and a
+    band of the last columns against the fp32 dequantize-matmul (on the GPU: the oracle would take
+    minutes), for the 2-byte and the 4-byte epilogue."""
+    m, n, k = 65536 + 16, 32768 + 8, 128
+    g = torch.Generator(device="cuda").manual_seed(11)
+    aq = ops().quantize(torch.empty((m, k), dtype=torch.bfloat16, device="cuda").normal_(generator=g), 0, 1)
+    bq = ops().quantize(torch.empty((n, k), dtype=torch.bfloat16, device="cuda").normal_(generator=g), 0, 1)
+    bias = torch.empty((1, n), dtype=torch.float32, device="cuda").normal_(generator=g)
+    da, db = gpu_dequant(aq, m), gpu_dequant(bq, n)
+    rows = torch.tensor([0, 1, 255, 256, m // 2, m - 17, m - 1], device="cuda")
+    for dt in (torch.bfloat16, torch.float32):
+        d = torch.full((m, n), 7.0, dtype=dt, device="cuda")
+        ops().linear(*aq, *bq, bias=bias, out=d)
+        ref = (da[rows] @ db.t() + bias).to(dt)
+        torch.testing.assert_close(d[rows], ref, atol=ATOL, rtol=RTOL)
+        refc = (da @ db[n - 40:].t() + bias[:, n - 40:]).to(dt)
+        torch.testing.assert_close(d[:, n - 40:], refc, atol=ATOL, rtol=RTOL)
+        del d, ref, refc
+    torch.cuda.empty_cache()
+
+
 def test_fused_skinny_edge_activations():
     """Blocks of zeros, a negative zero, one huge outlier and a whole row of zeros through the fused
     entry point: bytes, scales and global scale equal the oracle's."""

@@ -321,6 +321,35 @@ def test_rowwise_edges_and_max_scale():
         assert torch.equal(raw, eo), (prec, kw, (raw != eo).nonzero()[:4])
 
 
+def test_more_than_2_to_31_elements():
+    """A tensor of 2.15e9 elements (4.3 GB): offsets past 32 bits.  The oracle would take minutes at
+    this size, so the check is by parts: with the global scale of the whole tensor given, quantizing
+    the two halves separately must give the bytes and scales of the one big call, the global scale
+    must be the maximum / 2688, and two sampled row bands must equal the oracle."""
+    from ac4k_kernel_amd import _rocm_ops
+    R, K = 65536 + 16, 32768
+    x = torch.empty((R, K), dtype=torch.bfloat16, device="cuda")
+    x.normal_(generator=torch.Generator(device="cuda").manual_seed(5))
+    x[R - 3, K - 5] = 37.0  # the maximum sits past the 2^31-th element
+    out, sf, gs = ops().quantize(x, 0, 1)
+    assert gs.item() == (torch.tensor(37.0, dtype=torch.float32) / 2688.0).item()
+    for r0, r1 in ((0, 32768), (32768, R)):
+        xo, xs = torch.empty_like(out[r0:r1]), torch.empty_like(sf[:, r0:r1])
+        _rocm_ops.quantize_nvfp4(xo, xs, x[r0:r1], gs, 0, 1, False)
+        assert torch.equal(xo, out[r0:r1])
+        assert torch.equal(xs.view(torch.uint8), sf[:, r0:r1].contiguous().view(torch.uint8))
+    for r0 in (0, R - 64):  # 64-row bands against the oracle, global scale of the whole tensor
+        band = x[r0:r0 + 64].cpu()
+        eo, es, _ = T.quantize_nvfp4(band, 0, 1, False, gs=gs.cpu())
+        assert torch.equal(out[r0:r0 + 64].cpu(), eo)
+        assert torch.equal(sf[:, r0:r0 + 64].cpu().contiguous().view(torch.uint8), es)
+    o8, s8 = ops().quantize(x, 0, 1, precision="fp8e4m3")
+    e8, es8 = T.quantize_fp8(x[R - 64:].cpu(), 0, 1)
+    assert torch.equal(o8[R - 64:].cpu().view(torch.uint8), e8) and torch.equal(s8[R - 64:].cpu(), es8)
+    del x, out, sf, o8, s8
+    torch.cuda.empty_cache()
+
+
 def test_error_behaviour():
     o = ops()
     x = make_input((8, 64), seed=7).cuda()
