@@ -349,7 +349,7 @@ def main():
     global SETTLE_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all", choices=["all", "linear", "quantize", "traffic"])
     ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
