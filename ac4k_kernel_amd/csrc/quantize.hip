@@ -372,6 +372,7 @@ struct OnePassGeom {
   uint32_t total_chunks;  // 64-element chunks in the tensor
   uint32_t ncc;           // chunks per row (K / 64)
   uint32_t R, Rp, lead;   // rows per leading index, padded rows, number of leading indices
+  uint32_t swizzle;       // reduce dim permuted inside every 32-group (a lane quad holds one group)
 };
 
 // 16-byte load that bypasses the per-XCD L2 (device-coherent), completed before it returns
@@ -430,6 +431,10 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
     const uint32_t lv = (j % GS) * OP_THREADS + tid;  // vector inside the group
     v[j] = make_uint4(0, 0, 0, 0);
     if ((lv >> 3) < nvalid[j / GS]) v[j] = in[(uint64_t)cb[j / GS] * 8 + lv];
+  }
+  if (g.swizzle) {  // wave-uniform; four consecutive lanes hold one 32-group, valid or not as a whole
+#pragma unroll
+    for (int j = 0; j < NV; ++j) v[j] = swizzle_nvfp4_quad(v[j], (int)lane);
   }
   if (tid < 128) lut[tid] = g_rcp_e4m3.v[tid];
   uint32_t bm[NV];  // 16-block maxima (bf16 bits)
@@ -585,6 +590,7 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_small_kernel(
   const float gs = bf16_bits_to_f32(gm) / max_scale;
   if (blockIdx.x == 0 && tid == 0) *gs_out = gs;
   const float alpha = 1.0f / gs;
+  if (g.swizzle) own = swizzle_nvfp4_quad(own, (int)lane);  // the maximum above does not depend on the order
   uint32_t bm = absmax_bf16x8(own);
   bm = umax32(bm, dpp_u32<DPP_QUAD_XOR1>(bm));
   uint32_t code;
@@ -1120,14 +1126,15 @@ static bool try_quantize_nvfp4_onepass(void *out, void *sf, float *gs, const voi
                                        int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR, int64_t sK,
                                        int swizzle, float max_scale, hipStream_t st) {
   const int64_t ticks = g_sync_timeout_ticks.load();
-  if (ticks < 0 || swizzle || sK != 1 || K % 64 != 0 || sR != K) return false;
+  if (ticks < 0 || sK != 1 || K % 64 != 0 || sR != K) return false;
   if ((d1 > 1 && s1 != R * K) || (d0 > 1 && s0 != d1 * R * K)) return false;
   if (reinterpret_cast<uintptr_t>(in) & 15) return false;
   const int64_t lead = d0 * d1, chunks = lead * R * (K / 64);
   int nwg = device_cu_count();
   if (nwg > OP_MAX_WGS) nwg = OP_MAX_WGS;
   if (nwg < 8 || chunks > (int64_t)nwg * 128 * OP_MAX_NV) return false;
-  const OnePassGeom g{(uint32_t)chunks, (uint32_t)(K / 64), (uint32_t)R, (uint32_t)align_up(R, 16), (uint32_t)lead};
+  const OnePassGeom g{(uint32_t)chunks, (uint32_t)(K / 64), (uint32_t)R, (uint32_t)align_up(R, 16), (uint32_t)lead,
+                      swizzle ? 1u : 0u};
   if (chunks <= 128 * SMALL_MAX_SEGS) {  // small: one launch, no grid wait
     launch_small(static_cast<uint32_t *>(out), static_cast<uint32_t *>(sf), static_cast<const uint4 *>(in), gs, g,
                  max_scale, st);
