@@ -225,6 +225,66 @@ def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True, key=None, wi
             "roofline": rl, "ms_with_activation_quantize": ms_with_quantize, "rotating_weight_copies": ncopy}
 
 
+def _read_sclk_mhz():
+    """Current shader clock in MHz as the driver reports it: the starred line of pp_dpm_sclk in sysfs,
+    else what `rocm-smi --showclocks` prints (run as a child process); None when neither is readable."""
+    import glob
+    import re
+    import subprocess
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")):
+        try:
+            for ln in open(path).read().splitlines():
+                m = re.search(r"(\d+)\s*Mhz\s*\*", ln, re.I)
+                if m:
+                    return float(m.group(1)), "sysfs pp_dpm_sclk"
+        except OSError:
+            pass
+    try:
+        r = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20)
+        for ln in r.stdout.splitlines():
+            m = re.search(r"sclk clock level.*\((\d+)\s*Mhz\)", ln, re.I)
+            if m:
+                return float(m.group(1)), "rocm-smi --showclocks"
+    except (OSError, subprocess.SubprocessError):
+        pass
+    return None, None
+
+
+def shader_clock_under_load(ops, n=8192, seconds=1.5):
+    """Shader clock while the n^3 NVFP4 linear runs back to back (outside every timed region): a host
+    thread keeps the queue full, the main thread samples the driver's clock read-out.  The roofline
+    peak assumes 2.4 GHz; this is the clock the power limit leaves the kernel."""
+    import threading
+    idle, src = _read_sclk_mhz()
+    if src is None:
+        return {"under_load_mhz": None, "before_mhz": None, "source": None, "assumed_by_peak_mhz": 2400}
+    aq = ops.quantize(make_input((n, n), seed=0).cuda(), 0, 1)
+    bq = ops.quantize(make_input((n, n), seed=1).cuda(), 0, 1)
+    out = torch.empty((n, n), dtype=torch.bfloat16, device="cuda")
+    stop = [False]
+
+    def work():
+        while not stop[0]:
+            for _ in range(50):
+                ops.linear(*aq, *bq, out=out)
+            torch.cuda.synchronize()
+
+    th = threading.Thread(target=work)
+    th.start()
+    samples = []
+    try:
+        time.sleep(0.6 * seconds)
+        for _ in range(3):
+            samples.append(_read_sclk_mhz()[0])
+            time.sleep(0.13 * seconds)
+    finally:
+        stop[0] = True
+        th.join()
+    samples = sorted(x for x in samples if x is not None)
+    return {"under_load_mhz": samples[len(samples) // 2] if samples else None, "before_mhz": idle, "source": src,
+            "assumed_by_peak_mhz": 2400, "workload": f"NVFP4 linear M=N=K={n} back to back"}
+
+
 def vendor_gemm_yardstick(steps, warmup, n=8192):
     """What the vendor library's dense 16-bit GEMM (torch.matmul) sustains on this box at n^3: not part
     of the product and not a baseline of the metric (its operands are dense fp16/bf16, nothing is
@@ -401,6 +461,15 @@ def main():
             line["cpu_baseline"] = cpu_linear_baseline(8192, 8192)
             log(f"[bench] cpu linear oracle: {line['cpu_baseline']['value']:.3f} TFLOP/s")
         if args.workload == "all":
+            line["shader_clock"] = shader_clock_under_load(ops)
+            mhz = line["shader_clock"]["under_load_mhz"]
+            if mhz:  # the same MFMA count per clock at the clock the power limit leaves
+                line["shader_clock"]["peak_at_this_clock_TFLOP/s"] = MFMA_PEAK_TFLOPS * mhz / 2400.0
+                line["shader_clock"]["frac_of_peak_at_this_clock"] = lin["TFLOP/s"] / (MFMA_PEAK_TFLOPS * mhz / 2400.0)
+            log(f"[bench] shader clock: {mhz} MHz under the 8192^3 linear, "
+                f"{line['shader_clock']['before_mhz']} MHz before it ({line['shader_clock']['source']}); "
+                f"the {MFMA_PEAK_TFLOPS:.0f} TFLOP/s peak assumes 2400 MHz"
+                + (f"; {100 * line['shader_clock']['frac_of_peak_at_this_clock']:.1f}% of the peak at this clock" if mhz else ""))
             line["vendor_dense_gemm"] = vendor_gemm_yardstick(S, W)
             log(f"[bench] yardstick, torch.matmul 8192^3 on already dense operands: "
                 f"{line['vendor_dense_gemm']['bf16_TFLOP/s']:.0f} TFLOP/s bf16, "
