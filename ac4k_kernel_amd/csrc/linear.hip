@@ -601,8 +601,20 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[MI][NJ], char *ld
     __syncthreads();
   }
   // the four outputs acc[i][j][4g .. 4g+3] of a lane, scaled, plus their bias b
+  // The 256x256 tile keeps its 256 sums per lane in accumulation registers.  Left alone, the compiler
+  // moves all of them to ordinary registers at the top of the epilogue and spills what does not fit;
+  // reading them with a volatile move keeps each read inside the pass that stages the value.
+  auto sum_of = [&](int i, int j, int e) {
+    if constexpr (MI * NJ == 16) {
+      float v;
+      asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[i][j][e]));
+      return v;
+    } else {
+      return acc[i][j][e];
+    }
+  };
   auto value4 = [&](int i, int j, int g, const float4 &b) {
-    float4 v = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+    float4 v = make_float4(sum_of(i, j, 4 * g), sum_of(i, j, 4 * g + 1), sum_of(i, j, 4 * g + 2), sum_of(i, j, 4 * g + 3));
     if constexpr (!RAW) {
       v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
     }
@@ -619,77 +631,67 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[MI][NJ], char *ld
       if constexpr (BIAS_DT != BIAS_NONE) b[g] = *reinterpret_cast<const float4 *>(bias_s + j * 32 + g * 8);
     }
   };
+  // 16-byte stores need rows that start on 16-byte boundaries; other shapes leave the staging block
+  // element by element (a rolled loop over LDS, so that this rare path costs no registers)
   const bool vec_ok = (N % (16 / S) == 0) && ((uintptr_t)out % 16 == 0);
-  if (vec_ok) {
-    char *stg = lds + wave * (RP * PITCH);
-    constexpr int CPR = WN * S / 16;   // 16-byte pieces per staged row
-    constexpr int RS = 64 / CPR;       // rows covered by one wave store
-    const int lrow = lane / CPR, lq = lane % CPR;
-    const int64_t row_bytes = N * S;
-    const uint32_t lane_off = (uint32_t)(lrow * row_bytes) + lq * 16;
-    char *out0 = reinterpret_cast<char *>(Dp) + (m0 * N + n0) * S;  // wave-uniform
-    const bool interior = m0 + 32 * MI <= M && n0 + WN <= N;
-    const bool col_ok = n0 + lq * (16 / S) < N;
-    const int64_t rl = M - m0 - lrow;
-    const int rows_left = rl > 32 * MI ? 32 * MI : (int)rl;  // rows of the block below this lane's first one
+  char *stg = lds + wave * (RP * PITCH);
+  constexpr int CPR = WN * S / 16;   // 16-byte pieces per staged row
+  constexpr int RS = 64 / CPR;       // rows covered by one wave store
+  const int lrow = lane / CPR, lq = lane % CPR;
+  const int64_t row_bytes = N * S;
+  const uint32_t lane_off = (uint32_t)(lrow * row_bytes) + lq * 16;
+  char *out0 = reinterpret_cast<char *>(Dp) + (m0 * N + n0) * S;  // wave-uniform
+  const bool interior = vec_ok && m0 + 32 * MI <= M && n0 + WN <= N;
+  const int64_t cl = N - n0 - lq * (16 / S);
+  const int cols_left = cl > 16 / S ? 16 / S : (int)cl;  // columns of this lane's piece inside the matrix
+  const int64_t rl = M - m0 - lrow;
+  const int rows_left = rl > 32 * MI ? 32 * MI : (int)rl;  // rows of the block below this lane's first one
 #pragma unroll
-    for (int p = 0; p < 32 * MI / RP; ++p) {
-      asm volatile("" ::: "memory");  // keeps the bias reads of one pass from being merged with the next one's
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        float4 b[4];
-        bias_of(j, b);
-#pragma unroll
-        for (int ii = 0; ii < RP / 32; ++ii) {
-          const int i = p * (RP / 32) + ii;
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const float4 v = value4(i, j, g, b[g]);
-            char *dst = stg + (ii * 32 + (lane & 31)) * PITCH + (j * 32 + g * 8 + half * 4) * S;
-            if constexpr (S == 2) *reinterpret_cast<uint2 *>(dst) = make_uint2(DE::cvt2(v.x, v.y), DE::cvt2(v.z, v.w));
-            else *reinterpret_cast<float4 *>(dst) = v;
-          }
-        }
-      }
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the staging block is private to the wave
-      // pass `it` stores rows it*RS .. it*RS+RS-1 of the block: a wave-uniform base that advances by
-      // RS rows, plus a fixed 32-bit lane offset; the bounds checks are per lane only on edge tiles
-      const char *src = stg + lrow * PITCH + lq * 16;
-      char *rowp = out0 + (int64_t)p * RP * row_bytes;
-      if (interior) {
-#pragma unroll
-        for (int it = 0; it < RP / RS; ++it)
-          *reinterpret_cast<uint4 *>(rowp + it * RS * row_bytes + lane_off) =
-              *reinterpret_cast<const uint4 *>(src + it * RS * PITCH);
-      } else {
-#pragma unroll
-        for (int it = 0; it < RP / RS; ++it) {
-          const uint4 v = *reinterpret_cast<const uint4 *>(src + it * RS * PITCH);
-          if (col_ok && p * RP + it * RS < rows_left) *reinterpret_cast<uint4 *>(rowp + it * RS * row_bytes + lane_off) = v;
-        }
-      }
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    }
-  } else {
+  for (int p = 0; p < 32 * MI / RP; ++p) {
+    asm volatile("" ::: "memory");  // keeps the bias reads of one pass from being merged with the next one's
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       float4 b[4];
       bias_of(j, b);
 #pragma unroll
-      for (int i = 0; i < MI; ++i) {
-        const int64_t m = m0 + i * 32 + (lane & 31);
+      for (int ii = 0; ii < RP / 32; ++ii) {
+        const int i = p * (RP / 32) + ii;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const float4 v = value4(i, j, g, b[g]);
-          const float ve[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int64_t n = n0 + j * 32 + g * 8 + half * 4 + q;
-            if (m < M && n < N) Dp[m * N + n] = DE::cvt(ve[q]);
-          }
+          char *dst = stg + (ii * 32 + (lane & 31)) * PITCH + (j * 32 + g * 8 + half * 4) * S;
+          if constexpr (S == 2) *reinterpret_cast<uint2 *>(dst) = make_uint2(DE::cvt2(v.x, v.y), DE::cvt2(v.z, v.w));
+          else *reinterpret_cast<float4 *>(dst) = v;
         }
       }
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the staging block is private to the wave
+    // pass `it` stores rows it*RS .. it*RS+RS-1 of the block: a wave-uniform base that advances by
+    // RS rows, plus a fixed 32-bit lane offset; the bounds checks are per lane only on edge tiles
+    const char *src = stg + lrow * PITCH + lq * 16;
+    char *rowp = out0 + (int64_t)p * RP * row_bytes;
+    if (interior) {
+#pragma unroll
+      for (int it = 0; it < RP / RS; ++it)
+        *reinterpret_cast<uint4 *>(rowp + it * RS * row_bytes + lane_off) =
+            *reinterpret_cast<const uint4 *>(src + it * RS * PITCH);
+    } else if (vec_ok) {
+#pragma unroll
+      for (int it = 0; it < RP / RS; ++it) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(src + it * RS * PITCH);
+        if (cols_left > 0 && p * RP + it * RS < rows_left) *reinterpret_cast<uint4 *>(rowp + it * RS * row_bytes + lane_off) = v;
+      }
+    } else {
+#pragma unroll 1
+      for (int it = 0; it < RP / RS; ++it) {
+        if (p * RP + it * RS >= rows_left) break;
+        const DT *se = reinterpret_cast<const DT *>(src + it * RS * PITCH);
+        DT *de = reinterpret_cast<DT *>(rowp + it * RS * row_bytes + lane_off);
+#pragma unroll 1
+        for (int e = 0; e < cols_left; ++e) de[e] = se[e];
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   }
 }
 
