@@ -1194,33 +1194,33 @@ static int launch_quantize_nvfp4(void *out, void *sf, const void *in, const Glob
   const uint16_t *x = static_cast<const uint16_t *>(in);
   const int64_t lead_all = d0 * d1;
   for (g.lead0 = 0; g.lead0 < lead_all; g.lead0 += 65535) {
-  const int64_t lead = lead_all - g.lead0 < 65535 ? lead_all - g.lead0 : 65535;
-  if (rowmajor_ok(in, K, s0, s1, sR, sK) && ceil_div(g.Kp, 64) * ceil_div(g.Rp, 16) < (1ll << 31)) {
-    const int64_t chunks = g.Kp / 64;
-    const bool sw = swizzle != 0;
-    // four chunks per wave row: a workgroup then covers 32 rows x 256 elements, and each scale
-    // column gets a 128-byte run; eight chunks per row measured 4-12 % slower on every shape
-    if (chunks >= 3)
-      launch_nvfp4_rowmajor<4>(o, s, x, gsrc, g, lead, st, sw);
-    else if (chunks == 2)
-      launch_nvfp4_rowmajor<2>(o, s, x, gsrc, g, lead, st, sw);
-    else
-      launch_nvfp4_rowmajor<1>(o, s, x, gsrc, g, lead, st, sw);
-  } else if (crossmajor_ok(in, R, s0, s1, sR, sK) && ceil_div(g.Rp, 128) <= 65535) {
-    // (position along the reduce dim as the fast grid index: the packed rows are written in runs along it)
-    const dim3 grid = crossmajor_grid(g, ceil_div(g.Kp / 64, 4), ceil_div(g.Rp, 128), lead);
-    if (swizzle)
-      hipLaunchKernelGGL(quantize_nvfp4_crossmajor_kernel<true>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
-    else
-      hipLaunchKernelGGL(quantize_nvfp4_crossmajor_kernel<false>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
-  } else {
-    AC4K_REQUIRE(g.Kp / 64 <= 65535, "reduce dim too large for the strided path (%lld)", (long long)K);
-    dim3 grid((unsigned)ceil_div(g.Rp, 256), (unsigned)(g.Kp / 64), (unsigned)lead);
-    if (swizzle)
-      hipLaunchKernelGGL(quantize_nvfp4_generic_kernel<true>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
-    else
-      hipLaunchKernelGGL(quantize_nvfp4_generic_kernel<false>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
-  }
+    const int64_t lead = lead_all - g.lead0 < 65535 ? lead_all - g.lead0 : 65535;
+    if (rowmajor_ok(in, K, s0, s1, sR, sK) && ceil_div(g.Kp, 64) * ceil_div(g.Rp, 16) < (1ll << 31)) {
+      const int64_t chunks = g.Kp / 64;
+      const bool sw = swizzle != 0;
+      // four chunks per wave row: a workgroup then covers 32 rows x 256 elements, and each scale
+      // column gets a 128-byte run; eight chunks per row measured 4-12 % slower on every shape
+      if (chunks >= 3)
+        launch_nvfp4_rowmajor<4>(o, s, x, gsrc, g, lead, st, sw);
+      else if (chunks == 2)
+        launch_nvfp4_rowmajor<2>(o, s, x, gsrc, g, lead, st, sw);
+      else
+        launch_nvfp4_rowmajor<1>(o, s, x, gsrc, g, lead, st, sw);
+    } else if (crossmajor_ok(in, R, s0, s1, sR, sK) && ceil_div(g.Rp, 128) <= 65535) {
+      // (position along the reduce dim as the fast grid index: the packed rows are written in runs along it)
+      const dim3 grid = crossmajor_grid(g, ceil_div(g.Kp / 64, 4), ceil_div(g.Rp, 128), lead);
+      if (swizzle)
+        hipLaunchKernelGGL(quantize_nvfp4_crossmajor_kernel<true>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
+      else
+        hipLaunchKernelGGL(quantize_nvfp4_crossmajor_kernel<false>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
+    } else {
+      AC4K_REQUIRE(g.Kp / 64 <= 65535, "reduce dim too large for the strided path (%lld)", (long long)K);
+      dim3 grid((unsigned)ceil_div(g.Rp, 256), (unsigned)(g.Kp / 64), (unsigned)lead);
+      if (swizzle)
+        hipLaunchKernelGGL(quantize_nvfp4_generic_kernel<true>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
+      else
+        hipLaunchKernelGGL(quantize_nvfp4_generic_kernel<false>, grid, dim3(256), 0, st, o, s, x, gsrc, g);
+    }
   }
   return 0;
 }
@@ -1292,58 +1292,58 @@ static int quantize_rowwise(void *out, float *sf, const void *in, const void *sm
   const uint16_t *x = static_cast<const uint16_t *>(in);
   const int64_t lead_all = d0 * d1;
   for (g.lead0 = 0; g.lead0 < lead_all; g.lead0 += 65535) {
-  const int64_t lead = lead_all - g.lead0 < 65535 ? lead_all - g.lead0 : 65535;
-  if (rowmajor_ok(in, K, s0, s1, sR, sK) && K <= 16384) {
-    const bool sw = swizzle != 0;
-    if (K <= 64)
-      launch_rowwise_rowmajor<FMT, 8, 1>(o, sf, x, smax, g, lead, st, sw);
-    else if (K <= 128)
-      launch_rowwise_rowmajor<FMT, 16, 1>(o, sf, x, smax, g, lead, st, sw);
-    else if (K <= 256)
-      launch_rowwise_rowmajor<FMT, 32, 1>(o, sf, x, smax, g, lead, st, sw);
-    else if (K <= 512)
-      launch_rowwise_rowmajor<FMT, 64, 1>(o, sf, x, smax, g, lead, st, sw);
-    else if (K <= 1024)
-      launch_rowwise_rowmajor<FMT, 64, 2>(o, sf, x, smax, g, lead, st, sw);
-    else if (K <= 2048)
-      launch_rowwise_rowmajor<FMT, 64, 4>(o, sf, x, smax, g, lead, st, sw);
-    else if (K <= 4096)
-      launch_rowwise_rowmajor<FMT, 64, 8>(o, sf, x, smax, g, lead, st, sw);
-    else if (K <= 8192)
-      launch_rowwise_rowmajor<FMT, 64, 16>(o, sf, x, smax, g, lead, st, sw);
-    else
-      launch_rowwise_rowmajor<FMT, 64, 32>(o, sf, x, smax, g, lead, st, sw);
-  } else if (!swizzle && rowmajor_ok(in, K, s0, s1, sR, sK)) {  // rows too long for the register file
-    dim3 grid((unsigned)ceil_div(g.Rp, 4), (unsigned)lead);
-    hipLaunchKernelGGL((quantize_rowwise_longrow_kernel<FMT>), grid, dim3(256), 0, st, o, sf, x, smax, g);
-  } else if (crossmajor_ok(in, R, s0, s1, sR, sK) && ceil_div(g.Rp, 128) <= 65535 && ceil_div(K, CM_KSPAN) <= 65535) {
-    // row maxima as bf16 bit patterns in the scale array, quantize from them, then scale them in place
-    uint32_t *bits = reinterpret_cast<uint32_t *>(sf) + g.lead0 * g.Rp;  // the kernels index by absolute lead
-    const int64_t nsf = lead * g.Rp;
-    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)ceil_div(nsf, 256)), dim3(256), 0, st, bits, nsf, 0u);
-    // Both kernels walk the grid along the dim of smaller input stride first (measured on
-    // (1,75600,40,128), cross 3, reduce 1: 412 us against 440 us; the nvfp4 kernel, whose packed
-    // rows are a quarter as long, loses 6% by the same change and keeps the reduce dim first).
-    const int64_t kblocks = ceil_div(g.Kp / 16, 16);  // of the quantize kernel; the maxima kernel has fewer
-    g.lead_fast = crossmajor_lead_fast(d1, s1, sK, kblocks);
-    hipLaunchKernelGGL(rowwise_crossmajor_amax_kernel, crossmajor_grid(g, ceil_div(K, CM_KSPAN), ceil_div(g.Rp, 128), lead),
-                       dim3(256), 0, st, reinterpret_cast<uint32_t *>(sf), x, g);
-    const dim3 grid = crossmajor_grid(g, kblocks, ceil_div(g.Rp, 128), lead);
-    if (swizzle)
-      hipLaunchKernelGGL((quantize_rowwise_crossmajor_kernel<FMT, true>), grid, dim3(256), 0, st, o,
-                         reinterpret_cast<const uint32_t *>(sf), x, smax, g);
-    else
-      hipLaunchKernelGGL((quantize_rowwise_crossmajor_kernel<FMT, false>), grid, dim3(256), 0, st, o,
-                         reinterpret_cast<const uint32_t *>(sf), x, smax, g);
-    hipLaunchKernelGGL(rowwise_crossmajor_finalize_kernel<FMT>, dim3((unsigned)ceil_div(nsf, 256)), dim3(256), 0, st,
-                       sf + g.lead0 * g.Rp, smax, nsf);
-  } else {
-    dim3 grid((unsigned)ceil_div(g.Rp, 256), (unsigned)lead);
-    if (swizzle)
-      hipLaunchKernelGGL((quantize_rowwise_generic_kernel<FMT, true>), grid, dim3(256), 0, st, o, sf, x, smax, g);
-    else
-      hipLaunchKernelGGL((quantize_rowwise_generic_kernel<FMT, false>), grid, dim3(256), 0, st, o, sf, x, smax, g);
-  }
+    const int64_t lead = lead_all - g.lead0 < 65535 ? lead_all - g.lead0 : 65535;
+    if (rowmajor_ok(in, K, s0, s1, sR, sK) && K <= 16384) {
+      const bool sw = swizzle != 0;
+      if (K <= 64)
+        launch_rowwise_rowmajor<FMT, 8, 1>(o, sf, x, smax, g, lead, st, sw);
+      else if (K <= 128)
+        launch_rowwise_rowmajor<FMT, 16, 1>(o, sf, x, smax, g, lead, st, sw);
+      else if (K <= 256)
+        launch_rowwise_rowmajor<FMT, 32, 1>(o, sf, x, smax, g, lead, st, sw);
+      else if (K <= 512)
+        launch_rowwise_rowmajor<FMT, 64, 1>(o, sf, x, smax, g, lead, st, sw);
+      else if (K <= 1024)
+        launch_rowwise_rowmajor<FMT, 64, 2>(o, sf, x, smax, g, lead, st, sw);
+      else if (K <= 2048)
+        launch_rowwise_rowmajor<FMT, 64, 4>(o, sf, x, smax, g, lead, st, sw);
+      else if (K <= 4096)
+        launch_rowwise_rowmajor<FMT, 64, 8>(o, sf, x, smax, g, lead, st, sw);
+      else if (K <= 8192)
+        launch_rowwise_rowmajor<FMT, 64, 16>(o, sf, x, smax, g, lead, st, sw);
+      else
+        launch_rowwise_rowmajor<FMT, 64, 32>(o, sf, x, smax, g, lead, st, sw);
+    } else if (!swizzle && rowmajor_ok(in, K, s0, s1, sR, sK)) {  // rows too long for the register file
+      dim3 grid((unsigned)ceil_div(g.Rp, 4), (unsigned)lead);
+      hipLaunchKernelGGL((quantize_rowwise_longrow_kernel<FMT>), grid, dim3(256), 0, st, o, sf, x, smax, g);
+    } else if (crossmajor_ok(in, R, s0, s1, sR, sK) && ceil_div(g.Rp, 128) <= 65535 && ceil_div(K, CM_KSPAN) <= 65535) {
+      // row maxima as bf16 bit patterns in the scale array, quantize from them, then scale them in place
+      uint32_t *bits = reinterpret_cast<uint32_t *>(sf) + g.lead0 * g.Rp;  // the kernels index by absolute lead
+      const int64_t nsf = lead * g.Rp;
+      hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)ceil_div(nsf, 256)), dim3(256), 0, st, bits, nsf, 0u);
+      // Both kernels walk the grid along the dim of smaller input stride first (measured on
+      // (1,75600,40,128), cross 3, reduce 1: 412 us against 440 us; the nvfp4 kernel, whose packed
+      // rows are a quarter as long, loses 6% by the same change and keeps the reduce dim first).
+      const int64_t kblocks = ceil_div(g.Kp / 16, 16);  // of the quantize kernel; the maxima kernel has fewer
+      g.lead_fast = crossmajor_lead_fast(d1, s1, sK, kblocks);
+      hipLaunchKernelGGL(rowwise_crossmajor_amax_kernel, crossmajor_grid(g, ceil_div(K, CM_KSPAN), ceil_div(g.Rp, 128), lead),
+                         dim3(256), 0, st, reinterpret_cast<uint32_t *>(sf), x, g);
+      const dim3 grid = crossmajor_grid(g, kblocks, ceil_div(g.Rp, 128), lead);
+      if (swizzle)
+        hipLaunchKernelGGL((quantize_rowwise_crossmajor_kernel<FMT, true>), grid, dim3(256), 0, st, o,
+                           reinterpret_cast<const uint32_t *>(sf), x, smax, g);
+      else
+        hipLaunchKernelGGL((quantize_rowwise_crossmajor_kernel<FMT, false>), grid, dim3(256), 0, st, o,
+                           reinterpret_cast<const uint32_t *>(sf), x, smax, g);
+      hipLaunchKernelGGL(rowwise_crossmajor_finalize_kernel<FMT>, dim3((unsigned)ceil_div(nsf, 256)), dim3(256), 0, st,
+                         sf + g.lead0 * g.Rp, smax, nsf);
+    } else {
+      dim3 grid((unsigned)ceil_div(g.Rp, 256), (unsigned)lead);
+      if (swizzle)
+        hipLaunchKernelGGL((quantize_rowwise_generic_kernel<FMT, true>), grid, dim3(256), 0, st, o, sf, x, smax, g);
+      else
+        hipLaunchKernelGGL((quantize_rowwise_generic_kernel<FMT, false>), grid, dim3(256), 0, st, o, sf, x, smax, g);
+    }
   }
   return check_launch(what);
 }
