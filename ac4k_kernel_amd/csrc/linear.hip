@@ -1124,7 +1124,8 @@ static int launch_tile256(const LinearArgs &a, hipStream_t st) {
 //
 // A workgroup (4 waves) owns 128 weight rows and one K-slice; every wave one 32-row tile.  It
 // first decodes its slice of the packed activation to fp16 (exact, without the global scale)
-// into LDS, shared by the four waves.  Lane (row r, half h) streams 64 contiguous bytes of its weight row per 256-k step
+// into LDS, shared by the four waves (with more than 16 activation rows, 512 k at a time, so that
+// the LDS footprint stays at 33 KB).  Lane (row r, half h) streams 64 contiguous bytes of its weight row per 256-k step
 // (elements [128h, 128h+128) of the step) and decodes them dword by dword into MFMA operands;
 // The MFMA is issued as
 // D^T = W . Ahat^T so a lane ends up with 4 consecutive n for one m.  K-slices of one row
@@ -1162,7 +1163,11 @@ __global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) 
   const int64_t ng = blockIdx.y, n0 = ng * SK_ROWS + wave * 32;
   const int64_t kbeg = (int64_t)ksl * a.ks_len;
   const int nsteps = a.ks_len / SK_STEP;  // 1..4
-  const int pitch = a.ks_len * 2 + 16;    // LDS row pitch in bytes (16 bytes of padding: no bank conflicts)
+  // With more than 16 activation rows a 1024-k slice goes through LDS in two halves of 512 k, which
+  // keeps the slice at 33 KB and three workgroups on a CU.
+  const bool halves = a.M > 16 && nsteps == 4;
+  const int lds_k = halves ? 512 : a.ks_len;  // k positions held in LDS at a time
+  const int pitch = lds_k * 2 + 16;       // LDS row pitch in bytes (16 bytes of padding: no bank conflicts)
 
   // activation slice -> LDS as its exact fp16 dequantization (without the global scale).  A thread
   // takes 32 elements (16 packed bytes, two 16-blocks) at a time; every load of the slice is issued
@@ -1201,20 +1206,24 @@ __global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) 
       S[t][1] = sp[(int64_t)(t * 4 + 1) * a.Np];
     }
   }
-  // decode of the activation slice, in the shadow of the weight loads
+  // decode of the activation slice (or of its half `part`), in the shadow of the weight loads
+  auto decode_activation = [&](int part) {
 #pragma unroll
-  for (int it = 0; it < MAX_IT; ++it) {
-    const int i = it * 256 + tid;
-    if (i < total) {
-      const int m = i / vec_per_row, v = i % vec_per_row;
-      const f16x2 sc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(ac[it], 1.0f, false);
-      f16x8 *dst = reinterpret_cast<f16x8 *>(slds + m * pitch + v * 64);
-      dst[0] = decode_dword<false>(aw[it].x, sc);
-      dst[1] = decode_dword<false>(aw[it].y, sc);
-      dst[2] = decode_dword<true>(aw[it].z, sc);
-      dst[3] = decode_dword<true>(aw[it].w, sc);
+    for (int it = 0; it < MAX_IT; ++it) {
+      const int i = it * 256 + tid;
+      if (i < total) {
+        const int m = i / vec_per_row, v = i % vec_per_row;
+        if (halves && (v >> 4) != part) continue;
+        const f16x2 sc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(ac[it], 1.0f, false);
+        f16x8 *dst = reinterpret_cast<f16x8 *>(slds + m * pitch + (halves ? v & 15 : v) * 64);
+        dst[0] = decode_dword<false>(aw[it].x, sc);
+        dst[1] = decode_dword<false>(aw[it].y, sc);
+        dst[2] = decode_dword<true>(aw[it].z, sc);
+        dst[3] = decode_dword<true>(aw[it].w, sc);
+      }
     }
-  }
+  };
+  decode_activation(0);
   __syncthreads();
 
   f32x16 acc0, acc1;
@@ -1224,6 +1233,11 @@ __global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) 
   const char *arow = slds + am * pitch + h * 256;
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
+    if (t == 2 && halves) {  // second half of the slice replaces the first in LDS
+      __syncthreads();
+      decode_activation(1);
+      __syncthreads();
+    }
     if (t < nsteps) {
       f16x2 sc[2][2];  // [chunk][block pair] -> scales of blocks (0,1) and (2,3) of each 64-chunk
 #pragma unroll
@@ -1239,7 +1253,7 @@ __global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) 
           const int blk = (4 * q + d) >> 1;   // 0..7: chunk blk/4, block blk%4
           const f16x2 pair = sc[blk >> 2][(blk & 3) >> 1];
           f16x8 wdec = (blk & 1) ? decode_dword<true>(w[d], pair) : decode_dword<false>(w[d], pair);
-          const f16x8 afrag = *reinterpret_cast<const f16x8 *>(arow + t * 512 + (q * 4 + d) * 16);
+          const f16x8 afrag = *reinterpret_cast<const f16x8 *>(arow + (halves ? t & 1 : t) * 512 + (q * 4 + d) * 16);
           if ((q * 4 + d) & 1)
             acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wdec, afrag, acc1, 0, 0, 0);
           else
@@ -1365,7 +1379,7 @@ static bool skinny_plan(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
   p.ks_len = ks;
   p.split_k = (int)(K / ks);
   p.partial_bytes = p.split_k > 1 ? (int64_t)p.split_k * M * N * 4 : 0;
-  p.lds_bytes = (int)M * (ks * 2 + 16);
+  p.lds_bytes = (int)M * ((M > 16 && ks == 1024 ? 512 : ks) * 2 + 16);
   return true;
 }
 
