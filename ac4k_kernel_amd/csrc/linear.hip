@@ -1152,8 +1152,11 @@ struct SkinnyArgs {
 constexpr int SK_ROWS = 128;   // weight rows per workgroup
 constexpr int SK_STEP = 256;   // k per step
 
-template <int D_DT, int BIAS_DT>
-__global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) {
+// MAX_IT: 16-byte activation vectors a lane may have to fetch (M * 32 / 256 rounded up): 1 for M <= 8, 2 for
+// M <= 16, 4 for M <= 32.  With one accumulator tile (the MFMAs of a lane then queue behind each other, which a
+// kernel that waits for memory does not notice) the two smaller variants fit four workgroups on a CU.
+template <int D_DT, int BIAS_DT, int MAX_IT>
+__global__ __launch_bounds__(256, MAX_IT <= 2 ? 4 : 3) void linear_nvfp4_skinny_kernel(SkinnyArgs a) {
   extern __shared__ __attribute__((aligned(16))) char slds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, h = lane >> 5;
@@ -1174,7 +1177,6 @@ __global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) 
   // before the first decode, so the slice costs one memory latency whatever M is.
   // (the activation loads go out before the weight stream: the memory counter is in order, so loads
   // issued behind the stream could only be waited for together with all of it)
-  constexpr int MAX_IT = 32 * (1024 / 32) / 256;  // M <= 32, slices of at most 1024 k
   const int vec_per_row = a.ks_len / 32;
   const int total = (int)a.M * vec_per_row;
   uint4 aw[MAX_IT];
@@ -1226,9 +1228,9 @@ __global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) 
   decode_activation(0);
   __syncthreads();
 
-  f32x16 acc0, acc1;
+  f32x16 acc0;
 #pragma unroll
-  for (int e = 0; e < 16; ++e) acc0[e] = acc1[e] = 0.0f;
+  for (int e = 0; e < 16; ++e) acc0[e] = 0.0f;
   const int am = r < (int)a.M ? r : (int)a.M - 1;  // lanes past M read a valid row; their outputs are dropped
   const char *arow = slds + am * pitch + h * 256;
 #pragma unroll
@@ -1254,16 +1256,11 @@ __global__ __launch_bounds__(256) void linear_nvfp4_skinny_kernel(SkinnyArgs a) 
           const f16x2 pair = sc[blk >> 2][(blk & 3) >> 1];
           f16x8 wdec = (blk & 1) ? decode_dword<true>(w[d], pair) : decode_dword<false>(w[d], pair);
           const f16x8 afrag = *reinterpret_cast<const f16x8 *>(arow + (halves ? t & 1 : t) * 512 + (q * 4 + d) * 16);
-          if ((q * 4 + d) & 1)
-            acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wdec, afrag, acc1, 0, 0, 0);
-          else
-            acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wdec, afrag, acc0, 0, 0, 0);
+          acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wdec, afrag, acc0, 0, 0, 0);
         }
       }
     }
   }
-#pragma unroll
-  for (int e = 0; e < 16; ++e) acc0[e] += acc1[e];
 
   // acc0: lane <-> m = r, element e <-> n = n0 + (e>>2)*8 + h*4 + (e&3): 4 consecutive n per group
   const int m = r;
@@ -1383,14 +1380,21 @@ static bool skinny_plan(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
   return true;
 }
 
-template <int D_DT, int BIAS_DT>
-static int launch_skinny(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_t st) {
-  auto *kern = linear_nvfp4_skinny_kernel<D_DT, BIAS_DT>;
+template <int D_DT, int BIAS_DT, int MAX_IT>
+static int launch_skinny_it(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_t st) {
+  auto *kern = linear_nvfp4_skinny_kernel<D_DT, BIAS_DT, MAX_IT>;
   static std::atomic<uint32_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, lds_ok, 32 * (1024 * 2 + 16))) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)p.split_k, (unsigned)p.groups), dim3(256), p.lds_bytes, st, a);
   if (p.split_k > 1) launch_reduce<D_DT, BIAS_DT>(a, st);
   return 0;
+}
+
+template <int D_DT, int BIAS_DT>
+static int launch_skinny(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_t st) {
+  if (a.M <= 8) return launch_skinny_it<D_DT, BIAS_DT, 1>(a, p, st);
+  if (a.M <= 16) return launch_skinny_it<D_DT, BIAS_DT, 2>(a, p, st);
+  return launch_skinny_it<D_DT, BIAS_DT, 4>(a, p, st);
 }
 
 template <int D_DT>
