@@ -13,6 +13,12 @@ in test/test_quantize_bandwidth.py:32-33, whole quantize() call, three rotating 
 buffers), under "linear_shapes" the other GEMM configurations and under "decode" the fused
 decode-sized linear.
 
+oracle/ is used by the CPU leg of the run only: the oracle is timed on the host cores as
+`cpu_baseline`, and the same oracle checks the quantizers' GPU output of the same inputs bit
+for bit (`bit_exact_vs_oracle`); --no-cpu-baseline skips both.  The GEMM check compares with an
+fp32 dequantize-matmul made of torch ops on the GPU.  Nothing that is timed on the GPU calls the
+oracle.
+
 A "step" is one pass of the timed op over one batch of synthetic input.  Timing uses
 events recorded on the stream the kernels are launched on (torch's current stream, which
 is the stream handed to the C ABI).  `roofline.traffic` is not measured live: it is the HBM
@@ -103,13 +109,14 @@ def quant_bytes(shape_rk, precision):
 
 
 def bench_quantize(ops, shape, precision, steps, warmup, outliers, check=True, nbuf=3, key=None):
-    from oracle import nvfp4_oracle as T
+    """`check`: the CPU leg of the run compares the GPU output of the first input with the oracle's, bit for bit."""
     xs_cpu = [make_input(shape, seed=s, outliers=outliers) for s in range(nbuf)]
     xs = [x.cuda() for x in xs_cpu]
     res = ops.quantize(xs[0], 0, 1, precision=precision)
     outs = [[torch.empty_like(t) for t in res[:2]] for _ in range(nbuf)]
     ok = None
     if check:
+        from oracle import nvfp4_oracle as T
         if precision == "nvfp4":
             e = T.quantize_nvfp4(xs_cpu[0], 0, 1)
             ok = (torch.equal(res[0].cpu(), e[0]) and torch.equal(res[1].cpu().view(torch.uint8), e[1])
@@ -172,10 +179,14 @@ def cpu_quantize_baseline(shape, outliers, budget_s=10.0):
 
 
 # --------------------------------------------------------------------------- linear
+# the sixteen E2M1 codes (test/test_linear_bench.py:18-35 of the reference holds the same table)
+E2M1_VALUES = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0]
+
+
 def gpu_dequant(q, rows):
-    from oracle import nvfp4_oracle as T
+    """fp32 dequantization of a packed operand with torch ops on the GPU (the GEMM check's reference)."""
     packed, sf, gs = q
-    lut = T.E2M1_LUT.cuda()
+    lut = torch.tensor(E2M1_VALUES, dtype=torch.float32, device="cuda")
     v = torch.stack((lut[(packed & 0xF).long()], lut[(packed >> 4).long()]), dim=-1).reshape(rows, -1, 16)
     s = sf.permute(1, 0, 2).reshape(sf.shape[1], -1)[:rows].float() * gs
     return (v * s.unsqueeze(-1)).reshape(rows, -1)
@@ -429,7 +440,10 @@ def main():
 
     if args.workload == "traffic":
         return run_traffic(ops)
-    check = not args.no_check
+    check = not args.no_check  # the GEMM checks: fp32 dequantize-matmul with torch ops on the GPU
+    # The CPU leg (the only user of oracle/): the oracle timed on the host cores as `cpu_baseline`, and the
+    # same oracle as the checker of the quantizers' GPU output.  --no-cpu-baseline skips all of it.
+    check_cpu = check and not args.no_cpu_baseline
     S, W = args.steps, args.warmup
     SETTLE_MS = args.settle_ms
     line = {"n_gpus": 1, "steps": S, "warmup": W, "warmup_settle_ms": SETTLE_MS, "higher_is_better": True,
@@ -438,10 +452,10 @@ def main():
     quant = None
     if args.workload in ("all", "quantize"):
         quant = {
-            "cfg2_nvfp4": bench_quantize(ops, (8192, 4096), "nvfp4", S, W, True, check, key="quantize_nvfp4_8192x4096"),
-            "cfg2_fp8e4m3": bench_quantize(ops, (8192, 4096), "fp8e4m3", S, W, True, check, key="quantize_fp8_8192x4096"),
-            "cfg2_int8": bench_quantize(ops, (8192, 4096), "int8", S, W, True, check, key="quantize_int8_8192x4096"),
-            "cfg1_nvfp4": bench_quantize(ops, (4096, 4096), "nvfp4", S, W, False, check),
+            "cfg2_nvfp4": bench_quantize(ops, (8192, 4096), "nvfp4", S, W, True, check_cpu, key="quantize_nvfp4_8192x4096"),
+            "cfg2_fp8e4m3": bench_quantize(ops, (8192, 4096), "fp8e4m3", S, W, True, check_cpu, key="quantize_fp8_8192x4096"),
+            "cfg2_int8": bench_quantize(ops, (8192, 4096), "int8", S, W, True, check_cpu, key="quantize_int8_8192x4096"),
+            "cfg1_nvfp4": bench_quantize(ops, (4096, 4096), "nvfp4", S, W, False, check_cpu),
         }
         for k_, v in quant.items():
             log(f"[bench] {k_}: {v['ms'] * 1e3:.1f} us  {v['GB/s']:.0f} GB/s  "
