@@ -39,6 +39,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+HOST = {}                   # host core counts of the CPU leg, filled in main()
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16 MFMA (identical rates)
 
@@ -173,7 +174,7 @@ def cpu_quantize_baseline(shape, outliers, budget_s=10.0):
         ts.append(time.perf_counter() - t0)
     t = sorted(ts)[len(ts) // 2]
     return {"value": quant_bytes(shape, "nvfp4") / t / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
-            "kind": "port",
+            "host": dict(HOST), "kind": "port",
             "sample": f"full nvfp4 quantize of one {shape[0]}x{shape[1]} bf16 tensor, median of {len(ts)} runs "
                       f"({time.perf_counter() - t_begin:.0f} s)"}
 
@@ -196,8 +197,13 @@ def linear_bytes(m, n, k):
     return (m + n) * k // 2 + ((m + 15) // 16 * 16 + (n + 15) // 16 * 16) * k // 16 + m * n * 2 + 8
 
 
-def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True, key=None, with_quantize=False):
-    a, b = make_input((m, k), seed=0), make_input((n, k), seed=1, std=wstd)
+def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True, key=None, with_quantize=False, gen_on_gpu=False):
+    if gen_on_gpu:  # very large operands: the host generator would take longer than the measurement
+        g = torch.Generator(device="cuda").manual_seed(0)
+        a = torch.empty((m, k), dtype=torch.float32, device="cuda").normal_(generator=g).to(torch.bfloat16)
+        b = (torch.empty((n, k), dtype=torch.float32, device="cuda").normal_(generator=g) * wstd).to(torch.bfloat16)
+    else:
+        a, b = make_input((m, k), seed=0), make_input((n, k), seed=1, std=wstd)
     aq, bq = ops.quantize(a.cuda(), 0, 1), ops.quantize(b.cuda(), 0, 1)
     out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
     ops.linear(*aq, *bq, out=out)
@@ -394,7 +400,7 @@ def cpu_linear_baseline(n, k, rows=8192, budget_s=10.0):
         ts.append(time.perf_counter() - t0)
     t = sorted(ts)[len(ts) // 2]
     return {"value": 2.0 * rows * n * k / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
-            "kind": "port",
+            "host": dict(HOST), "kind": "port",
             "sample": f"oracle fp32 dequantize + torch.matmul of the whole M={rows} N={n} K={k} problem, median of "
                       f"{len(ts)} runs ({time.perf_counter() - t_begin:.0f} s)"}
 
@@ -435,7 +441,17 @@ def main():
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1")
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
-    torch.set_num_threads(min(16, os.cpu_count() or 1))
+    # CPU leg: every host core the process may run on (a container's share can be smaller than
+    # os.cpu_count(); both are reported next to the thread count torch actually uses)
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        usable = os.cpu_count() or 1
+    env_cap = os.environ.get("OMP_NUM_THREADS")
+    threads = min(usable, int(env_cap)) if env_cap and env_cap.isdigit() and int(env_cap) > 0 else usable
+    torch.set_num_threads(max(1, threads))
+    HOST.update({"cpu_count": os.cpu_count(), "usable_cores": usable, "omp_num_threads_env": env_cap,
+                 "threads": torch.get_num_threads()})
     from ac4k_kernel_amd import ops
 
     if args.workload == "traffic":
@@ -516,6 +532,18 @@ def main():
             log("[bench] linear 8192^3 by output/bias dtype, TFLOP/s: "
                 + ", ".join(f"{k_} {v['TFLOP/s']:.0f}" for k_, v in epi.items()))
             line["linear_epilogues"] = epi
+            # the shapes the reference itself times (test/test_linear_tflops.py:190-203), M x N x K
+            refs = {}
+            for (m, n, k) in ((75600, 5120, 5120), (75600, 13824, 5120), (75600, 5120, 6912), (75600, 5120, 13824)):
+                refs[f"M{m}_N{n}_K{k}"] = bench_linear(ops, m, n, k, max(5, S // 3), W, wstd=0.02, check=check, gen_on_gpu=True)
+                torch.cuda.empty_cache()
+            for k_, v in refs.items():
+                log(f"[bench] ref shape {k_}: {v['ms']:.3f} ms  {v['TFLOP/s']:.1f} TFLOP/s  "
+                    f"{100 * v['roofline']['frac']:.1f}% of MFMA peak  ok={v['within_1e-2_of_fp32_dequant_matmul']}")
+                line[f"linear_{k_}_tflops"] = v["TFLOP/s"]
+                line[f"linear_{k_}_frac"] = v["roofline"]["frac"]
+                line[f"linear_{k_}_ok"] = v["within_1e-2_of_fp32_dequant_matmul"]
+            line["ref_shapes"] = refs
         if quant is not None:
             line["quantize"] = quant
     else:
@@ -525,7 +553,44 @@ def main():
                      "roofline": q["roofline"], "parity": q["bit_exact_vs_oracle"], "quantize": quant})
         if "cpu_baseline" in quant:
             line["cpu_baseline"] = quant["cpu_baseline"]
+    # The quantize half of the metric as flat scalar keys of the line, and a short summary as the LAST
+    # lines of stderr (what a captured tail keeps).
+    summary = []
+    if quant is not None:
+        for key, tag in (("cfg1_nvfp4", "quantize_nvfp4_4096x4096"), ("cfg2_nvfp4", "quantize_nvfp4_8192x4096"),
+                         ("cfg2_fp8e4m3", "quantize_fp8_8192x4096"), ("cfg2_int8", "quantize_int8_8192x4096")):
+            q = quant[key]
+            line[f"{tag}_gbs"] = q["GB/s"]
+            line[f"{tag}_frac"] = q["roofline"]["frac"]
+            line[f"{tag}_us"] = q["ms"] * 1e3
+            line[f"{tag}_bit_exact"] = q["bit_exact_vs_oracle"]
+            summary.append(f"{tag}: {q['ms'] * 1e3:.1f} us  {q['GB/s']:.0f} GB/s  frac {q['roofline']['frac']:.3f} of 8 TB/s  "
+                           f"bit_exact={q['bit_exact_vs_oracle']}")
+            if "global_scale_given" in q:
+                g_ = q["global_scale_given"]
+                line[f"{tag}_kernel_alone_frac"] = g_["frac_of_hbm_peak"]
+                summary[-1] += f"  (kernel alone, scale given: {g_['ms'] * 1e3:.1f} us, frac {g_['frac_of_hbm_peak']:.3f})"
+        if "cpu_baseline" in quant:
+            c = quant["cpu_baseline"]
+            line["quantize_cpu_baseline_gbs"] = c["value"]
+            summary.append(f"quantize cpu oracle: {c['value']:.2f} GB/s on {c['cores']} threads "
+                           f"(os.cpu_count {HOST.get('cpu_count')}, usable {HOST.get('usable_cores')}, "
+                           f"OMP_NUM_THREADS {HOST.get('omp_num_threads_env')})")
+    if "roofline" in line and line.get("unit") == "TFLOP/s":
+        summary.append(f"linear 8192^3: {line['ms_per_step']:.3f} ms  {line['value']:.1f} TFLOP/s  "
+                       f"frac {line['roofline']['frac']:.3f} of 2.5 PFLOP/s  ok={line.get('parity')}")
+    for k_ in ("decode", "linear_shapes"):
+        if k_ in line:
+            summary.append(k_ + ": " + "  ".join(f"{n_.split('_', 1)[1]} {v['ms'] * 1e3:.1f}us/{v['roofline']['frac']:.2f}"
+                                                 for n_, v in line[k_].items()))
+    if "ref_shapes" in line:
+        summary.append("ref shapes: " + "  ".join(f"{n_} {v['TFLOP/s']:.0f}TF/{v['roofline']['frac']:.2f}"
+                                                  for n_, v in line["ref_shapes"].items()))
+    line["host"] = dict(HOST)
     print(json.dumps(line), flush=True)
+    log("[bench] ---- summary (time, throughput, fraction of the roofline) ----")
+    for ln in summary:
+        log("[bench] " + ln)
 
 
 if __name__ == "__main__":

@@ -75,3 +75,25 @@ def test_python_checks_without_gpu():
     with pytest.raises(RuntimeError):  # CPU tensor: "must be a CUDA tensor"
         ops.quantize_fp8(torch.empty((4, 64), dtype=torch.float8_e4m3fn), torch.empty(16), x,
                          torch.tensor(448.0), 0, 1, False)
+
+
+def test_reference_import_lines_resolve():
+    """The import lines of the reference's callers (test/test_quantize_bench.py:7,
+    test/test_linear_bench.py:4) resolve to this library through the `ac4k_kernel` alias package."""
+    import ac4k_kernel
+    import ac4k_kernel_amd
+    from ac4k_kernel.ops import linear, quantize
+    from ac4k_kernel.ops.linear import Ac4kLinearOp
+    from ac4k_kernel.ops.quant import Ac4kQuantizeOp
+    import ac4k_kernel._rocm_ops as binding
+    assert ac4k_kernel.get_backend() == "rocm" and ac4k_kernel.get_arch() == "gfx950"
+    assert ac4k_kernel.get_info() == ac4k_kernel_amd.get_info()
+    assert quantize is ac4k_kernel_amd.ops.quantize and linear is ac4k_kernel_amd.ops.linear
+    assert binding is ac4k_kernel_amd._rocm_ops and binding.__backend__ == "rocm"
+    assert issubclass(Ac4kLinearOp, __import__("torch").nn.Module) and Ac4kQuantizeOp is not None
+    for name in ("quantize_nvfp4", "quantize_fp8", "quantize_int8", "linear_nvfp4"):
+        assert getattr(ac4k_kernel, name) is getattr(ac4k_kernel_amd, name)
+        assert getattr(ac4k_kernel.ops, name) is getattr(ac4k_kernel_amd.ops, name)
+    # the alias must not pull in the checker either
+    for f in ("__init__.py", os.path.join("ops", "__init__.py")):
+        assert "oracle" not in open(os.path.join(ROOT, "ac4k_kernel", f)).read()

@@ -91,8 +91,15 @@ def gpu_dequant(q, rows):
     return (v * s.unsqueeze(-1)).reshape(rows, -1)
 
 
-@pytest.mark.parametrize("m,n,k,wstd", [(4096, 4096, 4096, 1.0), (2048, 14336, 4096, 0.02), (16, 4096, 14336, 0.02),
-                                        (8192, 8192, 8192, 1.0)])
+# configuration 3, all eight LLM shapes of configuration 4, the headline 8192^3, and two of the
+# reference's own timed shapes (test/test_linear_tflops.py:190-203: M = 75600 leaves a ragged last
+# tile row and an output of more than 2^30 elements)
+LARGE_SHAPES = [(4096, 4096, 4096, 1.0), (8192, 8192, 8192, 1.0)]
+LARGE_SHAPES += [(m, n, k, 0.02) for (n, k) in ((14336, 4096), (4096, 14336)) for m in (16, 128, 2048, 8192)]
+LARGE_SHAPES += [(75600, 5120, 5120, 0.02), (75600, 13824, 5120, 0.02)]
+
+
+@pytest.mark.parametrize("m,n,k,wstd", LARGE_SHAPES)
 def test_large_shapes(m, n, k, wstd):
     a, b = make_input((m, k), seed=0), make_input((n, k), seed=1, std=wstd)
     aq, bq = gpu_quant(a), gpu_quant(b)
@@ -104,10 +111,12 @@ def test_large_shapes(m, n, k, wstd):
     fa = T.dequantize_nvfp4(ca[0][rows], ca[1][:, rows].contiguous(), ca[2])
     fb = T.dequantize_nvfp4(cb[0][cols], cb[1][:, cols].contiguous(), cb[2])
     ref = (fa @ fb.t()).to(torch.bfloat16)
-    torch.testing.assert_close(d.cpu()[rows][:, cols], ref, atol=ATOL, rtol=RTOL)
+    torch.testing.assert_close(d[rows.cuda()][:, cols.cuda()].cpu(), ref, atol=ATOL, rtol=RTOL)
     # (2) the whole matrix against a torch fp32 dequantize-matmul on the GPU
     full = (gpu_dequant(aq, m) @ gpu_dequant(bq, n).t()).to(torch.bfloat16)
     torch.testing.assert_close(d, full, atol=ATOL, rtol=RTOL)
+    del full, d
+    torch.cuda.empty_cache()
 
 
 @pytest.mark.parametrize("m,n,k", [(4096, 4096, 4096), (128, 4096, 14336), (8, 28672, 8192), (2048, 4096, 14336)])
