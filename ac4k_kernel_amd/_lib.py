@@ -29,6 +29,8 @@ SIGNATURES = {
     "ac4k_linear_nvfp4_skinny_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "ac4k_linear_nvfp4_skinny": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64,
                                         _vp, _i64, _vp]),
+    "ac4k_linear_nvfp4_skinny_static": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64,
+                                               _vp]),
     "ac4k_linear_nvfp4_fused_bf16": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int,
                                             _i64, _i64, _i64, _vp, _i64, _vp]),
 }

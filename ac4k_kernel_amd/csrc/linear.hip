@@ -14,6 +14,7 @@
 #include <string.h>
 
 #include <atomic>
+#include <mutex>
 #include <type_traits>
 
 #include "ac4k_common.h"
@@ -1579,12 +1580,14 @@ extern "C" __attribute__((visibility("default"))) int64_t ac4k_linear_nvfp4_skin
   return 0;
 }
 
-extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_skinny(void *D, int d_dtype, const void *A, const void *A_sf, const float *A_gs,
-                                        const void *B, const void *B_sf, const float *B_gs, const void *bias,
-                                        int bias_dtype, int64_t M, int64_t N, int64_t K, void *workspace,
-                                        int64_t workspace_bytes, ac4k_stream_t stream) {
+namespace ac4k {
+
+// body of the two workspace-assisted entry points (caller's workspace / the library's static array)
+static int linear_skinny_impl(void *D, int d_dtype, const void *A, const void *A_sf, const float *A_gs, const void *B,
+                              const void *B_sf, const float *B_gs, const void *bias, int bias_dtype, int64_t M,
+                              int64_t N, int64_t K, void *workspace, int64_t workspace_bytes, hipStream_t st,
+                              const char *what) {
   AC4K_REQUIRE(D && A && A_sf && A_gs && B && B_sf && B_gs, "null pointer argument");
-  hipStream_t st = (hipStream_t)stream;
   TilePlan mp;
   if (M > 32 && mid_plan(M, N, K, mp)) {  // few tiles, long K: split-K over the tile kernel
     AC4K_REQUIRE((((uintptr_t)A | (uintptr_t)B) & 15) == 0, "A and B must be 16-byte aligned");
@@ -1595,7 +1598,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_skinny(v
                   static_cast<const uint32_t *>(A_sf), static_cast<const uint32_t *>(B_sf), A_gs, B_gs, bias,
                   M, N, K, align_up(M, 16), align_up(N, 16)};
     if (int rc = dispatch_mid(la, mp, static_cast<float *>(workspace), d_dtype, bias_dtype, st)) return rc;
-    return check_launch("ac4k_linear_nvfp4_skinny");
+    return check_launch(what);
   }
   SkinnyPlan p;
   const bool ok = skinny_plan(M, N, K, p);
@@ -1603,7 +1606,61 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_skinny(v
   AC4K_REQUIRE(((uintptr_t)A & 15) == 0, "A must be 16-byte aligned");
   if (int rc = run_skinny(D, d_dtype, A, A_sf, A_gs, B, B_sf, B_gs, bias, bias_dtype, M, N, K, p, workspace, st))
     return rc;
-  return check_launch("ac4k_linear_nvfp4_skinny");
+  return check_launch(what);
+}
+
+// ---------------------------------------------------------------------------
+// Scratch of the entry point that allocates nothing: one array per GPU, held until the process ends.
+// In host code the array's name is only a handle: its device address comes from hipGetSymbolAddress,
+// once per device with that device current, and that pointer is what the kernels are given.
+// ---------------------------------------------------------------------------
+constexpr int64_t STATIC_SCRATCH_BYTES = AC4K_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+static int static_scratch(void **ptr_out) {
+  constexpr int MAX_DEV = 64;
+  static void *ptrs[MAX_DEV] = {};
+  static std::mutex mu;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return set_error("hipGetDevice: %s", hipGetErrorString(e));
+  AC4K_REQUIRE(dev >= 0 && dev < MAX_DEV, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) return set_error("hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    ptrs[dev] = p;
+  }
+  *ptr_out = ptrs[dev];
+  return 0;
+}
+
+}  // namespace ac4k
+
+extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_skinny(void *D, int d_dtype, const void *A, const void *A_sf, const float *A_gs,
+                                        const void *B, const void *B_sf, const float *B_gs, const void *bias,
+                                        int bias_dtype, int64_t M, int64_t N, int64_t K, void *workspace,
+                                        int64_t workspace_bytes, ac4k_stream_t stream) {
+  return linear_skinny_impl(D, d_dtype, A, A_sf, A_gs, B, B_sf, B_gs, bias, bias_dtype, M, N, K, workspace,
+                            workspace_bytes, (hipStream_t)stream, "ac4k_linear_nvfp4_skinny");
+}
+
+extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_skinny_static(void *D, int d_dtype, const void *A, const void *A_sf,
+                                               const float *A_gs, const void *B, const void *B_sf,
+                                               const float *B_gs, const void *bias, int bias_dtype, int64_t M,
+                                               int64_t N, int64_t K, ac4k_stream_t stream) {
+  const int64_t need = ac4k_linear_nvfp4_skinny_workspace_bytes(M, N, K);
+  AC4K_REQUIRE(need > 0, "no workspace-assisted path for this shape (ac4k_linear_nvfp4_skinny_workspace_bytes returns 0)");
+  AC4K_REQUIRE(need <= STATIC_SCRATCH_BYTES,
+               "shape needs %lld bytes of scratch, the static scratch holds %lld: use ac4k_linear_nvfp4_skinny with a "
+               "workspace of the caller",
+               (long long)need, (long long)STATIC_SCRATCH_BYTES);
+  void *ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  // the partial sums are written before they are read: nothing in the array has to start at zero
+  return linear_skinny_impl(D, d_dtype, A, A_sf, A_gs, B, B_sf, B_gs, bias, bias_dtype, M, N, K, ws,
+                            STATIC_SCRATCH_BYTES, (hipStream_t)stream, "ac4k_linear_nvfp4_skinny_static");
 }
 
 extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_fused_bf16(void *D, int d_dtype, const void *X, void *X_q, void *X_sf,

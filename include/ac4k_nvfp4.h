@@ -116,6 +116,22 @@ int ac4k_linear_nvfp4_skinny(void *D, int d_dtype, const void *A, const void *A_
                              int bias_dtype, int64_t M, int64_t N, int64_t K, void *workspace,
                              int64_t workspace_bytes, ac4k_stream_t stream);
 
+/* ac4k_linear_nvfp4_skinny without the workspace argument, for callers that cannot allocate
+ * device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  It has no counterpart in the reference.  The partial sums go to an array of
+ * AC4K_STATIC_SCRATCH_BYTES that is part of the library's device image: every GPU the library runs
+ * on holds one copy from the first call on that GPU until the process ends, and the call itself
+ * allocates and frees nothing.  Same shapes, checks and results as ac4k_linear_nvfp4_skinny; a
+ * shape whose ac4k_linear_nvfp4_skinny_workspace_bytes exceeds AC4K_STATIC_SCRATCH_BYTES is
+ * rejected.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (two
+ * streams, two host threads on different streams) race on it; calls on one stream do not.  Make the
+ * first call on a GPU outside graph capture (it looks up the array's address). */
+#define AC4K_STATIC_SCRATCH_BYTES (32ll << 20)
+int ac4k_linear_nvfp4_skinny_static(void *D, int d_dtype, const void *A, const void *A_sf,
+                                    const float *A_gs, const void *B, const void *B_sf,
+                                    const float *B_gs, const void *bias, int bias_dtype, int64_t M,
+                                    int64_t N, int64_t K, ac4k_stream_t stream);
+
 /* Fused decode-sized linear: quantize(X,0,1) followed by linear(...) in one call.  No single
  * reference function: it equals the composition the reference's tests make
  * (test/test_linear_bench.py:128-137) — the activation bytes, scales and global scale it
