@@ -21,6 +21,7 @@ SIGNATURES = {
     "ac4k_last_error": (_cp, []),
     "ac4k_global_scale_bf16": (_int, [_vp, _vp, _i64, _f32, _vp]),
     "ac4k_set_quantize_sync_timeout_us": (None, [_i64]),
+    "ac4k_debug_last_quantize_path": (_int, []),
     "ac4k_quantize_nvfp4": (_int, [_vp, _vp, _vp, _vp] + [_i64] * 8 + [_int, _vp]),
     "ac4k_quantize_nvfp4_bf16": (_int, [_vp, _vp, _vp, _vp] + [_i64] * 8 + [_int, _f32, _vp]),
     "ac4k_quantize_fp8": (_int, [_vp, _vp, _vp, _vp] + [_i64] * 8 + [_int, _vp]),
@@ -31,6 +32,7 @@ SIGNATURES = {
                                         _vp, _i64, _vp]),
     "ac4k_linear_nvfp4_skinny_static": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64,
                                                _vp]),
+    "ac4k_set_linear_tuning": (_int, [_int, _int, _int, _int]),
     "ac4k_linear_nvfp4_fused_bf16": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int,
                                             _i64, _i64, _i64, _vp, _i64, _vp]),
 }

@@ -39,10 +39,10 @@ def needs_build() -> bool:
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def build(force: bool = False, verbose: bool = True, extra_flags=(), out: str = LIB_PATH) -> str:
-    if not force and out == LIB_PATH and not needs_build():
-        return LIB_PATH
-    cmd = [HIPCC] + FLAGS + list(extra_flags) + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", out]
+OBJ_DIR = os.path.join(PKG_DIR, "_obj")
+
+
+def _run(cmd, verbose):
     if verbose:
         print("[ac4k build]", " ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -51,6 +51,30 @@ def build(force: bool = False, verbose: bool = True, extra_flags=(), out: str = 
         raise RuntimeError("hipcc failed:\n" + log)
     if verbose and log.strip():
         print(log)
+
+
+def build(force: bool = False, verbose: bool = True, extra_flags=(), out: str = LIB_PATH) -> str:
+    """One object per source file, compiled side by side, then one link.  An object is reused when it
+    is newer than its source, the headers and this file (only for the default flags and output)."""
+    if not force and out == LIB_PATH and not needs_build():
+        return LIB_PATH
+    from concurrent.futures import ThreadPoolExecutor
+    reuse = not force and out == LIB_PATH and not extra_flags
+    tag = "" if out == LIB_PATH else "." + os.path.splitext(os.path.basename(out))[0]
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    compile_flags = [f for f in FLAGS if f != "-shared"] + list(extra_flags)
+    common = HEADERS + [os.path.abspath(__file__)]
+    jobs, objs = [], []
+    for src_name in SOURCES:
+        src = os.path.join(CSRC, src_name)
+        obj = os.path.join(OBJ_DIR, src_name + tag + ".o")
+        objs.append(obj)
+        fresh = reuse and os.path.exists(obj) and all(os.path.getmtime(d) < os.path.getmtime(obj) for d in [src] + common)
+        if not fresh:
+            jobs.append([HIPCC] + compile_flags + ["-c", src, "-o", obj])
+    with ThreadPoolExecutor(max_workers=max(1, len(jobs))) as pool:
+        list(pool.map(lambda c: _run(c, verbose), jobs))
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fvisibility=hidden"] + objs + ["-o", out], verbose)
     return out
 
 

@@ -1045,13 +1045,16 @@ struct TilePlan {
 // second launch.  Big problems (192 or more of the largest tiles) take the largest tile as is.
 // The time per stage is a fit to measured loops of the five tile shapes: per 16-k sub-step about
 // 14 cycles per MFMA plus 5 per decode instruction, 400 cycles per stage on top, at 2.1 GHz.
+// Tuning overrides (ac4k_set_linear_tuning): a forced tile plan packed as mi | nj << 8 | splits << 16
+// (0 = the cost model decides) and a forced K slice of the decode-sized kernel (0 = automatic).
+static std::atomic<uint32_t> g_forced_tile_plan{0};
+static std::atomic<int> g_forced_skinny_ks{0};
+
 static TilePlan tile_plan(int64_t M, int64_t N, int64_t K, bool allow_split) {
   TilePlan best{M <= 128 ? 2 : 4, 4, 1, 0};
-  if (const char *e = getenv("AC4K_TILE_PLAN")) {  // tuning aid: "mi,nj,splits"
-    int mi = 0, nj = 0, sp = 0;
-    if (sscanf(e, "%d,%d,%d", &mi, &nj, &sp) == 3 && (mi == 2 || mi == 4) && (nj == 1 || nj == 2 || nj == 4) &&
-        !(mi == 4 && nj == 1) && sp >= 1 && sp <= K / P_BK && (sp == 1 || allow_split))
-      return TilePlan{mi, nj, sp, sp > 1 ? (int64_t)sp * M * N * 4 : 0};
+  if (const uint32_t f = g_forced_tile_plan.load(std::memory_order_relaxed)) {
+    const int mi = f & 0xff, nj = (f >> 8) & 0xff, sp = (int)(f >> 16);
+    if (sp <= K / P_BK && (sp == 1 || allow_split)) return TilePlan{mi, nj, sp, sp > 1 ? (int64_t)sp * M * N * 4 : 0};
   }
   const int64_t stages = K / P_BK;
   if (ceil_div(M, 64 * best.mi) * ceil_div(N, 256) >= 192) return best;
@@ -1369,7 +1372,7 @@ struct SkinnyPlan {
 static bool skinny_plan(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
   if (M < 1 || M > 32 || K % SK_STEP != 0 || N < 1) return false;
   int ks = 1024;
-  if (const char *e = getenv("AC4K_SKINNY_KS")) ks = atoi(e);  // tuning aid
+  if (const int f = g_forced_skinny_ks.load(std::memory_order_relaxed)) ks = f;  // 256, 512 or 1024
   while (ks > SK_STEP && K % ks != 0) ks >>= 1;
   p.groups = ceil_div(N, SK_ROWS);
   // short problems: use smaller slices to get enough workgroups in flight
@@ -1679,4 +1682,19 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_fused_bf
                           st))
     return rc;
   return check_launch("ac4k_linear_nvfp4_fused_bf16");
+}
+
+extern "C" __attribute__((visibility("default"))) int ac4k_set_linear_tuning(int mi, int nj, int splits, int skinny_ks) {
+  if (mi == 0 && nj == 0 && splits == 0) {
+    ac4k::g_forced_tile_plan.store(0);
+  } else {
+    AC4K_REQUIRE((mi == 2 || mi == 4) && (nj == 1 || nj == 2 || nj == 4) && !(mi == 4 && nj == 1) && splits >= 1 &&
+                     splits <= 0xffff,
+                 "tile plan must be mi in {2,4}, nj in {1,2,4} (not 4,1), 1 <= splits (got %d,%d,%d)", mi, nj, splits);
+    ac4k::g_forced_tile_plan.store((uint32_t)mi | ((uint32_t)nj << 8) | ((uint32_t)splits << 16));
+  }
+  AC4K_REQUIRE(skinny_ks == 0 || skinny_ks == 256 || skinny_ks == 512 || skinny_ks == 1024,
+               "skinny_ks must be 0 (automatic), 256, 512 or 1024 (got %d)", skinny_ks);
+  ac4k::g_forced_skinny_ks.store(skinny_ks);
+  return 0;
 }

@@ -13,6 +13,7 @@
 // reduce amax inside the wavefront with DPP, and store packed words.
 #include <atomic>
 #include <mutex>
+#include <type_traits>
 
 #include "ac4k_common.h"
 
@@ -27,16 +28,6 @@ __global__ void zero_u32_kernel(uint32_t *p) { *p = 0u; }
 constexpr int AMAX_THREADS = 256;
 constexpr int AMAX_UNROLL = 4;
 constexpr int AMAX_MAX_BLOCKS = 1024;  // four workgroups per CU
-constexpr int AMAX_SLOTS = 32;        // concurrent (device, stream) pairs served by the one-launch path
-
-// Per-slot scratch of the two-kernel reduction: pass 1 deposits one maximum per block, the
-// consumer (the quantize kernel, or a one-block finalize kernel) reduces the deposits.  A slot
-// belongs to one (device, stream) pair, whose calls the stream serialises, so a slot is never
-// used by two reductions at once.
-struct AmaxScratch {
-  uint32_t partial[AMAX_SLOTS][AMAX_MAX_BLOCKS];
-};
-__device__ AmaxScratch g_amax_scratch;
 
 // |x| maximum of this block's share of x[0..n) as a bf16 bit pattern (valid in thread 0).
 __device__ __forceinline__ uint32_t block_absmax_bf16(const uint16_t *__restrict__ x, int64_t n, int64_t head,
@@ -76,36 +67,10 @@ __device__ __forceinline__ uint32_t block_absmax_bf16(const uint16_t *__restrict
   return m;
 }
 
-// Pass 1 of the two-kernel reduction: every block deposits its maximum (no atomics: atomics of
-// many blocks on one address serialise at about 25-50 ns each across the 8 XCDs).
-__global__ __launch_bounds__(AMAX_THREADS) void amax_partials_bf16_kernel(const uint16_t *__restrict__ x, int64_t n,
-                                                                          int64_t head, int64_t nvec, int slot) {
-  const uint32_t m = block_absmax_bf16(x, n, head, nvec);
-  if (threadIdx.x == 0) g_amax_scratch.partial[slot][blockIdx.x] = m;
-}
-
-// max over the deposits of a slot, by every thread of the calling block (all must call it)
-__device__ __forceinline__ uint32_t reduce_amax_partials(int slot, int npart) {
-  uint32_t r = 0;
-  for (int b = threadIdx.x; b < npart; b += blockDim.x) r = umax32(r, g_amax_scratch.partial[slot][b]);
-  r = group_umax<64>(r);
-  __shared__ uint32_t red[16];
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = r;
-  __syncthreads();
-  r = 0;
-  for (int w = 0; w < (int)(blockDim.x >> 6); ++w) r = umax32(r, red[w]);
-  return r;
-}
-
-// Pass 2 when only the scale is wanted: one block.
-__global__ __launch_bounds__(AMAX_THREADS) void amax_finalize_kernel(float *__restrict__ gs, int slot, int npart,
-                                                                     float max_scale) {
-  const uint32_t r = reduce_amax_partials(slot, npart);
-  if (threadIdx.x == 0) *gs = bf16_bits_to_f32(r) / max_scale;
-}
-
-// Fallback when every slot is taken: *gs zeroed by a fill kernel, then an atomic max per block.
-// Division is monotone, so the max of the per-block quotients is the quotient of the max;
+// Global scale without any memory of the library's own: *gs is zeroed by a fill kernel, then every
+// block folds its quotient in with an atomic max - but only when the quotient beats the value it
+// reads first, so that after the first few blocks almost none touches the (cross-XCD, serialising)
+// atomic.  Division is monotone, so the max of the per-block quotients is the quotient of the max;
 // non-negative floats order like unsigned integers.
 __global__ __launch_bounds__(AMAX_THREADS) void amax_scale_bf16_atomic_kernel(
     uint32_t *__restrict__ gs_bits, const uint16_t *__restrict__ x, int64_t n, int64_t head, int64_t nvec,
@@ -147,26 +112,6 @@ static dim3 crossmajor_grid(const QuantGeom &g, int64_t kblocks, int64_t rowbloc
 // the reduce blocks)
 static int crossmajor_lead_fast(int64_t d1, int64_t s1, int64_t sK, int64_t kblocks) {
   return d1 > 1 && s1 < sK && kblocks <= 65535;
-}
-
-// Where a quantize kernel gets the global scale from: a device scalar (slot < 0), or the
-// deposits of the amax pass, in which case it also publishes the scale through `gs`.
-struct GlobalScaleSrc {
-  float *gs;
-  int slot, npart;
-  float max_scale;
-};
-
-// 1 / global_scale for the calling block (every thread must call it).
-__device__ __forceinline__ float load_alpha(const GlobalScaleSrc &src, bool publisher) {
-  float gs;
-  if (src.slot < 0) {
-    gs = *src.gs;
-  } else {
-    gs = bf16_bits_to_f32(reduce_amax_partials(src.slot, src.npart)) / src.max_scale;
-    if (publisher && threadIdx.x == 0) *src.gs = gs;
-  }
-  return 1.0f / gs;
 }
 
 // Correctly rounded fp32 reciprocals of the 128 non-negative E4M3 codes (entry 0 is 0, entry
@@ -251,11 +196,11 @@ __device__ __forceinline__ uint4 swizzle_fp8_pair(uint4 v, int lane) {
 //   ITER = wave passes per workgroup (independent loads in flight per lane)
 template <int CPR, int ITER, bool SWIZZLE>
 __global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
-    uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in, GlobalScaleSrc gsrc,
+    uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in, const float *__restrict__ gs_ptr,
     QuantGeom g) {
   __shared__ float lut[128];
   load_rcp_table(lut);
-  const float alpha = load_alpha(gsrc, blockIdx.x == 0 && blockIdx.y == 0);
+  const float alpha = 1.0f / *gs_ptr;
   constexpr int LPR = 8 * CPR;   // lanes per row
   constexpr int RW = 64 / LPR;   // rows per wave pass
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -299,11 +244,11 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_rowmajor_kernel(
 // contiguous one), and writes 32 packed bytes and one scale dword.
 template <bool SWIZZLE>
 __global__ __launch_bounds__(256) void quantize_nvfp4_generic_kernel(
-    uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in, GlobalScaleSrc gsrc,
+    uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in, const float *__restrict__ gs_ptr,
     QuantGeom g) {
   __shared__ float lut[128];
   load_rcp_table(lut);
-  const float alpha = load_alpha(gsrc, blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0);
+  const float alpha = 1.0f / *gs_ptr;
   const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t chunk = blockIdx.y, lead = blockIdx.z + g.lead0;
   if (r >= g.Rp) return;
@@ -352,19 +297,19 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_generic_kernel(
 // produced, so a two-kernel quantize reads its input twice.  Here every workgroup keeps its share
 // of the input in registers (NV 16-byte vectors per lane, 1024 lanes, one workgroup per CU),
 // publishes its maximum, waits until every workgroup has published, and quantizes from registers:
-// the input crosses the memory bus once.
+// the input crosses the memory bus once, and the call is ONE launch.
 //
 // Grid synchronisation: arrive[w] = (tag << 16) | bf16 maximum, one word per workgroup, written
-// and polled with device-coherent accesses.  The tag is a 16-bit launch number kept in device
-// memory (epoch[slot] + 1, never the 0 of untouched memory) and advanced by the repair launch, so
-// nothing is ever cleared and a call replays correctly from a captured graph.  The wait is bounded
-// (timeout in 100 MHz ticks).  A workgroup that times out - its peers were not all resident, e.g.
-// two such kernels sharing the GPU - returns without writing and without setting done[w]; so does
-// every workgroup when the scale is not a positive finite number.  The REPAIR instantiation is
-// launched right behind on the same stream: workgroups whose done[w] carries the tag leave at once,
-// the others redo their share with the maxima that are all published by then, using the full-range
-// arithmetic of the two-kernel path.  Every launch uses the same number of workgroups on a device,
-// so each launch overwrites every word the next one polls.
+// and polled with device-coherent accesses.  The tag is a 16-bit launch number (never the 0 of
+// untouched memory) that the host hands out per slot and passes as a kernel argument, so nothing
+// is ever cleared.  Every launch on a device uses the same number of workgroups, so each launch
+// overwrites every word the next one polls.  The wait is bounded (timeout in 100 MHz ticks): a
+// workgroup whose peers have not all published by then - they were not all resident (the GPU is
+// shared with other kernels), or another launch is using the same slot - stops waiting and computes
+// the maxima of the missing workgroups' shares itself, from memory.  Every workgroup therefore
+// finishes on its own whatever else runs on the GPU; words of a foreign tag are never used.  A
+// scale that is not a positive finite number takes the full-range arithmetic of the two-kernel
+// path in the same launch.
 //
 // Work split: the tensor is cut into groups of GS = min(NV, 8) segments of 1024 vectors (16 KB);
 // group g of workgroup w is group number g * gridDim.x + w, so that at any moment the grid reads
@@ -373,11 +318,9 @@ __global__ __launch_bounds__(256) void quantize_nvfp4_generic_kernel(
 constexpr int OP_THREADS = 1024;
 constexpr int OP_MAX_WGS = 256;
 constexpr int OP_MAX_NV = 16;
+constexpr int OP_SLOTS = 32;  // concurrent (device, stream) pairs with synchronisation words of their own
 struct OnePassSync {
-  uint32_t arrive[AMAX_SLOTS][OP_MAX_WGS];
-  uint32_t done[AMAX_SLOTS][OP_MAX_WGS];
-  uint32_t epoch[AMAX_SLOTS];
-  uint32_t giveup[AMAX_SLOTS];  // launches left for which the grid wait is skipped (see below)
+  uint32_t arrive[OP_SLOTS][OP_MAX_WGS];
 };
 __device__ __align__(256) OnePassSync g_onepass;
 
@@ -387,7 +330,7 @@ __device__ __align__(256) OnePassSync g_onepass;
 __device__ uint64_t g_onepass_timeline[OP_MAX_WGS][8];
 #define AC4K_TL(i)                                                         \
   do {                                                                     \
-    if (!REPAIR && threadIdx.x == 0) g_onepass_timeline[blockIdx.x][i] = wall_clock64(); \
+    if (threadIdx.x == 0) g_onepass_timeline[blockIdx.x][i] = wall_clock64(); \
   } while (0)
 #else
 #define AC4K_TL(i)
@@ -407,39 +350,43 @@ __device__ __forceinline__ uint4 ld_coherent_u4(const void *p) {
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 
-template <int NV, bool REPAIR>
+// |bf16| maximum over this lane's part of the share of workgroup `u` (the slow path of a workgroup
+// that stopped waiting for `u`): same split as the main kernel, read from memory, rolled loops.
+template <int NV>
+__device__ __forceinline__ uint32_t onepass_share_absmax(const uint4 *__restrict__ in, const OnePassGeom &g, uint32_t u,
+                                                        uint32_t nwg, uint32_t tid) {
+  constexpr int GS = NV < 8 ? NV : 8;
+  constexpr int NG = NV / GS;
+  constexpr uint32_t GC = GS * 128;
+  uint32_t m = 0;
+#pragma unroll 1
+  for (int q = 0; q < NG; ++q) {
+    const uint64_t first = ((uint64_t)q * nwg + u) * GC;
+    if (first >= g.total_chunks) break;
+    const uint32_t left = g.total_chunks - (uint32_t)first;
+    const uint32_t nvalid = left < GC ? left : GC;
+#pragma unroll 2
+    for (int jj = 0; jj < GS; ++jj) {
+      const uint32_t lv = jj * OP_THREADS + tid;
+      if ((lv >> 3) < nvalid) m = umax32(m, absmax_bf16x8(in[first * 8 + lv]));
+    }
+  }
+  return m;
+}
+
+template <int NV>
 __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
     uint32_t *__restrict__ out, uint32_t *__restrict__ sf, const uint4 *__restrict__ in, float *__restrict__ gs_out,
-    OnePassGeom g, int slot, float max_scale, uint64_t timeout_ticks) {
+    OnePassGeom g, int slot, uint32_t tag, float max_scale, uint64_t timeout_ticks) {
   constexpr int GS = NV < 8 ? NV : 8;  // segments per group
   constexpr int NG = NV / GS;          // groups per workgroup
   constexpr uint32_t GC = GS * 128;    // chunks per group
   __shared__ float lut[128];
   __shared__ uint32_t sfs[128 * NV];
   __shared__ uint32_t red[OP_THREADS / 64];
-  __shared__ uint32_t gmax_s;
+  __shared__ uint32_t gmax_s, helping_s;
+  __shared__ uint32_t miss4[OP_MAX_WGS / 4];  // one byte per workgroup: 1 = its maximum has to be recomputed here
   const uint32_t w = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  // the launch tag: the main launch derives it from the slot's counter, the repair launch reads it
-  // back from workgroup 0's word (published whatever happened next) and advances the counter
-  // A workgroup whose wait really ran out marks done[w] with bit 30; the repair launch then arms
-  // giveup[slot], and for that many launches the main kernel does not wait at all (its work is
-  // redone by the repair launch, at the speed of the two-kernel path), so that a GPU shared with
-  // other kernels costs one 200 us stall in 65 launches, not one per launch.
-  uint32_t tag;
-  if (REPAIR) {
-    tag = g_onepass.arrive[slot][0] >> 16;
-    if (w == 0 && tid == 0) g_onepass.epoch[slot] = tag;
-    const uint32_t d = g_onepass.done[slot][w];
-    if (d == (tag | 0x80000000u)) return;
-    if (d == (tag | 0x40000000u) && tid == 0) g_onepass.giveup[slot] = 64;
-  } else {
-    tag = (g_onepass.epoch[slot] + 1) & 0xffffu;
-    const uint32_t gu = g_onepass.giveup[slot];
-    if (gu) {
-      timeout_ticks = 0;
-      if (w == 0 && tid == 0) g_onepass.giveup[slot] = gu - 1;
-    }
-  }
 
   AC4K_TL(0);
   uint32_t cb[NG], nvalid[NG];  // first chunk and number of chunks of each group
@@ -471,89 +418,108 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
       bm[j] = umax32(bm[j], dpp_u32<DPP_QUAD_XOR1>(bm[j]));
       m = umax32(m, bm[j]);
     }
-    if (!REPAIR) {
-      m = group_umax<64>(m);
-      if (lane == 0) red[wave] = m;
-    }
+    m = group_umax<64>(m);
+    if (lane == 0) red[wave] = m;
   }
   __syncthreads();
   AC4K_TL(1);
   if (wave == 0) {
-    if (!REPAIR) {
-      uint32_t m = group_umax<16>(red[lane & 15]);
-      if (lane == 0)
-        __hip_atomic_store(&g_onepass.arrive[slot][w], (tag << 16) | m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    const uint32_t own = group_umax<16>(red[lane & 15]);
+    if (lane == 0)
+      __hip_atomic_store(&g_onepass.arrive[slot][w], (tag << 16) | own, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const uint32_t i0 = lane * 4;
     const uint64_t t_end = wall_clock64() + timeout_ticks;
-    uint32_t mm = 0;
-    bool ok = false;
-    while (REPAIR || wall_clock64() < t_end) {
-      const uint4 a = ld_coherent_u4(&g_onepass.arrive[slot][i0]);
-      const bool ready = (i0 + 0 >= nwg || (a.x >> 16) == tag) && (i0 + 1 >= nwg || (a.y >> 16) == tag) &&
-                         (i0 + 2 >= nwg || (a.z >> 16) == tag) && (i0 + 3 >= nwg || (a.w >> 16) == tag);
-      if (__all(ready)) {
-        mm = umax32(umax32(i0 + 0 < nwg ? a.x & 0xffffu : 0u, i0 + 1 < nwg ? a.y & 0xffffu : 0u),
-                    umax32(i0 + 2 < nwg ? a.z & 0xffffu : 0u, i0 + 3 < nwg ? a.w & 0xffffu : 0u));
-        ok = true;
-        break;
-      }
-      if (REPAIR) break;  // every maximum was published before the first launch ended
+    bool ok, r0, r1, r2, r3;
+    uint4 a;
+    while (true) {  // at least one poll, whatever the timeout
+      a = ld_coherent_u4(&g_onepass.arrive[slot][i0]);
+      r0 = (a.x >> 16) == tag;
+      r1 = (a.y >> 16) == tag;
+      r2 = (a.z >> 16) == tag;
+      r3 = (a.w >> 16) == tag;
+      const bool ready = (i0 + 0 >= nwg || r0) && (i0 + 1 >= nwg || r1) && (i0 + 2 >= nwg || r2) && (i0 + 3 >= nwg || r3);
+      ok = __all(ready);
+      if (ok || wall_clock64() >= t_end) break;
       __builtin_amdgcn_s_sleep(2);
     }
+    // maxima that were published under this launch's tag; the others are marked for recomputation
+    uint32_t mm = own;
+    mm = umax32(mm, (i0 + 0 < nwg && r0) ? a.x & 0xffffu : 0u);
+    mm = umax32(mm, (i0 + 1 < nwg && r1) ? a.y & 0xffffu : 0u);
+    mm = umax32(mm, (i0 + 2 < nwg && r2) ? a.z & 0xffffu : 0u);
+    mm = umax32(mm, (i0 + 3 < nwg && r3) ? a.w & 0xffffu : 0u);
     mm = group_umax<64>(mm);
+    miss4[lane] = ((i0 + 0 < nwg && !r0 && i0 + 0 != w) ? 1u : 0u) | ((i0 + 1 < nwg && !r1 && i0 + 1 != w) ? 0x100u : 0u) |
+                  ((i0 + 2 < nwg && !r2 && i0 + 2 != w) ? 0x10000u : 0u) | ((i0 + 3 < nwg && !r3 && i0 + 3 != w) ? 0x1000000u : 0u);
     if (lane == 0) {
-      gmax_s = ok ? mm : 0xffffffffu;
-      if (!REPAIR && !ok && timeout_ticks) g_onepass.done[slot][w] = tag | 0x40000000u;  // a wait that ran out
+      gmax_s = mm;
+      helping_s = ok ? 0u : 1u;
     }
   }
   __syncthreads();
-  const uint32_t gm = gmax_s;
+  uint32_t gm = gmax_s;
+  if (helping_s) {  // workgroup-uniform: the wait ran out
+    const uint8_t *miss = reinterpret_cast<const uint8_t *>(miss4);
+    uint32_t m = 0;
+#pragma unroll 1
+    for (uint32_t u = 0; u < nwg; ++u)
+      if (miss[u]) m = umax32(m, onepass_share_absmax<NV>(in, g, u, nwg, tid));
+    m = group_umax<64>(m);
+    if (lane == 0) red[wave] = m;  // wave 0 finished reading `red` before the barrier above
+    __syncthreads();
+    gm = umax32(gm, group_umax<16>(red[lane & 15]));
+  }
   AC4K_TL(2);
-  if (gm == 0xffffffffu) return;
   const float gs = bf16_bits_to_f32(gm) / max_scale;
   const float alpha = 1.0f / gs;
-  // With a positive finite alpha no product below is NaN and no block scale reaches 464 (it is at
-  // most 448 * (1 + 3e-7)), so the clamp and the NaN cases of the full code are not needed.
-  if (!REPAIR && !(alpha > 0.0f && alpha < __builtin_inff())) return;
   if (w == 0 && tid == 0) *gs_out = gs;
+  // With a positive finite alpha no product below is NaN and no block scale reaches 464 (it is at
+  // most 448 * (1 + 3e-7)), so the clamp and the NaN cases of the full arithmetic are not needed.
+  const bool fast = alpha > 0.0f && alpha < __builtin_inff();
 
   uint8_t *sfb = reinterpret_cast<uint8_t *>(sfs);
+  auto emit = [&](auto full_range) {
+    constexpr bool FULL = decltype(full_range)::value;
 #pragma unroll
-  for (int q = 0; q < NG; ++q) {
-    uint32_t code[GS];
-    float o[GS];
+    for (int q = 0; q < NG; ++q) {
+      uint32_t code[GS];
+      float o[GS];
 #pragma unroll
-    for (int jj = 0; jj < GS; ++jj) {
-      const int j = q * GS + jj;
-      if (REPAIR) {
-        o[jj] = nvfp4_block_scale(bf16_bits_to_f32(bm[j]), alpha, lut, code[jj]);
-      } else {
-        const float s32 = alpha * (bf16_bits_to_f32(bm[j]) * 0.16666666666666666f);
-        code[jj] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(s32, 0.0f, 0, false);
-        o[jj] = lut[code[jj]];
+      for (int jj = 0; jj < GS; ++jj) {
+        const int j = q * GS + jj;
+        if (FULL) {
+          o[jj] = nvfp4_block_scale(bf16_bits_to_f32(bm[j]), alpha, lut, code[jj]);
+        } else {
+          const float s32 = alpha * (bf16_bits_to_f32(bm[j]) * 0.16666666666666666f);
+          code[jj] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(s32, 0.0f, 0, false);
+          o[jj] = lut[code[jj]];
+        }
+      }
+#pragma unroll
+      for (int jj = 0; jj < GS; ++jj) {
+        const int j = q * GS + jj;
+        const uint32_t lv = jj * OP_THREADS + tid;
+        uint32_t packed;
+        if (FULL) {
+          packed = nvfp4_pack8(v[j], o[jj]);
+        } else {
+          const float oo = alpha * o[jj];
+          const float f[8] = {bf16_lo(v[j].x) * oo, bf16_hi(v[j].x) * oo, bf16_lo(v[j].y) * oo, bf16_hi(v[j].y) * oo,
+                              bf16_lo(v[j].z) * oo, bf16_hi(v[j].z) * oo, bf16_lo(v[j].w) * oo, bf16_hi(v[j].w) * oo};
+          packed = f32x8_to_e2m1x8(f);
+        }
+        if ((lv >> 3) < nvalid[q]) {
+          st_stream_u1(out + (uint64_t)cb[q] * 8 + lv, packed);
+          // scale byte (lv % 8) / 2 of chunk lv / 8; both lanes of a 16-block hold the same code
+          if ((lane & 1) == 0) sfb[q * GC * 4 + (lv >> 1)] = (uint8_t)code[jj];
+        }
       }
     }
-#pragma unroll
-    for (int jj = 0; jj < GS; ++jj) {
-      const int j = q * GS + jj;
-      const uint32_t lv = jj * OP_THREADS + tid;
-      uint32_t packed;
-      if (REPAIR) {
-        packed = nvfp4_pack8(v[j], o[jj]);
-      } else {
-        const float oo = alpha * o[jj];
-        const float f[8] = {bf16_lo(v[j].x) * oo, bf16_hi(v[j].x) * oo, bf16_lo(v[j].y) * oo, bf16_hi(v[j].y) * oo,
-                            bf16_lo(v[j].z) * oo, bf16_hi(v[j].z) * oo, bf16_lo(v[j].w) * oo, bf16_hi(v[j].w) * oo};
-        packed = f32x8_to_e2m1x8(f);
-      }
-      if ((lv >> 3) < nvalid[q]) {
-        st_stream_u1(out + (uint64_t)cb[q] * 8 + lv, packed);
-        // scale byte (lv % 8) / 2 of chunk lv / 8; both lanes of a 16-block hold the same code
-        if ((lane & 1) == 0) sfb[q * GC * 4 + (lv >> 1)] = (uint8_t)code[jj];
-      }
-    }
-  }
+  };
+  if (fast)
+    emit(std::false_type{});
+  else
+    emit(std::true_type{});
   __syncthreads();
   AC4K_TL(3);
   // scales: LDS holds one dword per chunk in (row, chunk column) order; memory wants, per chunk
@@ -578,7 +544,6 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
     for (uint32_t i = w * per + tid; i < hi; i += OP_THREADS) sf[(uint64_t)(i / pad) * g.Rp + g.R + i % pad] = 0u;
   }
   AC4K_TL(4);
-  if (!REPAIR && tid == 0) g_onepass.done[slot][w] = tag | 0x80000000u;
 }
 
 // ---------------------------------------------------------------------------
@@ -834,11 +799,11 @@ __device__ __forceinline__ int fp8_swizzle_src(int p) { return ((p & 3) >> 1) * 
 
 template <bool SWIZZLE>
 __global__ __launch_bounds__(256) void quantize_nvfp4_crossmajor_kernel(
-    uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in, GlobalScaleSrc gsrc,
+    uint8_t *__restrict__ out, uint8_t *__restrict__ sf, const uint16_t *__restrict__ in, const float *__restrict__ gs_ptr,
     QuantGeom g) {
   __shared__ float lut[128];
   load_rcp_table(lut);
-  const float alpha = load_alpha(gsrc, blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0);
+  const float alpha = 1.0f / *gs_ptr;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int kb = lane & 3, rg = lane >> 2;
   const CrossMajorIdx gi = crossmajor_idx(g);
@@ -1004,8 +969,29 @@ static int check_geom(const void *out, const void *sf, const void *in, const voi
   AC4K_REQUIRE(out && sf && in && scalar, "null pointer argument");
   AC4K_REQUIRE(d0 >= 1 && d1 >= 1 && R >= 1 && K >= 1, "sizes must be positive (d0=%lld d1=%lld R=%lld K=%lld)",
                (long long)d0, (long long)d1, (long long)R, (long long)K);
-  AC4K_REQUIRE(s0 >= 0 && s1 >= 0 && sR >= 1 && sK >= 1, "strides must be positive");
+  AC4K_REQUIRE(s0 >= 0 && s1 >= 0 && sR >= 1 && sK >= 1 && (d0 == 1 || s0 >= 1) && (d1 == 1 || s1 >= 1),
+               "strides must be positive");
   return 0;
+}
+
+// Do the four dims, in some order, tile d0*d1*R*K contiguous elements exactly?  (Dims of size 1 may
+// carry any stride.)
+static bool dense_permutation(int64_t d0, int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
+                              int64_t sK) {
+  int64_t size[4] = {d0, d1, R, K}, stride[4] = {s0, s1, sR, sK};
+  for (int i = 1; i < 4; ++i)  // insertion sort by stride
+    for (int j = i; j > 0 && stride[j] < stride[j - 1]; --j) {
+      const int64_t ts = stride[j], tz = size[j];
+      stride[j] = stride[j - 1]; size[j] = size[j - 1];
+      stride[j - 1] = ts; size[j - 1] = tz;
+    }
+  int64_t expect = 1;
+  for (int i = 0; i < 4; ++i) {
+    if (size[i] == 1) continue;
+    if (stride[i] != expect) return false;
+    expect *= size[i];
+  }
+  return true;
 }
 
 static bool rowmajor_ok(const void *in, int64_t K, int64_t s0, int64_t s1, int64_t sR, int64_t sK) {
@@ -1020,7 +1006,7 @@ static bool crossmajor_ok(const void *in, int64_t R, int64_t s0, int64_t s1, int
 }
 
 template <int CPR>
-static void launch_nvfp4_rowmajor(uint8_t *out, uint8_t *sf, const uint16_t *in, const GlobalScaleSrc &gs,
+static void launch_nvfp4_rowmajor(uint8_t *out, uint8_t *sf, const uint16_t *in, const float *gs,
                                   const QuantGeom &g, int64_t lead, hipStream_t st, bool swizzle) {
   constexpr int ITER = 4;
   constexpr int ROWS = 4 * (8 / CPR) * ITER;
@@ -1037,54 +1023,61 @@ using namespace ac4k;
 
 namespace ac4k {
 
-// (device, stream) -> scratch slot.  Slots are handed out on first use and never recycled;
-// when they run out the caller gets -1 and takes the path without scratch.  A call captured into
-// a graph keeps the slot of the stream it was captured on.
-// Calls that enqueue several launches sharing a scratch slot (maxima, then their consumer) hold this
-// lock while they enqueue, so that two host threads feeding the same stream cannot interleave
-// their launches (the stream would then run a consumer against the other call's maxima).
-static std::mutex g_enqueue_mutex;
+// (device, stream) -> slot of synchronisation words for the single-launch quantizer, plus the launch
+// tag.  A stream keeps its slot while it is among the OP_SLOTS most recently used streams of its
+// device; a newcomer takes a free slot or evicts the least recently used one.  Tags count on per
+// slot, so two launches that meet on one slot (an evicted stream whose kernel is still running)
+// carry different tags: each of them then misses words of its own tag, stops waiting after the
+// timeout and finishes through the kernel's slow path - slower, never wrong.
+constexpr int OP_MAX_DEVICES = 16;
+struct OnePassSlot {
+  hipStream_t st;
+  uint64_t last_use;  // 0 = never used
+  uint32_t tag;
+};
+static std::mutex g_slot_mutex;
+static OnePassSlot g_slots[OP_MAX_DEVICES][OP_SLOTS];
+static uint64_t g_slot_clock = 0;
 
-static int amax_slot(hipStream_t st) {
-  static std::mutex mu;
-  static struct { int dev; hipStream_t st; } table[AMAX_SLOTS];
-  static int used = 0;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return -1;
-  std::lock_guard<std::mutex> lock(mu);
-  int per_dev = 0;
-  for (int i = 0; i < used; ++i) {
-    if (table[i].dev == dev && table[i].st == st) return per_dev;
-    if (table[i].dev == dev) ++per_dev;
+static bool onepass_slot(hipStream_t st, int *slot, uint32_t *tag) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= OP_MAX_DEVICES) return false;
+  std::lock_guard<std::mutex> lock(g_slot_mutex);
+  OnePassSlot *t = g_slots[dev];
+  int pick = -1, oldest = 0;
+  for (int i = 0; i < OP_SLOTS; ++i) {
+    if (t[i].last_use && t[i].st == st) {
+      pick = i;
+      break;
+    }
+    if (t[i].last_use < t[oldest].last_use) oldest = i;  // never-used slots (0) come first
   }
-  if (used >= AMAX_SLOTS) return -1;
-  table[used].dev = dev;
-  table[used].st = st;
-  ++used;
-  return per_dev;  // index among this device's streams: each device has its own copy of the scratch
+  if (pick < 0) {
+    pick = oldest;
+    t[pick].st = st;
+  }
+  t[pick].last_use = ++g_slot_clock;
+  t[pick].tag = t[pick].tag % 0xffffu + 1;  // 1 .. 65535
+  *slot = pick;
+  *tag = t[pick].tag;
+  return true;
 }
 
-// Launches pass 1 (block maxima into the slot's scratch).  Returns the number of deposits, or
-// 0 when no slot is free / the input is empty (the caller then takes the atomic path).
-static int launch_amax_partials(const void *x, int64_t n, hipStream_t st, int *slot_out) {
-  if (n == 0) return 0;
-  const int slot = amax_slot(st);
-  if (slot < 0) return 0;
-  const uintptr_t addr = reinterpret_cast<uintptr_t>(x);
-  int64_t head = ((16 - (addr & 15)) & 15) / 2;
-  if (head > n) head = n;
-  const int64_t nvec = (n - head) / 8;
-  int64_t blocks = ceil_div(nvec, (int64_t)AMAX_THREADS * AMAX_UNROLL);
-  if (blocks < 1) blocks = 1;
-  if (blocks > AMAX_MAX_BLOCKS) blocks = AMAX_MAX_BLOCKS;
-  hipLaunchKernelGGL(amax_partials_bf16_kernel, dim3((unsigned)blocks), dim3(AMAX_THREADS), 0, st,
-                     static_cast<const uint16_t *>(x), n, head, nvec, slot);
-  *slot_out = slot;
-  return (int)blocks;
+// True while `st` records into a graph (or when that cannot be told).  A captured launch would replay
+// with the tag and the slot of the capture, possibly next to other replays or eager launches on the
+// same slot, so captured calls take the path whose whole state lives in the caller's buffers.
+static bool stream_is_capturing(hipStream_t st) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;
+  }
+  return status != hipStreamCaptureStatusNone;
 }
 
-// Fallback without scratch: *gs zeroed by a fill kernel, then one atomic max per block.
-static void launch_global_scale_atomic(float *gs, const void *x, int64_t n, float max_scale, hipStream_t st) {
+// *gs = max|x| / max_scale with no scratch of the library's own: *gs zeroed by a fill kernel, then
+// block maxima folded in with (mostly skipped) atomics.
+static void launch_global_scale(float *gs, const void *x, int64_t n, float max_scale, hipStream_t st) {
   hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(1), 0, st, reinterpret_cast<uint32_t *>(gs));
   if (n == 0) return;
   const uintptr_t addr = reinterpret_cast<uintptr_t>(x);
@@ -1093,23 +1086,18 @@ static void launch_global_scale_atomic(float *gs, const void *x, int64_t n, floa
   const int64_t nvec = (n - head) / 8;
   int64_t blocks = ceil_div(nvec, (int64_t)AMAX_THREADS * AMAX_UNROLL);
   if (blocks < 1) blocks = 1;
-  if (blocks > 256) blocks = 256;  // every block ends with an atomic on the same address
+  if (blocks > AMAX_MAX_BLOCKS) blocks = AMAX_MAX_BLOCKS;
   hipLaunchKernelGGL(amax_scale_bf16_atomic_kernel, dim3((unsigned)blocks), dim3(AMAX_THREADS), 0, st,
                      reinterpret_cast<uint32_t *>(gs), static_cast<const uint16_t *>(x), n, head, nvec, max_scale);
 }
 
-static void launch_global_scale(float *gs, const void *x, int64_t n, float max_scale, hipStream_t st) {
-  int slot = -1;
-  const int npart = launch_amax_partials(x, n, st, &slot);
-  if (npart > 0)
-    hipLaunchKernelGGL(amax_finalize_kernel, dim3(1), dim3(AMAX_THREADS), 0, st, gs, slot, npart, max_scale);
-  else
-    launch_global_scale_atomic(gs, x, n, max_scale, st);
-}
-
-// Bound of the single-launch quantizer's grid wait in 100 MHz ticks (200 us); 0 sends every
-// workgroup to the repair launch, a negative value switches the single-launch path off.
+// Bound of the single-launch quantizer's grid wait in 100 MHz ticks (200 us); 0 = one look at the
+// other workgroups' words, then the slow path; a negative value switches the single-launch path off.
 static std::atomic<int64_t> g_sync_timeout_ticks{20000};
+
+// which path the last ac4k_quantize_nvfp4_bf16 call of this host thread took (introspection for tests)
+enum QuantPath { QPATH_NONE = 0, QPATH_SMALL = 1, QPATH_ONEPASS = 2, QPATH_TWO_KERNEL = 3 };
+static thread_local int g_last_quantize_path = QPATH_NONE;
 
 static int device_cu_count() {
   static std::atomic<int> cached[64];
@@ -1125,15 +1113,13 @@ static int device_cu_count() {
 
 template <int NV>
 static void launch_onepass(uint32_t *out, uint32_t *sf, const uint4 *in, float *gs, const OnePassGeom &g, int nwg,
-                           int slot, float max_scale, uint64_t ticks, hipStream_t st) {
-  hipLaunchKernelGGL((quantize_nvfp4_onepass_kernel<NV, false>), dim3(nwg), dim3(OP_THREADS), 0, st, out, sf, in, gs,
-                     g, slot, max_scale, ticks);
-  hipLaunchKernelGGL((quantize_nvfp4_onepass_kernel<NV, true>), dim3(nwg), dim3(OP_THREADS), 0, st, out, sf, in, gs,
-                     g, slot, max_scale, ticks);
+                           int slot, uint32_t tag, float max_scale, uint64_t ticks, hipStream_t st) {
+  hipLaunchKernelGGL((quantize_nvfp4_onepass_kernel<NV>), dim3(nwg), dim3(OP_THREADS), 0, st, out, sf, in, gs, g, slot,
+                     tag, max_scale, ticks);
 }
 
 // Up to 16 segments (256 KB) every workgroup can afford to read the whole tensor for its maximum:
-// one launch of a few microseconds, against two launches and a grid wait.
+// one launch of a few microseconds, no grid wait.
 constexpr int SMALL_MAX_SEGS = 16;
 
 static void launch_small(uint32_t *out, uint32_t *sf, const uint4 *in, float *gs, const OnePassGeom &g,
@@ -1147,46 +1133,47 @@ static void launch_small(uint32_t *out, uint32_t *sf, const uint4 *in, float *gs
   else hipLaunchKernelGGL(quantize_nvfp4_small_kernel<16>, grid, block, 0, st, out, sf, in, gs, g, max_scale);
 }
 
-// Global scale + nvfp4 quantize of a dense [lead, R, K] tensor in one pass over the input, when
-// the shape allows it.  Returns false (nothing launched) when the caller has to take the
-// two-kernel path.
-static bool try_quantize_nvfp4_onepass(void *out, void *sf, float *gs, const void *in, int64_t d0, int64_t d1,
-                                       int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR, int64_t sK,
-                                       int swizzle, float max_scale, hipStream_t st) {
+// Global scale + nvfp4 quantize of a dense [lead, R, K] tensor in one launch, when the shape allows
+// it.  Returns QPATH_NONE (nothing launched) when the caller has to take the two-kernel path.
+static int try_quantize_nvfp4_onepass(void *out, void *sf, float *gs, const void *in, int64_t d0, int64_t d1,
+                                      int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR, int64_t sK,
+                                      int swizzle, float max_scale, hipStream_t st) {
   const int64_t ticks = g_sync_timeout_ticks.load();
-  if (ticks < 0 || sK != 1 || K % 64 != 0 || sR != K) return false;
-  if ((d1 > 1 && s1 != R * K) || (d0 > 1 && s0 != d1 * R * K)) return false;
-  if (reinterpret_cast<uintptr_t>(in) & 15) return false;
+  if (ticks < 0 || sK != 1 || K % 64 != 0 || sR != K) return QPATH_NONE;
+  if ((d1 > 1 && s1 != R * K) || (d0 > 1 && s0 != d1 * R * K)) return QPATH_NONE;
+  if (reinterpret_cast<uintptr_t>(in) & 15) return QPATH_NONE;
   const int64_t lead = d0 * d1, chunks = lead * R * (K / 64);
   int nwg = device_cu_count();
   if (nwg > OP_MAX_WGS) nwg = OP_MAX_WGS;
-  if (nwg < 8 || chunks > (int64_t)nwg * 128 * OP_MAX_NV) return false;
+  if (nwg < 8 || chunks > (int64_t)nwg * 128 * OP_MAX_NV) return QPATH_NONE;
   const OnePassGeom g{(uint32_t)chunks, (uint32_t)(K / 64), (uint32_t)R, (uint32_t)align_up(R, 16), (uint32_t)lead,
                       swizzle ? 1u : 0u};
-  if (chunks <= 128 * SMALL_MAX_SEGS) {  // small: one launch, no grid wait
+  if (chunks <= 128 * SMALL_MAX_SEGS) {  // small: one launch, no grid wait, no state
     launch_small(static_cast<uint32_t *>(out), static_cast<uint32_t *>(sf), static_cast<const uint4 *>(in), gs, g,
                  max_scale, st);
-    return true;
+    return QPATH_SMALL;
   }
-  const int slot = amax_slot(st);
-  if (slot < 0) return false;
+  if (stream_is_capturing(st)) return QPATH_NONE;
+  int slot = -1;
+  uint32_t tag = 0;
+  if (!onepass_slot(st, &slot, &tag)) return QPATH_NONE;
   const int64_t per_wg = ceil_div(chunks, (int64_t)nwg * 128);  // 16 KB segments per workgroup
   uint32_t *o = static_cast<uint32_t *>(out), *s = static_cast<uint32_t *>(sf);
   const uint4 *x = static_cast<const uint4 *>(in);
   if (per_wg <= 1)
-    launch_onepass<1>(o, s, x, gs, g, nwg, slot, max_scale, (uint64_t)ticks, st);
+    launch_onepass<1>(o, s, x, gs, g, nwg, slot, tag, max_scale, (uint64_t)ticks, st);
   else if (per_wg <= 2)
-    launch_onepass<2>(o, s, x, gs, g, nwg, slot, max_scale, (uint64_t)ticks, st);
+    launch_onepass<2>(o, s, x, gs, g, nwg, slot, tag, max_scale, (uint64_t)ticks, st);
   else if (per_wg <= 4)
-    launch_onepass<4>(o, s, x, gs, g, nwg, slot, max_scale, (uint64_t)ticks, st);
+    launch_onepass<4>(o, s, x, gs, g, nwg, slot, tag, max_scale, (uint64_t)ticks, st);
   else if (per_wg <= 8)
-    launch_onepass<8>(o, s, x, gs, g, nwg, slot, max_scale, (uint64_t)ticks, st);
+    launch_onepass<8>(o, s, x, gs, g, nwg, slot, tag, max_scale, (uint64_t)ticks, st);
   else
-    launch_onepass<16>(o, s, x, gs, g, nwg, slot, max_scale, (uint64_t)ticks, st);
-  return true;
+    launch_onepass<16>(o, s, x, gs, g, nwg, slot, tag, max_scale, (uint64_t)ticks, st);
+  return QPATH_ONEPASS;
 }
 
-static int launch_quantize_nvfp4(void *out, void *sf, const void *in, const GlobalScaleSrc &gsrc, int64_t d0,
+static int launch_quantize_nvfp4(void *out, void *sf, const void *in, const float *gsrc, int64_t d0,
                                  int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR, int64_t sK,
                                  int swizzle, hipStream_t st) {
   QuantGeom g{d1, R, K, align_up(K, 64), align_up(R, 16), s0, s1, sR, sK, 0};
@@ -1232,7 +1219,6 @@ extern "C" __attribute__((visibility("default"))) int ac4k_global_scale_bf16(flo
   AC4K_REQUIRE(gs && (x || n == 0), "null pointer argument");
   AC4K_REQUIRE(n >= 0, "n must be non-negative");
   AC4K_REQUIRE((reinterpret_cast<uintptr_t>(x) & 1) == 0, "x must be 2-byte aligned");
-  std::lock_guard<std::mutex> lock(g_enqueue_mutex);
   launch_global_scale(gs, x, n, max_scale, (hipStream_t)stream);
   return check_launch("ac4k_global_scale_bf16");
 }
@@ -1241,8 +1227,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_quantize_nvfp4(void *
                                    int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
                                    int64_t sK, int swizzle, ac4k_stream_t stream) {
   if (int rc = check_geom(out, sf, in, global_scale, d0, d1, R, K, s0, s1, sR, sK)) return rc;
-  const GlobalScaleSrc gsrc{const_cast<float *>(global_scale), -1, 0, 0.0f};
-  if (int rc = launch_quantize_nvfp4(out, sf, in, gsrc, d0, d1, R, K, s0, s1, sR, sK, swizzle, (hipStream_t)stream))
+  if (int rc = launch_quantize_nvfp4(out, sf, in, global_scale, d0, d1, R, K, s0, s1, sR, sK, swizzle, (hipStream_t)stream))
     return rc;
   return check_launch("ac4k_quantize_nvfp4");
 }
@@ -1251,22 +1236,23 @@ extern "C" __attribute__((visibility("default"))) int ac4k_quantize_nvfp4_bf16(v
                                         int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
                                         int64_t sK, int swizzle, float max_scale, ac4k_stream_t stream) {
   if (int rc = check_geom(out, sf, in, global_scale, d0, d1, R, K, s0, s1, sR, sK)) return rc;
+  // the global scale is the maximum over the d0*d1*R*K elements that start at `in`: the four dims
+  // must tile that range exactly (any order), as the contiguous tensor of the reference op does
+  AC4K_REQUIRE(dense_permutation(d0, d1, R, K, s0, s1, sR, sK),
+               "in must be a dense (permuted) tensor: its strides do not tile d0*d1*R*K contiguous elements");
   hipStream_t st = (hipStream_t)stream;
-  std::lock_guard<std::mutex> lock(g_enqueue_mutex);
-  if (try_quantize_nvfp4_onepass(out, sf, global_scale, in, d0, d1, R, K, s0, s1, sR, sK, swizzle, max_scale, st))
-    return check_launch("ac4k_quantize_nvfp4_bf16");
-  // pass 1 leaves one maximum per block in the stream's scratch slot; the quantize kernel
-  // reduces them itself and publishes the scale, so the whole op is two launches
-  int slot = -1;
-  const int npart = launch_amax_partials(in, d0 * d1 * R * K, st, &slot);
-  GlobalScaleSrc gsrc{global_scale, slot, npart, max_scale};
-  if (npart == 0) {
-    launch_global_scale_atomic(global_scale, in, d0 * d1 * R * K, max_scale, st);
-    gsrc.slot = -1;
-  }
-  if (int rc = launch_quantize_nvfp4(out, sf, in, gsrc, d0, d1, R, K, s0, s1, sR, sK, swizzle, st)) return rc;
+  g_last_quantize_path = try_quantize_nvfp4_onepass(out, sf, global_scale, in, d0, d1, R, K, s0, s1, sR, sK, swizzle,
+                                                    max_scale, st);
+  if (g_last_quantize_path != QPATH_NONE) return check_launch("ac4k_quantize_nvfp4_bf16");
+  // two passes over the input, all state in the caller's buffers: fill, maxima into *global_scale,
+  // then the quantize kernel that reads it
+  g_last_quantize_path = QPATH_TWO_KERNEL;
+  launch_global_scale(global_scale, in, d0 * d1 * R * K, max_scale, st);
+  if (int rc = launch_quantize_nvfp4(out, sf, in, global_scale, d0, d1, R, K, s0, s1, sR, sK, swizzle, st)) return rc;
   return check_launch("ac4k_quantize_nvfp4_bf16");
 }
+
+extern "C" __attribute__((visibility("default"))) int ac4k_debug_last_quantize_path(void) { return ac4k::g_last_quantize_path; }
 
 namespace ac4k {
 

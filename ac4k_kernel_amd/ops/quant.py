@@ -26,13 +26,21 @@ _SCALE_MAX_CACHE = {}
 
 
 def _scale_max_tensor(value, dtype, device):
-    """0-dim device scalar for scale_max; the reference builds one with torch.full on every call
-    (quant.py:130-135,177-182), here it is kept per (value, dtype, device)."""
+    """0-dim device scalar for scale_max.  The reference builds one with torch.full on every call
+    (quant.py:130-135,177-182); here it is kept per (value, dtype, device) once it exists with its
+    value in place.  While the current stream records into a graph nothing is cached: a tensor made
+    there lives in the graph's memory pool and is only filled when the graph replays."""
     key = (value, dtype, device)
     t = _SCALE_MAX_CACHE.get(key)
-    if t is None:
-        t = torch.full([], value, dtype=dtype, device=device)
-        _SCALE_MAX_CACHE[key] = t
+    if t is not None:
+        return t
+    t = torch.full([], value, dtype=dtype, device=device)
+    if device.type == "cuda" and torch.cuda.is_current_stream_capturing():
+        return t
+    # the fill ran on the current stream; later calls may come from other streams, so the cached
+    # tensor is handed out only after the fill has completed
+    torch.cuda.current_stream(device).synchronize() if device.type == "cuda" else None
+    _SCALE_MAX_CACHE[key] = t
     return t
 
 

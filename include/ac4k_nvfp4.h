@@ -64,18 +64,32 @@ int ac4k_quantize_nvfp4(void *out, void *sf, const void *in, const float *global
 
 /* The nvfp4 branch of Ac4kQuantizeOp.forward in one call
  * (python/ac4k_kernel/ops/quant.py:187-242): *global_scale = max|in| / max_scale over the whole
- * (contiguous) input, then ac4k_quantize_nvfp4 with it.  One launch for dense tensors of up to
- * 256 KB, else two; nothing to initialise, no host synchronisation. */
+ * input, then ac4k_quantize_nvfp4 with it.  `in` must be dense: the four dims, in any order, tile
+ * d0*d1*R*K contiguous elements (the reference op makes its input contiguous, :201); other strides
+ * are rejected.  Nothing to initialise, no host synchronisation.
+ *   - dense row-major tensors (sK == 1, K % 64 == 0, 16-byte aligned) of up to 256 KB: one launch;
+ *   - the same up to 64 MiB: one launch of a kernel whose workgroups exchange their maxima through
+ *     synchronisation words inside the library (32 sets per GPU, handed to the most recently used
+ *     streams), see ac4k_set_quantize_sync_timeout_us;
+ *   - everything else, and every call made while `stream` is capturing into a graph: three launches
+ *     (fill, maxima, quantize) whose whole state is *global_scale - safe to replay on any stream,
+ *     next to anything. */
 int ac4k_quantize_nvfp4_bf16(void *out, void *sf, float *global_scale, const void *in, int64_t d0,
                              int64_t d1, int64_t R, int64_t K, int64_t s0, int64_t s1, int64_t sR,
                              int64_t sK, int swizzle, float max_scale, ac4k_stream_t stream);
 
-/* Tuning knob of ac4k_quantize_nvfp4_bf16 (no counterpart in the reference).  Dense tensors between
- * 256 KB and 64 MiB are quantized in one pass over the input by a kernel whose workgroups wait for each other;
- * the wait is bounded by this many microseconds (default 200), after which the workgroups that gave
- * up are redone by a second launch that is always enqueued behind the first.  0 sends every workgroup
- * down that second path (used by the tests); a negative value selects the two-kernel quantizer. */
+/* Tuning knob of ac4k_quantize_nvfp4_bf16 (no counterpart in the reference): the workgroups of the
+ * single-launch kernel wait for each other's maxima for at most this many microseconds (default
+ * 200).  A workgroup whose wait runs out - its peers were not all resident because other kernels
+ * hold the GPU - recomputes the missing maxima from memory itself and finishes: slower, same bits.
+ * 0 = look once, then recompute (used by the tests); a negative value switches the single-launch
+ * kernel off (three launches, as under graph capture). */
 void ac4k_set_quantize_sync_timeout_us(int64_t us);
+
+/* Introspection for tests (no counterpart in the reference): which path the last
+ * ac4k_quantize_nvfp4_bf16 call of the calling host thread took: 0 none yet, 1 small one-launch
+ * kernel, 2 single-launch kernel with the grid wait, 3 fill + maxima + quantize. */
+int ac4k_debug_last_quantize_path(void);
 
 /* Replaces ac4k::quantize_fp8 (lib/cuda/sm120/quantize_fp8.cu:192-290).
  * out: e4m3 [d0,d1,R,align_up(K,16)];  sf: fp32 [d0,d1,align_up(R,16)] = amax/scale_max.
@@ -131,6 +145,13 @@ int ac4k_linear_nvfp4_skinny_static(void *D, int d_dtype, const void *A, const v
                                     const float *A_gs, const void *B, const void *B_sf,
                                     const float *B_gs, const void *bias, int bias_dtype, int64_t M,
                                     int64_t N, int64_t K, ac4k_stream_t stream);
+
+/* Tuning aid of the linear entry points (no counterpart in the reference; results stay within the
+ * same tolerance): forces the tile of the packed-operand kernel to (64 mi) x (64 nj) with `splits` K
+ * ranges (mi in {2,4}, nj in {1,2,4}, not (4,1); splits > 1 only takes effect in the workspace entry
+ * points) and the K slice of the decode-sized kernel (256, 512 or 1024).  Zeros give the choice back
+ * to the library's cost model.  Process-wide; returns non-zero on values outside these sets. */
+int ac4k_set_linear_tuning(int mi, int nj, int splits, int skinny_ks);
 
 /* Fused decode-sized linear: quantize(X,0,1) followed by linear(...) in one call.  No single
  * reference function: it equals the composition the reference's tests make

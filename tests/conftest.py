@@ -30,3 +30,17 @@ def make_input(shape, seed=0, outliers=False, dist="normal", std=1.0):
         mask = torch.rand(shape, generator=g) < 0.001
         x = torch.where(mask, x * 20.0, x)
     return x.to(torch.bfloat16)
+
+
+@pytest.fixture
+def linear_tuning():
+    """Forces a tile plan / K slice of the linear kernels for one test (ac4k_set_linear_tuning) and gives
+    the choice back to the library afterwards."""
+    from ac4k_kernel_amd import _lib
+    lib = _lib.load()
+
+    def force(mi=0, nj=0, splits=0, skinny_ks=0):
+        _lib.check(lib.ac4k_set_linear_tuning(mi, nj, splits, skinny_ks))
+
+    yield force
+    lib.ac4k_set_linear_tuning(0, 0, 0, 0)

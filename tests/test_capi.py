@@ -18,7 +18,7 @@ def declared_functions():
 def test_header_and_loader_agree():
     from ac4k_kernel_amd import _lib
     names = declared_functions()
-    assert len(names) >= 11
+    assert len(names) >= 18
     assert sorted(_lib.SIGNATURES) == names
     lib = _lib.load()
     for n in names:
@@ -56,6 +56,17 @@ def test_argument_rejection_without_gpu():
     assert rc != 0 and b"multiple of 16" in lib.ac4k_last_error()
     rc = lib.ac4k_linear_nvfp4(one, 7, one, one, one, one, one, one, None, 0, 4, 4, 64, None)
     assert rc != 0 and b"bfloat16, half or float" in lib.ac4k_last_error()
+    # a sliced view (rows of 64 taken out of rows of 128) is not dense: the global scale would be taken
+    # over the wrong elements, so the one-call quantizer refuses it; so it does a zero stride on a real dim
+    rc = lib.ac4k_quantize_nvfp4_bf16(one, one, one, one, 1, 1, 4, 64, 0, 0, 128, 1, 0, 2688.0, None)
+    assert rc != 0 and b"dense" in lib.ac4k_last_error()
+    rc = lib.ac4k_quantize_nvfp4_bf16(one, one, one, one, 1, 3, 4, 64, 0, 0, 64, 1, 0, 2688.0, None)
+    assert rc != 0 and b"strides must be positive" in lib.ac4k_last_error()
+    # tuning values outside the instantiated kernels are refused, zeros are accepted
+    assert lib.ac4k_set_linear_tuning(4, 1, 1, 0) != 0 and b"tile plan" in lib.ac4k_last_error()
+    assert lib.ac4k_set_linear_tuning(0, 0, 0, 2048) != 0 and b"skinny_ks" in lib.ac4k_last_error()
+    assert lib.ac4k_set_linear_tuning(0, 0, 0, 0) == 0
+    assert lib.ac4k_debug_last_quantize_path() in (0, 1, 2, 3)
     rc = lib.ac4k_linear_nvfp4_fused_bf16(one, 0, one, one, one, one, one, one, one, None, 0, 64, 4, 64, one, 0, None)
     assert rc != 0 and b"1 <= M <= 32" in lib.ac4k_last_error()
     with pytest.raises(RuntimeError):

@@ -104,9 +104,9 @@ LINEAR_CASES = [
 
 @pytest.mark.parametrize("odt", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("m,n,k,plan", LINEAR_CASES)
-def test_linear_stays_inside_its_output(m, n, k, plan, odt, monkeypatch):
+def test_linear_stays_inside_its_output(m, n, k, plan, odt, linear_tuning):
     if plan:
-        monkeypatch.setenv("AC4K_TILE_PLAN", plan)
+        linear_tuning(*[int(v) for v in plan.split(",")])
     aq = ops().quantize(make_input((m, k), seed=m).cuda(), 0, 1)
     bq = ops().quantize(make_input((n, k), seed=n, std=0.02).cuda(), 0, 1)
     bias = make_input((1, n), seed=7).float().cuda()

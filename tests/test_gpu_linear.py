@@ -241,13 +241,13 @@ def test_mid_m_shapes(m, n, k):
 
 
 # every tile shape of the packed-LDS kernel (64*mi rows x 64*nj columns, its own LDS stage depth),
-# alone and split along K, forced through the library's tuning variable; ragged M and N included
+# alone and split along K, forced through ac4k_set_linear_tuning; ragged M and N included
 TILE_PLANS = [(2, 1, 1), (2, 2, 1), (2, 4, 1), (4, 2, 1), (4, 4, 1), (2, 1, 3), (2, 2, 2), (2, 4, 5), (4, 2, 2), (4, 4, 4)]
 
 
 @pytest.mark.parametrize("mi,nj,splits", TILE_PLANS)
-def test_tile_plans(mi, nj, splits, monkeypatch):
-    monkeypatch.setenv("AC4K_TILE_PLAN", f"{mi},{nj},{splits}")
+def test_tile_plans(mi, nj, splits, linear_tuning):
+    linear_tuning(mi, nj, splits)
     for (m, n, k) in [(64 * mi, 128 * nj, 1280), (64 * mi + 37, 64 * nj * 3 - 10, 1536), (33, 136, 2048)]:
         run_case(m, n, k, seed=mi * 100 + nj * 10 + splits, wstd=0.02)
         run_case(m, n, k, bias_dtype=torch.bfloat16, o_dtype=torch.float32, seed=m + n, wstd=0.02)

@@ -20,7 +20,8 @@ def ops():
 def check_nvfp4(x, cross, red, swz=False, oracle=T, **kw):
     out, sf, gs = ops().quantize(x.cuda(), cross, red, swizzle=swz, **kw)
     eo, es, eg = oracle.quantize_nvfp4(x, cross, red, swz, **({"max_scale": kw["max_scale"]} if "max_scale" in kw else {}))
-    assert gs.dtype == torch.float32 and gs.dim() == 0 and gs.item() == eg.item(), (gs.item(), eg.item())
+    same_gs = gs.item() == eg.item() or (gs.item() != gs.item() and eg.item() != eg.item())  # NaN equals NaN here
+    assert gs.dtype == torch.float32 and gs.dim() == 0 and same_gs, (gs.item(), eg.item())
     assert out.dtype == torch.uint8 and sf.dtype == torch.float8_e4m3fn
     assert list(out.shape) == list(eo.shape) and list(sf.shape) == list(es.shape)
     sfb = sf.cpu().view(torch.uint8)
@@ -102,24 +103,40 @@ ONEPASS_SHAPES = [((64, 128), 0, 1), ((8192, 4096), 0, 1), ((4096, 4096), 0, 1),
                   ((5000, 64), 0, 1), ((1, 8192), 0, 1), ((32, 8192), 0, 1), ((6100, 5120), 0, 1)]
 
 
+# which path ac4k_quantize_nvfp4_bf16 took: ac4k_debug_last_quantize_path()
+PATH_SMALL, PATH_ONEPASS, PATH_TWO_KERNEL = 1, 2, 3
+
+
 @pytest.mark.parametrize("timeout_us", [200, 0, -1])
 def test_nvfp4_single_launch_paths(timeout_us):
+    """200: the grid wait as shipped; 0: every workgroup looks once at the others' words and recomputes
+    the maxima that are missing from memory (the path of a wait that ran out); -1: single-launch
+    kernel off (fill + maxima + quantize)."""
     from ac4k_kernel_amd import _lib
     L = _lib.load()
     L.ac4k_set_quantize_sync_timeout_us(timeout_us)
     try:
         for i, (shape, c, r) in enumerate(ONEPASS_SHAPES):
             check_nvfp4(make_input(shape, seed=40 + i, outliers=True), c, r)
+            numel = 1
+            for d in shape:
+                numel *= d
+            expect = PATH_SMALL if numel * 2 <= 256 * 1024 and timeout_us >= 0 else (PATH_ONEPASS if timeout_us >= 0 else PATH_TWO_KERNEL)
+            assert L.ac4k_debug_last_quantize_path() == expect, (shape, L.ac4k_debug_last_quantize_path())
             check_nvfp4(make_input(shape, seed=80 + i, outliers=True), c, r, swz=True)
         # repeated calls on one stream reuse the synchronisation words with a new launch number
         x = make_input((512, 1024), seed=3)
         for _ in range(5):
             check_nvfp4(x, 0, 1)
-        # scales that are not positive finite numbers go down the repair path
+        # scales that are not positive finite numbers take the full-range arithmetic
         check_nvfp4(torch.zeros(128, 256, dtype=torch.bfloat16), 0, 1)
-        z = make_input((128, 256), seed=5)
-        z[5, 7] = float("inf")
-        check_nvfp4(z, 0, 1)
+        check_nvfp4(torch.zeros(1024, 256, dtype=torch.bfloat16), 0, 1)
+        for rows in (128, 2048):
+            z = make_input((rows, 256), seed=5)
+            z[5, 7] = float("inf")
+            check_nvfp4(z, 0, 1)
+            z[5, 7] = float("nan")
+            check_nvfp4(z, 0, 1)
     finally:
         L.ac4k_set_quantize_sync_timeout_us(200)
 
@@ -165,18 +182,23 @@ def test_crossmajor_layouts(shape, cross, red, swz):
 
 
 def test_nvfp4_graph_replay():
-    """A captured quantize call replays correctly: nothing in it depends on host-side state that
-    changes from launch to launch, and eager calls in between do not disturb it."""
+    """A captured quantize call replays correctly: under capture the library takes the path whose whole
+    state is in the caller's buffers, so nothing in it depends on host-side state that changes from
+    launch to launch, and eager calls in between do not disturb it."""
+    from ac4k_kernel_amd import _lib
+    L = _lib.load()
     shape = (2048, 1024)
     static = make_input(shape, seed=1).cuda()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         ops().quantize(static, 0, 1)
+        assert L.ac4k_debug_last_quantize_path() == PATH_ONEPASS
     torch.cuda.current_stream().wait_stream(side)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         out, sf, gs = ops().quantize(static, 0, 1)
+        assert L.ac4k_debug_last_quantize_path() == PATH_TWO_KERNEL
     for seed in (11, 12, 13, 14):
         x = make_input(shape, seed=seed, outliers=True)
         static.copy_(x.cuda())
@@ -188,9 +210,66 @@ def test_nvfp4_graph_replay():
         check_nvfp4(make_input((300, 640), seed=seed), 0, 1)  # eager work between the replays
 
 
+def test_nvfp4_graph_replay_next_to_eager_calls():
+    """Two captured quantizes replay on a second stream while the capture stream and a third stream run
+    eager single-launch quantizes: captured calls share no state with anything, every result is exact."""
+    shapes = [(2048, 1024), (1024, 4096)]
+    xs = [make_input(sh, seed=30 + i, outliers=True) for i, sh in enumerate(shapes)]
+    exp = [T.quantize_nvfp4(x, 0, 1, False) for x in xs]
+    statics = [x.cuda() for x in xs]
+    graphs, outs = [], []
+    for st in statics:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            outs.append(ops().quantize(st, 0, 1))
+        graphs.append(g)
+    replay_stream, eager_stream = torch.cuda.Stream(), torch.cuda.Stream()
+    eager_in = make_input((4096, 2048), seed=77, outliers=True)
+    eager_exp = T.quantize_nvfp4(eager_in, 0, 1, False)
+    eager_dev = eager_in.cuda()
+    torch.cuda.synchronize()
+    eager_res = []
+    for rep in range(3):
+        with torch.cuda.stream(replay_stream):
+            for g in graphs:
+                g.replay()
+        eager_res.append(ops().quantize(eager_dev, 0, 1))          # on the stream the graphs were captured from
+        with torch.cuda.stream(eager_stream):
+            eager_res.append(ops().quantize(eager_dev, 0, 1))
+        torch.cuda.synchronize()
+        for (out, sf, gs), (eo, es, eg) in zip(outs, exp):
+            assert gs.item() == eg.item()
+            assert torch.equal(out.cpu(), eo) and torch.equal(sf.cpu().view(torch.uint8), es)
+    for out, sf, gs in eager_res:
+        assert gs.item() == eager_exp[2].item()
+        assert torch.equal(out.cpu(), eager_exp[0]) and torch.equal(sf.cpu().view(torch.uint8), eager_exp[1])
+
+
+def test_nvfp4_slots_are_recycled():
+    """A process that keeps creating and destroying streams keeps the single-launch path: the 100th
+    stream gets synchronisation words like the first."""
+    from ac4k_kernel_amd import _lib
+    L = _lib.load()
+    x = make_input((1024, 2048), seed=55, outliers=True)
+    exp = T.quantize_nvfp4(x, 0, 1, False)
+    dx = x.cuda()
+    torch.cuda.synchronize()
+    for i in range(100):
+        st = torch.cuda.Stream()
+        with torch.cuda.stream(st):
+            out, sf, gs = ops().quantize(dx, 0, 1)
+            assert L.ac4k_debug_last_quantize_path() == PATH_ONEPASS, i
+        st.synchronize()
+        if i % 33 == 0 or i == 99:
+            assert gs.item() == exp[2].item()
+            assert torch.equal(out.cpu(), exp[0]) and torch.equal(sf.cpu().view(torch.uint8), exp[1])
+        del st
+
+
 def test_nvfp4_many_streams():
-    """More (device, stream) pairs than the library has scratch slots: the late streams take the
-    paths without scratch and every result is still exact."""
+    """More streams at once than the library has sets of synchronisation words: late streams evict the
+    least recently used ones, whose kernels may still be waiting on those words - such a kernel stops
+    waiting after its timeout and finishes through its slow path.  Every result is still exact."""
     x = make_input((300, 640), seed=21, outliers=True)
     big = make_input((2048, 2048), seed=22)
     ex, eb = T.quantize_nvfp4(x, 0, 1, False), T.quantize_nvfp4(big, 0, 1, False)
