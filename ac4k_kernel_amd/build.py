@@ -78,5 +78,17 @@ def build(force: bool = False, verbose: bool = True, extra_flags=(), out: str = 
     return out
 
 
+TIMELINE_LIB_PATH = os.path.join(PKG_DIR, "libac4k_nvfp4_timeline.so")
+
+
+def build_timeline(verbose: bool = True) -> str:
+    """The same sources with the kernels' clock stamps compiled in (profiling aid, not the product):
+    load it with AC4K_NVFP4_LIB=<path> for `bench.py --workload quantize-timeline`."""
+    return build(force=True, verbose=verbose, extra_flags=["-DAC4K_ONEPASS_TIMELINE"], out=TIMELINE_LIB_PATH)
+
+
 if __name__ == "__main__":
-    print(build(force="--force" in sys.argv))
+    if "--timeline" in sys.argv:
+        print(build_timeline())
+    else:
+        print(build(force="--force" in sys.argv))

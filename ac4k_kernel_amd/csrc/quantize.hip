@@ -320,7 +320,7 @@ constexpr int OP_MAX_WGS = 256;
 constexpr int OP_MAX_NV = 16;
 constexpr int OP_SLOTS = 32;  // concurrent (device, stream) pairs with synchronisation words of their own
 struct OnePassSync {
-  uint32_t arrive[OP_SLOTS][OP_MAX_WGS];
+  uint32_t arrive[OP_SLOTS][OP_MAX_WGS];  // the words of 32 workgroups share a 128-byte line
 };
 __device__ __align__(256) OnePassSync g_onepass;
 
@@ -389,6 +389,9 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
   const uint32_t w = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
   AC4K_TL(0);
+  // The deadline of the grid wait counts from here: reading the 100 MHz clock takes about as long as a
+  // trip to memory, and here that time hides behind the loads.
+  const uint64_t t_end = wall_clock64() + timeout_ticks;
   uint32_t cb[NG], nvalid[NG];  // first chunk and number of chunks of each group
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
@@ -409,48 +412,67 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
     for (int j = 0; j < NV; ++j) v[j] = swizzle_nvfp4_quad(v[j], (int)lane);
   }
   if (tid < 128) lut[tid] = g_rcp_e4m3.v[tid];
-  uint32_t bm[NV];  // 16-block maxima (bf16 bits)
+  float bm6[NV];  // 16-block maxima times 1/6 (first product of the block scale; it does not need the global scale)
   {
     uint32_t m = 0;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-      bm[j] = absmax_bf16x8(v[j]);
-      bm[j] = umax32(bm[j], dpp_u32<DPP_QUAD_XOR1>(bm[j]));
-      m = umax32(m, bm[j]);
+      uint32_t b = absmax_bf16x8(v[j]);
+      b = umax32(b, dpp_u32<DPP_QUAD_XOR1>(b));
+      m = umax32(m, b);
+      bm6[j] = bf16_bits_to_f32(b) * 0.16666666666666666f;
+      asm volatile("" : "+v"(bm6[j]));  // formed here, while the loads are still arriving, not after the wait
     }
     m = group_umax<64>(m);
     if (lane == 0) red[wave] = m;
   }
   __syncthreads();
   AC4K_TL(1);
-  if (wave == 0) {
+  // The last wave publishes the workgroup's maximum; wave 0 polls (a wave that did both would wait for
+  // the store's acknowledgement, a round trip of its own, before its first poll returns).  The first
+  // poll goes out about 1 us after the store (40 x 64 cycles): measured on MI355X, a poll sent right
+  // behind the workgroup's own loads and store comes back about 3 us later, one sent 1 us later within
+  // 0.5 us, and until the last workgroup arrives there is nothing to see anyway (the workgroups finish
+  // their loads within about 2.5 us of each other).  Measured time from the last arrival until every
+  // workgroup knows the maximum: 3.1 us without the delay, 1.0 - 1.6 us with it; delays of 20 / 30 /
+  // 50 / 80 x 64 cycles gave up to 2.2 / 1.9 / 1.9 / 2.7 us.
+  if (wave == OP_THREADS / 64 - 1) {
     const uint32_t own = group_umax<16>(red[lane & 15]);
     if (lane == 0)
       __hip_atomic_store(&g_onepass.arrive[slot][w], (tag << 16) | own, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (wave == 0) {
+    const uint32_t own = group_umax<16>(red[lane & 15]);
     const uint32_t i0 = lane * 4;
-    const uint64_t t_end = wall_clock64() + timeout_ticks;
-    bool ok, r0, r1, r2, r3;
-    uint4 a;
-    while (true) {  // at least one poll, whatever the timeout
-      a = ld_coherent_u4(&g_onepass.arrive[slot][i0]);
-      r0 = (a.x >> 16) == tag;
-      r1 = (a.y >> 16) == tag;
-      r2 = (a.z >> 16) == tag;
-      r3 = (a.w >> 16) == tag;
-      const bool ready = (i0 + 0 >= nwg || r0) && (i0 + 1 >= nwg || r1) && (i0 + 2 >= nwg || r2) && (i0 + 3 >= nwg || r3);
-      ok = __all(ready);
-      if (ok || wall_clock64() >= t_end) break;
+    if (timeout_ticks) __builtin_amdgcn_s_sleep(40);
+    bool ok, r0, r1, r2, r3, lane_ready = false;
+    uint4 a = make_uint4(0, 0, 0, 0);
+    for (uint32_t it = 0;; ++it) {  // at least one poll, whatever the timeout
+      // only lanes that still miss one of their four words look again: towards the end of the wait a
+      // poll touches one or two lines instead of eight, and every workgroup polls the same ones
+      if (!lane_ready) a = ld_coherent_u4(&g_onepass.arrive[slot][i0]);
+      // (the own word counts as published: its store may not have reached memory yet)
+      r0 = (a.x >> 16) == tag || i0 + 0 == w;
+      r1 = (a.y >> 16) == tag || i0 + 1 == w;
+      r2 = (a.z >> 16) == tag || i0 + 2 == w;
+      r3 = (a.w >> 16) == tag || i0 + 3 == w;
+      lane_ready = (i0 + 0 >= nwg || r0) && (i0 + 1 >= nwg || r1) && (i0 + 2 >= nwg || r2) && (i0 + 3 >= nwg || r3);
+      ok = __all(lane_ready);
+      if (ok) break;
+      // the clock is looked at on every fourth poll only (and at once when the bound is zero)
+      if ((timeout_ticks == 0 || (it & 3) == 3) && wall_clock64() >= t_end) break;
       __builtin_amdgcn_s_sleep(2);
     }
     // maxima that were published under this launch's tag; the others are marked for recomputation
+    // (the own word may be stale in `a`: its maximum comes from `own`)
     uint32_t mm = own;
-    mm = umax32(mm, (i0 + 0 < nwg && r0) ? a.x & 0xffffu : 0u);
-    mm = umax32(mm, (i0 + 1 < nwg && r1) ? a.y & 0xffffu : 0u);
-    mm = umax32(mm, (i0 + 2 < nwg && r2) ? a.z & 0xffffu : 0u);
-    mm = umax32(mm, (i0 + 3 < nwg && r3) ? a.w & 0xffffu : 0u);
+    mm = umax32(mm, (i0 + 0 < nwg && r0 && i0 + 0 != w) ? a.x & 0xffffu : 0u);
+    mm = umax32(mm, (i0 + 1 < nwg && r1 && i0 + 1 != w) ? a.y & 0xffffu : 0u);
+    mm = umax32(mm, (i0 + 2 < nwg && r2 && i0 + 2 != w) ? a.z & 0xffffu : 0u);
+    mm = umax32(mm, (i0 + 3 < nwg && r3 && i0 + 3 != w) ? a.w & 0xffffu : 0u);
     mm = group_umax<64>(mm);
-    miss4[lane] = ((i0 + 0 < nwg && !r0 && i0 + 0 != w) ? 1u : 0u) | ((i0 + 1 < nwg && !r1 && i0 + 1 != w) ? 0x100u : 0u) |
-                  ((i0 + 2 < nwg && !r2 && i0 + 2 != w) ? 0x10000u : 0u) | ((i0 + 3 < nwg && !r3 && i0 + 3 != w) ? 0x1000000u : 0u);
+    miss4[lane] = ((i0 + 0 < nwg && !r0) ? 1u : 0u) | ((i0 + 1 < nwg && !r1) ? 0x100u : 0u) |
+                  ((i0 + 2 < nwg && !r2) ? 0x10000u : 0u) | ((i0 + 3 < nwg && !r3) ? 0x1000000u : 0u);
     if (lane == 0) {
       gmax_s = mm;
       helping_s = ok ? 0u : 1u;
@@ -478,48 +500,68 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
   const bool fast = alpha > 0.0f && alpha < __builtin_inff();
 
   uint8_t *sfb = reinterpret_cast<uint8_t *>(sfs);
-  auto emit = [&](auto full_range) {
-    constexpr bool FULL = decltype(full_range)::value;
+  if (fast) {
 #pragma unroll
     for (int q = 0; q < NG; ++q) {
-      uint32_t code[GS];
-      float o[GS];
+      // block scale codes, four to a register (two conversions), and the multipliers
+      uint32_t codes[(GS + 3) / 4];
+      float oo[GS];
 #pragma unroll
-      for (int jj = 0; jj < GS; ++jj) {
-        const int j = q * GS + jj;
-        if (FULL) {
-          o[jj] = nvfp4_block_scale(bf16_bits_to_f32(bm[j]), alpha, lut, code[jj]);
-        } else {
-          const float s32 = alpha * (bf16_bits_to_f32(bm[j]) * 0.16666666666666666f);
-          code[jj] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(s32, 0.0f, 0, false);
-          o[jj] = lut[code[jj]];
-        }
+      for (int c4 = 0; c4 < (GS + 3) / 4; ++c4) {
+        float s32[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s32[i] = c4 * 4 + i < GS ? alpha * bm6[q * GS + c4 * 4 + i] : 0.0f;
+        int wd = __builtin_amdgcn_cvt_pk_fp8_f32(s32[0], s32[1], 0, false);
+        codes[c4] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(s32[2], s32[3], wd, true);
       }
+#pragma unroll
+      for (int jj = 0; jj < GS; ++jj) oo[jj] = alpha * lut[(codes[jj / 4] >> (8 * (jj % 4))) & 0xffu];
+      uint32_t *op = out + (uint64_t)cb[q] * 8 + tid;
+      uint8_t *sp = sfb + q * GC * 4 + (tid >> 1);
+      // a whole group (every group but the tensor's last ones) needs no predicates at all
+      auto store_group = [&](auto whole_group) {
+        constexpr bool WHOLE = decltype(whole_group)::value;
+#pragma unroll
+        for (int jj = 0; jj < GS; ++jj) {
+          const int j = q * GS + jj;
+          const float m_ = oo[jj];
+          const float f[8] = {bf16_lo(v[j].x) * m_, bf16_hi(v[j].x) * m_, bf16_lo(v[j].y) * m_, bf16_hi(v[j].y) * m_,
+                              bf16_lo(v[j].z) * m_, bf16_hi(v[j].z) * m_, bf16_lo(v[j].w) * m_, bf16_hi(v[j].w) * m_};
+          const uint32_t packed = f32x8_to_e2m1x8(f);
+          if (WHOLE || ((jj * OP_THREADS + tid) >> 3) < nvalid[q]) st_stream_u1(op + jj * OP_THREADS, packed);
+        }
+        // scale byte (lv % 8) / 2 of chunk lv / 8; both lanes of a 16-block hold the same code
+        if ((lane & 1) == 0) {
+#pragma unroll
+          for (int jj = 0; jj < GS; ++jj)
+            if (WHOLE || ((jj * OP_THREADS + tid) >> 3) < nvalid[q])
+              sp[jj * (OP_THREADS / 2)] = (uint8_t)(codes[jj / 4] >> (8 * (jj % 4)));
+        }
+      };
+      if (nvalid[q] == GC)  // workgroup-uniform
+        store_group(std::true_type{});
+      else
+        store_group(std::false_type{});
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < NG; ++q) {
 #pragma unroll
       for (int jj = 0; jj < GS; ++jj) {
         const int j = q * GS + jj;
         const uint32_t lv = jj * OP_THREADS + tid;
-        uint32_t packed;
-        if (FULL) {
-          packed = nvfp4_pack8(v[j], o[jj]);
-        } else {
-          const float oo = alpha * o[jj];
-          const float f[8] = {bf16_lo(v[j].x) * oo, bf16_hi(v[j].x) * oo, bf16_lo(v[j].y) * oo, bf16_hi(v[j].y) * oo,
-                              bf16_lo(v[j].z) * oo, bf16_hi(v[j].z) * oo, bf16_lo(v[j].w) * oo, bf16_hi(v[j].w) * oo};
-          packed = f32x8_to_e2m1x8(f);
-        }
+        uint32_t code;
+        // (amax / 6 was formed before the wait; nvfp4_block_scale forms the same product)
+        const float s32 = alpha * bm6[j];
+        code = f32_to_ue4m3_satfinite(s32);
+        const uint32_t packed = nvfp4_pack8(v[j], alpha * lut[code]);
         if ((lv >> 3) < nvalid[q]) {
           st_stream_u1(out + (uint64_t)cb[q] * 8 + lv, packed);
-          // scale byte (lv % 8) / 2 of chunk lv / 8; both lanes of a 16-block hold the same code
-          if ((lane & 1) == 0) sfb[q * GC * 4 + (lv >> 1)] = (uint8_t)code[jj];
+          if ((lane & 1) == 0) sfb[q * GC * 4 + (lv >> 1)] = (uint8_t)code;
         }
       }
     }
-  };
-  if (fast)
-    emit(std::false_type{});
-  else
-    emit(std::true_type{});
+  }
   __syncthreads();
   AC4K_TL(3);
   // scales: LDS holds one dword per chunk in (row, chunk column) order; memory wants, per chunk
@@ -1353,3 +1395,15 @@ extern "C" __attribute__((visibility("default"))) int ac4k_quantize_int8(void *o
 extern "C" __attribute__((visibility("default"))) void ac4k_set_quantize_sync_timeout_us(int64_t us) {
   ac4k::g_sync_timeout_ticks.store(us < 0 ? -1 : us * 100);
 }
+
+#ifdef AC4K_ONEPASS_TIMELINE
+// Timeline build only: copies the per-workgroup clock stamps of the last single-launch quantize to
+// host memory ([256][8] 100 MHz ticks: 0 kernel entry, 1 loads in registers and own maximum known,
+// 2 global maximum known, 3 nibbles stored, 4 scales stored).  Synchronises the device.
+extern "C" __attribute__((visibility("default"))) int ac4k_debug_onepass_timeline(uint64_t *host_out) {
+  hipError_t e = hipDeviceSynchronize();
+  if (e == hipSuccess)
+    e = hipMemcpyFromSymbol(host_out, HIP_SYMBOL(ac4k::g_onepass_timeline), sizeof(uint64_t) * ac4k::OP_MAX_WGS * 8);
+  return e == hipSuccess ? 0 : ac4k::set_error("ac4k_debug_onepass_timeline: %s", hipGetErrorString(e));
+}
+#endif

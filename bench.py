@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the NVFP4 path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|linear|quantize|traffic]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|linear|quantize|traffic|quantize-timeline]
                     [--no-cpu-baseline] [--no-check]
 
 Prints ONE JSON line.  The headline `value` is the NVFP4 linear at M=N=K=8192 (the
@@ -425,13 +425,53 @@ def run_traffic(ops):
     print(json.dumps({"traffic_run": "done"}))
 
 
+def run_quantize_timeline(ops, reps=20):
+    """Phase boundaries of the single-launch nvfp4 quantizer from clock stamps inside the kernel
+    (needs the library built by `python ac4k_kernel_amd/build.py --timeline`, loaded through
+    AC4K_NVFP4_LIB).  Per phase: microseconds after the first workgroup's entry, over all
+    workgroups (min / mean / max), median over `reps` isolated launches."""
+    import ctypes
+    import statistics
+    from ac4k_kernel_amd import _lib
+    L = _lib.load()
+    fn = getattr(L, "ac4k_debug_onepass_timeline", None)
+    if fn is None:
+        sys.exit("bench.py: this library has no clock stamps; build with `python ac4k_kernel_amd/build.py --timeline` "
+                 "and set AC4K_NVFP4_LIB to the library it prints")
+    fn.restype, fn.argtypes = ctypes.c_int, [ctypes.c_void_p]
+    names = ["entry", "loads_done_own_max", "global_max_known", "nibbles_stored", "scales_stored"]
+    res = {}
+    for tag, shape, outl in (("cfg1_4096x4096", (4096, 4096), False), ("cfg2_8192x4096", (8192, 4096), True)):
+        xs = [make_input(shape, seed=s_, outliers=outl).cuda() for s_ in range(3)]
+        outs = [ops.quantize(x, 0, 1) for x in xs]
+        buf = (ctypes.c_uint64 * (256 * 8))()
+        rows = {n_: {"min": [], "mean": [], "max": []} for n_ in names}
+        for r in range(reps + 3):
+            j = r % 3
+            ops.quantize(xs[j], 0, 1, output=outs[j][0], sf=outs[j][1])
+            _lib.check(fn(buf))
+            if r < 3:
+                continue
+            t = [[buf[w * 8 + i] for i in range(5)] for w in range(256)]
+            t0 = min(x[0] for x in t)
+            for i, n_ in enumerate(names):
+                col = [(x[i] - t0) * 0.01 for x in t]
+                rows[n_]["min"].append(min(col)); rows[n_]["mean"].append(sum(col) / len(col)); rows[n_]["max"].append(max(col))
+        res[tag] = {n_: {k_: round(statistics.median(v), 2) for k_, v in d.items()} for n_, d in rows.items()}
+        log(f"[timeline] {tag}: us after the first workgroup's entry, min / mean / max over 256 workgroups (median of {reps} launches)")
+        for n_ in names:
+            d = res[tag][n_]
+            log(f"[timeline]   {n_:22s} {d['min']:7.2f} {d['mean']:7.2f} {d['max']:7.2f}")
+    print(json.dumps({"quantize_timeline_us": res}))
+
+
 def main():
     global SETTLE_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", choices=["all", "linear", "quantize", "traffic"])
+    ap.add_argument("--workload", default="all", choices=["all", "linear", "quantize", "traffic", "quantize-timeline"])
     ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
                     help="keep the untimed warm-up going for this long (clock ramp); 0 = exactly --warmup calls")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -456,6 +496,8 @@ def main():
 
     if args.workload == "traffic":
         return run_traffic(ops)
+    if args.workload == "quantize-timeline":
+        return run_quantize_timeline(ops)
     check = not args.no_check  # the GEMM checks: fp32 dequantize-matmul with torch ops on the GPU
     # The CPU leg (the only user of oracle/): the oracle timed on the host cores as `cpu_baseline`, and the
     # same oracle as the checker of the quantizers' GPU output.  --no-cpu-baseline skips all of it.
