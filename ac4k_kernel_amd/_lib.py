@@ -32,7 +32,7 @@ SIGNATURES = {
                                         _vp, _i64, _vp]),
     "ac4k_linear_nvfp4_skinny_static": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64,
                                                _vp]),
-    "ac4k_set_linear_tuning": (_int, [_int, _int, _int, _int]),
+    "ac4k_set_linear_tuning": (_int, [_int, _int, _int, _int, _int]),
     "ac4k_linear_nvfp4_fused_bf16": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int,
                                             _i64, _i64, _i64, _vp, _i64, _vp]),
 }

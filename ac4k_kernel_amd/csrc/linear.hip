@@ -1363,17 +1363,253 @@ static void launch_reduce(const SkinnyArgs &a, hipStream_t st) {
     hipLaunchKernelGGL((skinny_reduce_kernel<D_DT, BIAS_DT, 1>), dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, a);
 }
 
+// ===========================================================================
+// Decode-sized linear (1 <= M <= 32, K % 256 == 0): the weights are streamed once, through LDS.
+//
+// A workgroup (8 waves) owns 128 weight rows and a contiguous range of 256-k stages.  Weights, weight
+// scales, the packed activation rows and their scales go from global memory straight into an LDS ring
+// of ST_PS stages with LDS-DMA loads: lane l of a transfer fetches piece l % 8 of row l / 8, so eight
+// lanes read one 128-byte run of a row, and every request is a full 64-byte line.  (With loads into
+// registers in the MFMA operand layout every lane reads from a different row: four times the address
+// work per byte, and the partial sums of a K split on top.)  Wave (wn, kh) = (wave % 4, wave / 4) takes
+// weight rows 32 wn .. 32 wn + 31 and the 64-chunks 2 kh, 2 kh + 1 of every stage: its packed
+// fragments of the NEXT stage travel from LDS to registers while it decodes the current ones in
+// registers (weights and activation alike: 4 converts + 4 packed multiplies per 8 elements) and
+// issues D^T += W . Xhat^T with v_mfma_f32_32x32x16_f16, so a lane ends up with four consecutive n for
+// one m.  One workgroup barrier per stage: a stage costs about 0.45 us of barrier, transfer issue and
+// waits whatever its size, which is why it is 256 k long (128-k stages: 40 us on N = 28672, K = 8192).
+// The two k halves meet through LDS at the end, always added in the same order.  Activation rows past
+// M read row M - 1 and feed outputs that are never stored.  With one K range per tile the epilogue
+// applies gsA*gsB and the bias and stores D; with several (too few tiles to fill the GPU) the fp32
+// sums go to the caller's workspace and skinny_reduce_kernel adds the ranges in order.
+// ===========================================================================
+constexpr int ST_BN = 128;        // weight rows per workgroup
+constexpr int ST_THREADS = 512;
+constexpr int ST_BK = 256;        // k per stage (four 64-chunks)
+constexpr int ST_ROW = ST_BK / 2; // packed bytes per row per stage
+constexpr int ST_PS = 6;
+constexpr int ST_NPIECES = 4;     // LDS-DMA instructions per wave per stage
+constexpr int ST_OFF_B = 0;
+constexpr int ST_OFF_A = ST_OFF_B + ST_BN * ST_ROW;     // 32 packed activation rows
+constexpr int ST_OFF_SFB = ST_OFF_A + 32 * ST_ROW;      // weight scale dwords [chunk][128 rows]
+constexpr int ST_OFF_SFA = ST_OFF_SFB + 4 * ST_BN * 4;  // activation scale dwords [chunk][32 rows]
+constexpr int ST_STAGE_BYTES = ST_OFF_SFA + 4 * 32 * 4;
+constexpr int ST_LDS_BYTES = ST_PS * ST_STAGE_BYTES;
+static_assert(ST_LDS_BYTES <= 160 * 1024, "the ring must fit in the CU's LDS");
+static_assert((ST_PS - 3) * ST_NPIECES <= 63, "the wait counts must fit the 6-bit counter");
+static_assert(ST_LDS_BYTES >= 4 * 64 * 16 * 4, "the ring doubles as the exchange buffer of the two k halves");
+
+template <int D_DT, int BIAS_DT>
+__global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(SkinnyArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char stlds[];
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, r32 = lane & 31;
+  const int swave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wn = swave & 3, kh = swave >> 2;
+  const int64_t n0 = (int64_t)blockIdx.x * ST_BN;
+  const int nst_all = (int)(a.K / ST_BK);
+  const int s0 = (int)((int64_t)nst_all * blockIdx.y / a.split_k);
+  const int nst = (int)((int64_t)nst_all * (blockIdx.y + 1) / a.split_k) - s0;  // >= 1: split_k <= stages
+  const int64_t kb = a.K >> 1;
+
+  auto uniform_ptr = [](const void *p) {  // pin a wave-uniform pointer to scalar registers
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
+  };
+  // LDS holds row-major 128-byte rows (lane l of a transfer lands at 16 l: eight rows per transfer);
+  // the eight 16-byte pieces of row r sit at positions piece ^ (r & 7), which spreads a fragment read
+  // (one piece of each of 32 rows) over all LDS banks.  Unswizzled those reads fall on a quarter of the
+  // banks and, issued by eight waves every stage, held the transfers back (40 us against 31 us on
+  // N = 28672, K = 8192).
+  // --- this wave's four transfers of a stage: lane offsets (loop invariant), LDS destinations, sources
+  // (1, 2) weight rows swave * 16 + {0..7}, {8..15}, 128 B each
+  uint32_t offW[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int loc = swave * 16 + q * 8 + (lane >> 3);
+    int64_t row = n0 + loc;
+    row = row < a.N ? row : a.N - 1;  // rows past N read the last row; their outputs are never stored
+    offW[q] = (uint32_t)((row - n0) * kb + ((lane & 7) ^ (loc & 7)) * 16);
+  }
+  const uint8_t *srcW = uniform_ptr(a.B + n0 * kb + (int64_t)s0 * ST_ROW);
+  const uint32_t ldsW = (uint32_t)__builtin_amdgcn_readfirstlane(ST_OFF_B + swave * 2048);
+  // (3) weight scales: chunk swave / 2, rows (swave % 2) * 64 + lane of the tile
+  int64_t srow = n0 + (swave & 1) * 64 + lane;
+  srow = srow < a.Np ? srow : a.Np - 1;
+  const uint32_t offS = (uint32_t)(srow * 4);
+  const int64_t strideS = 4 * a.Np * 4;  // bytes per stage (four chunk planes)
+  const uint8_t *srcS = uniform_ptr(reinterpret_cast<const uint8_t *>(a.B_sf) + (int64_t)(swave >> 1) * a.Np * 4 + s0 * strideS);
+  const uint32_t ldsS = (uint32_t)__builtin_amdgcn_readfirstlane(ST_OFF_SFB + (swave >> 1) * (ST_BN * 4) + (swave & 1) * 256);
+  // (4) waves 0..3: packed activation rows swave * 8 + {0..7}; waves 4, 5: activation scales of chunks
+  //     2 (swave - 4) + {0, 1}; waves 6, 7 repeat those of waves 4, 5 (every wave issues the same count)
+  uint32_t off4, lds4;
+  const uint8_t *src4;
+  int64_t stride4;
+  if (swave < 4) {
+    const int loc = swave * 8 + (lane >> 3);
+    const int64_t row = loc < a.M ? loc : a.M - 1;  // rows past M read row M - 1; their outputs are never stored
+    off4 = (uint32_t)(row * kb + ((lane & 7) ^ (loc & 7)) * 16);
+    stride4 = ST_ROW;
+    src4 = uniform_ptr(a.Aq + (int64_t)s0 * ST_ROW);
+    lds4 = (uint32_t)__builtin_amdgcn_readfirstlane(ST_OFF_A + swave * 1024);
+  } else {
+    const int pair = swave & 1;  // chunks 2 pair, 2 pair + 1
+    const int64_t row = r32 < a.Mp ? r32 : a.Mp - 1;
+    off4 = (uint32_t)(((2 * pair + half) * a.Mp + row) * 4);
+    stride4 = 4 * a.Mp * 4;
+    src4 = uniform_ptr(a.A_sf + s0 * stride4);
+    lds4 = (uint32_t)__builtin_amdgcn_readfirstlane(ST_OFF_SFA + pair * 256);
+  }
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)stlds;
+  auto issue_stage = [&](int slot, int st) {  // st: stage index inside this workgroup's range
+    const uint32_t base = lds_base + slot * ST_STAGE_BYTES;
+    const uint8_t *pw = srcW + (int64_t)st * ST_ROW;
+    dma16(pw, offW[0], base, ldsW);
+    dma16(pw, offW[1], base, ldsW + 1024);
+    dma4(srcS + st * strideS, offS, base, ldsS);
+    if (swave < 4)
+      dma16(src4 + st * stride4, off4, base, lds4);
+    else
+      dma4(src4 + st * stride4, off4, base, lds4);
+  };
+
+  // this wave's fragments of one stage: for each of its two 64-chunks (2 kh, 2 kh + 1) 32 packed
+  // elements of a weight row and of an activation row (the lane's half of the chunk) and the two block
+  // scales of each
+  struct StageFrags {
+    uint4 w[2], x[2];
+    uint32_t ws[2], xs[2];
+  };
+  const int wrow_l = wn * 32 + r32;
+  int wf_off[2], xf_off[2];
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const int piece = kh * 4 + c * 2 + half;
+    wf_off[c] = ST_OFF_B + wrow_l * ST_ROW + ((piece ^ (wrow_l & 7)) * 16);
+    xf_off[c] = ST_OFF_A + r32 * ST_ROW + ((piece ^ (r32 & 7)) * 16);
+  }
+  const int ws_off = ST_OFF_SFB + (kh * 2) * (ST_BN * 4) + wrow_l * 4 + half * 2;
+  const int xs_off = ST_OFF_SFA + (kh * 2) * (32 * 4) + r32 * 4 + half * 2;
+  auto load_frags = [&](int slot) {
+    const char *st = stlds + slot * ST_STAGE_BYTES;
+    StageFrags f;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      f.w[c] = *reinterpret_cast<const uint4 *>(st + wf_off[c]);
+      f.x[c] = *reinterpret_cast<const uint4 *>(st + xf_off[c]);
+      f.ws[c] = *reinterpret_cast<const uint16_t *>(st + ws_off + c * (ST_BN * 4));
+      f.xs[c] = *reinterpret_cast<const uint16_t *>(st + xs_off + c * (32 * 4));
+    }
+    return f;
+  };
+
+  f32x16 acc[2];  // one per chunk of the pair: two independent accumulation chains
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[c][e] = 0.0f;
+
+  // prologue: stages 0 .. PS-2 in flight (past the range: the last stage again, into slots nobody
+  // reads), stages 0 and 1 landed, fragments of stage 0 in registers
+  const int last = nst - 1;
+#pragma unroll
+  for (int d = 0; d < ST_PS - 1; ++d) issue_stage(d, d < last ? d : last);
+  wait_vmcnt<(ST_PS - 3) * ST_NPIECES>();
+  __syncthreads();
+  StageFrags cur = load_frags(0);
+
+  int slot_next = 1, slot_dma = ST_PS - 1;
+  for (int s = 0; s < nst; ++s) {
+    // fragments of the next stage (it landed before the previous barrier) travel from LDS while this
+    // stage is decoded and multiplied (past the range: a stage nobody uses)
+    const StageFrags nxt = load_frags(slot_next);
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const f16x2 wsc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(cur.ws[c], 1.0f, false);
+      const f16x2 xsc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(cur.xs[c], 1.0f, false);
+      acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<false>(cur.w[c].x, wsc), decode_dword<false>(cur.x[c].x, xsc), acc[c], 0, 0, 0);
+      acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<false>(cur.w[c].y, wsc), decode_dword<false>(cur.x[c].y, xsc), acc[c], 0, 0, 0);
+      acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<true>(cur.w[c].z, wsc), decode_dword<true>(cur.x[c].z, xsc), acc[c], 0, 0, 0);
+      acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<true>(cur.w[c].w, wsc), decode_dword<true>(cur.x[c].w, xsc), acc[c], 0, 0, 0);
+    }
+    // refill the slot of the stage before this one (everybody read it before the previous barrier)
+    const int sd = s + ST_PS - 1;
+    issue_stage(slot_dma, sd < last ? sd : last);
+    wait_vmcnt<(ST_PS - 3) * ST_NPIECES>();  // own transfers of stage s + 2 have landed
+    __syncthreads();
+    cur = nxt;
+    slot_next = slot_next + 1 == ST_PS ? 0 : slot_next + 1;
+    slot_dma = slot_dma + 1 == ST_PS ? 0 : slot_dma + 1;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-DMA may land after this point: the ring is reused
+  __syncthreads();
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[0][e] += acc[1][e];
+  // the sums of the upper k half join those of the lower one (always in this order)
+  float4 *xch = reinterpret_cast<float4 *>(stlds) + (wn * 64 + lane) * 4;
+  if (kh == 1) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) xch[g] = make_float4(acc[0][4 * g], acc[0][4 * g + 1], acc[0][4 * g + 2], acc[0][4 * g + 3]);
+  }
+  __syncthreads();
+  if (kh == 1) return;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const float4 o = xch[g];
+    acc[0][4 * g] += o.x; acc[0][4 * g + 1] += o.y; acc[0][4 * g + 2] += o.z; acc[0][4 * g + 3] += o.w;
+  }
+
+  // acc: lane <-> m = r32, element e <-> n = (e >> 2) * 8 + half * 4 + (e & 3): four consecutive n per group
+  const int m = r32;
+  if (m >= (int)a.M) return;
+  const int64_t nw = n0 + wn * 32;
+  if (a.split_k > 1) {
+    float *pp = a.partial + ((int64_t)blockIdx.y * a.M + m) * a.N;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int64_t n = nw + g * 8 + half * 4;
+      if (n + 3 < a.N && (a.N & 3) == 0) {
+        *reinterpret_cast<float4 *>(pp + n) = make_float4(acc[0][4 * g], acc[0][4 * g + 1], acc[0][4 * g + 2], acc[0][4 * g + 3]);
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (n + q < a.N) pp[n + q] = acc[0][4 * g + q];
+      }
+    }
+    return;
+  }
+  using DE = Elem<D_DT>;
+  typename DE::T *Dp = static_cast<typename DE::T *>(a.D);
+  const float scale = (*a.A_gs) * (*a.B_gs);
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int64_t n = nw + (e >> 2) * 8 + half * 4 + (e & 3);
+    if (n < a.N) {
+      float v = acc[0][e] * scale;
+      if constexpr (BIAS_DT != BIAS_NONE) v += Elem<BIAS_DT>::load(a.bias, n);
+      Dp[(int64_t)m * a.N + n] = DE::cvt(v);
+    }
+  }
+}
+
+// Plan of a decode-sized linear: which of the two kernels, its K split and the fp32 scratch it needs.
+enum { DECODE_REGISTERS = 1, DECODE_LDS_RING = 2 };
 struct SkinnyPlan {
-  int ks_len, split_k;
+  int kind;                // DECODE_REGISTERS: linear_nvfp4_skinny_kernel; DECODE_LDS_RING: linear_nvfp4_stream_kernel
+  int ks_len;              // register kernel: k per workgroup (256, 512 or 1024)
+  int split_k;             // K ranges; > 1 needs `partial_bytes` of fp32 scratch
   int64_t partial_bytes, groups;
   int lds_bytes;
 };
+static std::atomic<int> g_forced_decode_kernel{0};  // ac4k_set_linear_tuning: 0 = by shape
 
-static bool skinny_plan(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
-  if (M < 1 || M > 32 || K % SK_STEP != 0 || N < 1) return false;
+// Register kernel: K slices of up to 1024, halved until about 768 workgroups are in flight.
+static void plan_registers(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
   int ks = 1024;
-  if (const int f = g_forced_skinny_ks.load(std::memory_order_relaxed)) ks = f;  // 256, 512 or 1024
+  const int f = g_forced_skinny_ks.load(std::memory_order_relaxed);
+  if (f == 256 || f == 512 || f == 1024) ks = f;
   while (ks > SK_STEP && K % ks != 0) ks >>= 1;
+  p.kind = DECODE_REGISTERS;
   p.groups = ceil_div(N, SK_ROWS);
   // short problems: use smaller slices to get enough workgroups in flight
   while (ks > SK_STEP && p.groups * (K / ks) < 768) ks >>= 1;
@@ -1381,6 +1617,47 @@ static bool skinny_plan(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
   p.split_k = (int)(K / ks);
   p.partial_bytes = p.split_k > 1 ? (int64_t)p.split_k * M * N * 4 : 0;
   p.lds_bytes = (int)M * ((M > 16 && ks == 1024 ? 512 : ks) * 2 + 16);
+}
+
+// LDS-ring kernel: one K range per 128-row tile when the tiles alone fill the GPU; otherwise the
+// smallest number of ranges that gives about 200 workgroups, each range at least two stages long.
+static void plan_lds_ring(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
+  p.kind = DECODE_LDS_RING;
+  p.groups = ceil_div(N, ST_BN);
+  const int64_t stages = K / ST_BK;
+  int64_t splits = 1;
+  if (const int f = g_forced_skinny_ks.load(std::memory_order_relaxed)) {  // forced length of a K range
+    splits = K / f;
+  } else if (p.groups < 192) {
+    splits = ceil_div(200, p.groups);
+    if (splits > stages / 2) splits = stages / 2;
+    if (splits > 32) splits = 32;
+  }
+  if (splits < 1) splits = 1;
+  if (splits > stages) splits = stages;
+  p.ks_len = 0;
+  p.split_k = (int)splits;
+  p.partial_bytes = splits > 1 ? splits * M * N * 4 : 0;
+  p.lds_bytes = ST_LDS_BYTES;
+}
+
+// Shapes of the decode-sized kernels (both need K % 256 == 0) and the choice between them: the
+// register kernel streams a little faster at small M (all its loads are in flight at once, four
+// workgroups per CU) but pays for partial sums and a second launch, and its registers run out as M
+// grows; the LDS-ring kernel takes nearly the same time for every M <= 32 and needs no second launch
+// when N alone fills the GPU.  Measured, linear alone, register / LDS-ring kernel in us:
+//   N = 28672, K = 8192:  M = 1 30.9 / 34.0, M = 8 34.7 / 34.5, M = 12 37.2 / 35.9, M = 16 41.0 / 37.0, M = 32 45.2 / 37.9
+//   N = 14336, K = 4096:  M = 8 14.3 / 16.2, M = 12 16.1 / 16.2, M = 16 17.0 / 16.2, M = 32 21.8 / 16.8
+//   N = 4096, K = 14336:  M = 8 16.2 / 17.3, M = 12 17.2 / 17.5, M = 16 18.2 / 17.4, M = 32 22.2 / 17.9
+static bool skinny_plan(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
+  if (M < 1 || M > 32 || K % SK_STEP != 0 || N < 1) return false;
+  const bool ring_ok = (K >> 1) * ST_BN < (1ll << 31) && N < (1ll << 27);  // 32-bit lane offsets
+  int kind = g_forced_decode_kernel.load(std::memory_order_relaxed);
+  if (kind == 0) kind = M >= 12 ? DECODE_LDS_RING : DECODE_REGISTERS;
+  if (kind == DECODE_LDS_RING && ring_ok)
+    plan_lds_ring(M, N, K, p);
+  else
+    plan_registers(M, N, K, p);
   return true;
 }
 
@@ -1390,15 +1667,25 @@ static int launch_skinny_it(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_
   static std::atomic<uint32_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, lds_ok, 32 * (1024 * 2 + 16))) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)p.split_k, (unsigned)p.groups), dim3(256), p.lds_bytes, st, a);
-  if (p.split_k > 1) launch_reduce<D_DT, BIAS_DT>(a, st);
   return 0;
 }
 
 template <int D_DT, int BIAS_DT>
 static int launch_skinny(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_t st) {
-  if (a.M <= 8) return launch_skinny_it<D_DT, BIAS_DT, 1>(a, p, st);
-  if (a.M <= 16) return launch_skinny_it<D_DT, BIAS_DT, 2>(a, p, st);
-  return launch_skinny_it<D_DT, BIAS_DT, 4>(a, p, st);
+  if (p.kind == DECODE_LDS_RING) {
+    auto *kern = linear_nvfp4_stream_kernel<D_DT, BIAS_DT>;
+    static std::atomic<uint32_t> lds_ok{0};
+    if (int rc = allow_dynamic_lds(kern, lds_ok, ST_LDS_BYTES)) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)p.groups, (unsigned)p.split_k), dim3(ST_THREADS), ST_LDS_BYTES, st, a);
+  } else {
+    int rc;
+    if (a.M <= 8) rc = launch_skinny_it<D_DT, BIAS_DT, 1>(a, p, st);
+    else if (a.M <= 16) rc = launch_skinny_it<D_DT, BIAS_DT, 2>(a, p, st);
+    else rc = launch_skinny_it<D_DT, BIAS_DT, 4>(a, p, st);
+    if (rc) return rc;
+  }
+  if (p.split_k > 1) launch_reduce<D_DT, BIAS_DT>(a, st);
+  return 0;
 }
 
 template <int D_DT>
@@ -1676,7 +1963,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_fused_bf
   const bool ok = skinny_plan(M, N, K, p);
   if (int rc = check_skinny(p, ok, B, workspace, workspace_bytes)) return rc;
   hipStream_t st = (hipStream_t)stream;
-  AC4K_REQUIRE(K % 64 == 0 && ((uintptr_t)X & 15) == 0, "activation must be 16-byte aligned with K %% 64 == 0");
+  AC4K_REQUIRE(((uintptr_t)X & 15) == 0, "activation must be 16-byte aligned");
   if (int rc = ac4k_quantize_nvfp4_bf16(X_q, X_sf, X_gs, X, 1, 1, M, K, 0, 0, K, 1, 0, 2688.0f, stream)) return rc;
   if (int rc = run_skinny(D, d_dtype, X_q, X_sf, X_gs, B, B_sf, B_gs, bias, bias_dtype, M, N, K, p, workspace,
                           st))
@@ -1684,7 +1971,11 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_fused_bf
   return check_launch("ac4k_linear_nvfp4_fused_bf16");
 }
 
-extern "C" __attribute__((visibility("default"))) int ac4k_set_linear_tuning(int mi, int nj, int splits, int skinny_ks) {
+extern "C" __attribute__((visibility("default"))) int ac4k_set_linear_tuning(int mi, int nj, int splits, int skinny_ks,
+                                                                          int decode_kernel) {
+  AC4K_REQUIRE(decode_kernel >= 0 && decode_kernel <= 2,
+               "decode_kernel must be 0 (by shape), 1 (register kernel) or 2 (LDS-ring kernel) (got %d)", decode_kernel);
+  ac4k::g_forced_decode_kernel.store(decode_kernel);
   if (mi == 0 && nj == 0 && splits == 0) {
     ac4k::g_forced_tile_plan.store(0);
   } else {
@@ -1693,8 +1984,8 @@ extern "C" __attribute__((visibility("default"))) int ac4k_set_linear_tuning(int
                  "tile plan must be mi in {2,4}, nj in {1,2,4} (not 4,1), 1 <= splits (got %d,%d,%d)", mi, nj, splits);
     ac4k::g_forced_tile_plan.store((uint32_t)mi | ((uint32_t)nj << 8) | ((uint32_t)splits << 16));
   }
-  AC4K_REQUIRE(skinny_ks == 0 || skinny_ks == 256 || skinny_ks == 512 || skinny_ks == 1024,
-               "skinny_ks must be 0 (automatic), 256, 512 or 1024 (got %d)", skinny_ks);
+  AC4K_REQUIRE(skinny_ks >= 0 && skinny_ks % 256 == 0, "skinny_ks must be 0 (automatic) or a multiple of 256 (got %d)",
+               skinny_ks);
   ac4k::g_forced_skinny_ks.store(skinny_ks);
   return 0;
 }

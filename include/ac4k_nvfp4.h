@@ -116,8 +116,9 @@ int ac4k_linear_nvfp4(void *D, int d_dtype, const void *A, const void *A_sf, con
 /* Linear for shapes that need device scratch to run well: same contract as ac4k_linear_nvfp4
  * (lib/cuda/sm120/linear_nvfp4.cu:753-901; the reference runs every shape through its one
  * 128x128 tile kernel).  Two families:
- *   - decode-sized, 1 <= M <= 32 and K % 256 == 0: a weight-streaming split-K kernel; the
- *     workspace receives the fp32 partial sums of the K-slices; A and B 16-byte aligned;
+ *   - decode-sized, 1 <= M <= 32 and K % 256 == 0: kernels that stream the weights once (into
+ *     registers for M < 12, through an LDS ring above); the workspace receives the fp32 partial sums
+ *     of their K ranges when they split K; A and B 16-byte aligned;
  *   - 32 < M with too few output tiles to fill the GPU and K % 128 == 0: split-K over the tile
  *     kernel (tile shape and number of K ranges chosen by a cost model); the workspace receives
  *     the fp32 partial sums; A and B 16-byte aligned.
@@ -149,9 +150,11 @@ int ac4k_linear_nvfp4_skinny_static(void *D, int d_dtype, const void *A, const v
 /* Tuning aid of the linear entry points (no counterpart in the reference; results stay within the
  * same tolerance): forces the tile of the packed-operand kernel to (64 mi) x (64 nj) with `splits` K
  * ranges (mi in {2,4}, nj in {1,2,4}, not (4,1); splits > 1 only takes effect in the workspace entry
- * points) and the K slice of the decode-sized kernel (256, 512 or 1024).  Zeros give the choice back
- * to the library's cost model.  Process-wide; returns non-zero on values outside these sets. */
-int ac4k_set_linear_tuning(int mi, int nj, int splits, int skinny_ks);
+ * points), the length of a K range of the decode-sized kernels (a multiple of 256; the register
+ * kernel takes 256, 512 or 1024) and which decode-sized kernel runs (1 = weights streamed into
+ * registers, 2 = weights streamed through an LDS ring).  Zeros give each choice back to the library.
+ * Process-wide; returns non-zero on values outside these sets. */
+int ac4k_set_linear_tuning(int mi, int nj, int splits, int skinny_ks, int decode_kernel);
 
 /* Fused decode-sized linear: quantize(X,0,1) followed by linear(...) in one call.  No single
  * reference function: it equals the composition the reference's tests make

@@ -39,8 +39,8 @@ def linear_tuning():
     from ac4k_kernel_amd import _lib
     lib = _lib.load()
 
-    def force(mi=0, nj=0, splits=0, skinny_ks=0):
-        _lib.check(lib.ac4k_set_linear_tuning(mi, nj, splits, skinny_ks))
+    def force(mi=0, nj=0, splits=0, skinny_ks=0, decode_kernel=0):
+        _lib.check(lib.ac4k_set_linear_tuning(mi, nj, splits, skinny_ks, decode_kernel))
 
     yield force
-    lib.ac4k_set_linear_tuning(0, 0, 0, 0)
+    lib.ac4k_set_linear_tuning(0, 0, 0, 0, 0)

@@ -63,9 +63,10 @@ def test_argument_rejection_without_gpu():
     rc = lib.ac4k_quantize_nvfp4_bf16(one, one, one, one, 1, 3, 4, 64, 0, 0, 64, 1, 0, 2688.0, None)
     assert rc != 0 and b"strides must be positive" in lib.ac4k_last_error()
     # tuning values outside the instantiated kernels are refused, zeros are accepted
-    assert lib.ac4k_set_linear_tuning(4, 1, 1, 0) != 0 and b"tile plan" in lib.ac4k_last_error()
-    assert lib.ac4k_set_linear_tuning(0, 0, 0, 2048) != 0 and b"skinny_ks" in lib.ac4k_last_error()
-    assert lib.ac4k_set_linear_tuning(0, 0, 0, 0) == 0
+    assert lib.ac4k_set_linear_tuning(4, 1, 1, 0, 0) != 0 and b"tile plan" in lib.ac4k_last_error()
+    assert lib.ac4k_set_linear_tuning(0, 0, 0, 100, 0) != 0 and b"skinny_ks" in lib.ac4k_last_error()
+    assert lib.ac4k_set_linear_tuning(0, 0, 0, 0, 3) != 0 and b"decode_kernel" in lib.ac4k_last_error()
+    assert lib.ac4k_set_linear_tuning(0, 0, 0, 0, 0) == 0
     assert lib.ac4k_debug_last_quantize_path() in (0, 1, 2, 3)
     rc = lib.ac4k_linear_nvfp4_fused_bf16(one, 0, one, one, one, one, one, one, one, None, 0, 64, 4, 64, one, 0, None)
     assert rc != 0 and b"1 <= M <= 32" in lib.ac4k_last_error()

@@ -120,10 +120,15 @@ def test_linear_stays_inside_its_output(m, n, k, plan, odt, linear_tuning):
         assert same_bytes(w.t, ref), (m, n, k, plan, shift)
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 1000, 1024), (5, 136, 2048), (32, 520, 512), (128, 1024, 4096), (96, 300, 2048)])
-def test_workspace_linear_stays_inside_workspace_and_output(m, n, k):
+@pytest.mark.parametrize("kind", [0, 1, 2])  # decode-sized shapes: the library's choice, register kernel, LDS-ring kernel
+@pytest.mark.parametrize("m,n,k", [(1, 1000, 1024), (5, 136, 2048), (32, 520, 512), (16, 130, 3584), (128, 1024, 4096),
+                                   (96, 300, 2048)])
+def test_workspace_linear_stays_inside_workspace_and_output(m, n, k, kind, linear_tuning):
     from ac4k_kernel_amd import _lib
     L = _lib.load()
+    if kind and m > 32:
+        pytest.skip("the kernel choice only exists for decode-sized shapes")
+    linear_tuning(decode_kernel=kind)
     aq = ops().quantize(make_input((m, k), seed=m).cuda(), 0, 1)
     bq = ops().quantize(make_input((n, k), seed=n, std=0.02).cuda(), 0, 1)
     nbytes = L.ac4k_linear_nvfp4_skinny_workspace_bytes(m, n, k)

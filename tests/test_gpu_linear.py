@@ -204,6 +204,20 @@ def test_decode_sized_shapes(m, n, k):
     run_case(m, n, k, bias_dtype=torch.bfloat16, o_dtype=torch.float16, seed=n, wstd=0.02)
 
 
+# both decode-sized kernels at every M class (the library picks by M; here each is forced): ragged N,
+# one K range and several, every output / bias type
+@pytest.mark.parametrize("kind", [1, 2])
+@pytest.mark.parametrize("m", [1, 5, 8, 11, 12, 16, 17, 31, 32])
+def test_decode_kernels_forced(kind, m, linear_tuning):
+    linear_tuning(decode_kernel=kind)
+    for (n, k) in [(1000, 1024), (130, 256), (384, 3584), (4096, 2048)]:
+        run_case(m, n, k, seed=m + k + kind, wstd=0.02)
+    run_case(m, 520, 1536, bias_dtype=torch.float32, o_dtype=torch.float32, seed=m, wstd=0.02)
+    run_case(m, 200, 768, bias_dtype=torch.bfloat16, o_dtype=torch.float16, seed=m + 1, wstd=0.02)
+    linear_tuning(skinny_ks=256, decode_kernel=kind)  # as many K ranges as K allows
+    run_case(m, 333, 1280, bias_dtype=torch.float16, seed=m + 2, wstd=0.02)
+
+
 @pytest.mark.parametrize("m", [1, 8, 32])
 def test_fused_decode_config5(m):
     n, k = 28672, 8192
