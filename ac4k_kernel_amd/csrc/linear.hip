@@ -736,10 +736,13 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   const int kt0 = (int)((int64_t)nkt_all * blockIdx.y / sk.splits);
   const int nkt = (int)((int64_t)nkt_all * (blockIdx.y + 1) / sk.splits) - kt0;
 
-  // LDS-DMA.  One transfer moves 16 rows x 64 B: lane l reads piece l%4 of row l/4, so four
-  // adjacent lanes cover one 64-byte sector, and lands at LDS base + 16*l, i.e. row-major 64-byte
-  // rows.  The 32-bit lane offset is loop invariant and the 64-bit part is a scalar base that
-  // advances by 64 bytes per stage.
+  // LDS-DMA.  One transfer moves 16 rows x 64 B: the four lanes 4r .. 4r+3 read the four 16-byte
+  // pieces of row r (one 64-byte sector) and land at LDS base + 16*l, i.e. row-major 64-byte rows.
+  // Piece p of row r sits at position p ^ ((r >> 1) & 3) of its row: a fragment read takes one piece
+  // of each of 32 rows, and unswizzled those addresses fall on a quarter of the LDS banks (an
+  // eight-way conflict on every ds_read_b128).  The 32-bit lane offset is loop invariant and the
+  // 64-bit part is a scalar base that advances by 64 bytes per stage.
+  const int dma_piece = (lane & 3) ^ ((lane >> 3) & 3);  // tile rows of a transfer start at a multiple of 16
   const int swave = __builtin_amdgcn_readfirstlane(wave);
   const int64_t kb = a.K >> 1;
   uint32_t offA[NDA], offB[NDB];
@@ -747,13 +750,13 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   for (int q = 0; q < NDA; ++q) {
     int64_t ra = (swave * NDA + q) * 16 + (lane >> 2);
     ra = tm * BM + ra < a.M ? ra : a.M - 1 - tm * BM;  // rows past the matrix read the last valid row
-    offA[q] = (uint32_t)(ra * kb + (lane & 3) * 16);
+    offA[q] = (uint32_t)(ra * kb + dma_piece * 16);
   }
 #pragma unroll
   for (int q = 0; q < NDB; ++q) {
     int64_t rb = (swave * NDB + q) * 16 + (lane >> 2);
     rb = tn * BN + rb < a.N ? rb : a.N - 1 - tn * BN;
-    offB[q] = (uint32_t)(rb * kb + (lane & 3) * 16);
+    offB[q] = (uint32_t)(rb * kb + dma_piece * 16);
   }
   auto uniform_ptr = [](const void *p) {  // pin a wave-uniform pointer to scalar registers
     const uint64_t v = (uint64_t)p;
@@ -842,8 +845,10 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   // fragment addresses inside a stage (bytes)
-  const int fa_off = (wm * (32 * MI) + (lane & 31)) * P_ROW + half * 16;
-  const int fb_off = PL::OFF_B + (wn * (32 * NJ) + (lane & 31)) * P_ROW + half * 16;
+  // (a lane's rows differ by multiples of 32, so the swizzle term of its row is (lane >> 1) & 3 for all of them)
+  const int fa_off = (wm * (32 * MI) + (lane & 31)) * P_ROW;
+  const int fb_off = PL::OFF_B + (wn * (32 * NJ) + (lane & 31)) * P_ROW;
+  const int piece_off[2] = {((0 + half) ^ ((lane >> 1) & 3)) * 16, ((2 + half) ^ ((lane >> 1) & 3)) * 16};  // chunk 0, chunk 1
   // a lane needs the two scale bytes of its half of the chunk: blocks 2*half, 2*half+1
   const int sa_off = PL::OFF_SFA + (wm * (32 * MI) + (lane & 31)) * 4 + half * 2;
   const int sb_off = PL::OFF_SFB + (wn * (32 * NJ) + (lane & 31)) * 4 + half * 2;
@@ -854,8 +859,8 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     const char *st = plds + stage_off;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      if (i < MI) PA[c][i] = *reinterpret_cast<const uint4 *>(st + fa_off + c * 32 + i * 32 * P_ROW);
-      if (i < NJ) PB[c][i] = *reinterpret_cast<const uint4 *>(st + fb_off + c * 32 + i * 32 * P_ROW);
+      if (i < MI) PA[c][i] = *reinterpret_cast<const uint4 *>(st + fa_off + piece_off[c] + i * 32 * P_ROW);
+      if (i < NJ) PB[c][i] = *reinterpret_cast<const uint4 *>(st + fb_off + piece_off[c] + i * 32 * P_ROW);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
