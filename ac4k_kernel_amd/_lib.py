@@ -33,6 +33,11 @@ SIGNATURES = {
     "ac4k_linear_nvfp4_skinny_static": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64,
                                                _vp]),
     "ac4k_set_linear_tuning": (_int, [_int, _int, _int, _int, _int]),
+    "ac4k_prepack_weight_nvfp4_bytes": (_i64, [_i64, _i64]),
+    "ac4k_prepack_weight_nvfp4": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
+    "ac4k_linear_nvfp4_prepacked_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "ac4k_linear_nvfp4_prepacked": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64,
+                                           _vp, _i64, _vp]),
     "ac4k_linear_nvfp4_fused_bf16": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int,
                                             _i64, _i64, _i64, _vp, _i64, _vp]),
 }

@@ -193,6 +193,46 @@ def linear_nvfp4(D, A, A_sf, A_global_scale, B, B_sf, B_global_scale, bias=None)
                                     B_global_scale.data_ptr(), bias_ptr, bias_tag, M, N, K, _stream()))
 
 
+def prepack_weight_nvfp4(B, B_sf) -> torch.Tensor:
+    """Weight image of B [N, K/2] / B_sf [K/64, align_up(N,16), 4] for linear_nvfp4_prepacked: a uint8
+    tensor of ac4k_prepack_weight_nvfp4_bytes(N, K) bytes.  K must be a multiple of 128."""
+    _check(B.dim() == 2, "b must be a 2d matrix")
+    _check_tensor(B, torch.uint8, "b")
+    N, K = B.size(0), B.size(1) * 2
+    _check(B_sf.dim() == 3, "scale_b must be a 3d matrix")
+    _check_tensor(B_sf, torch.float8_e4m3fn, "scale_", "b")
+    _check(B_sf.shape == ((K + 63) // 64, _align_up(N, 16), 4), "scale_b has an invalid shape")
+    nbytes = _L.ac4k_prepack_weight_nvfp4_bytes(N, K)
+    _check(nbytes > 0, "no weight image for N = {}, K = {}: K must be a multiple of 128", N, K)
+    image = torch.empty((nbytes,), dtype=torch.uint8, device=B.device)
+    _lib.check(_L.ac4k_prepack_weight_nvfp4(image.data_ptr(), B.data_ptr(), B_sf.data_ptr(), N, K, _stream()))
+    return image
+
+
+def linear_nvfp4_prepacked(D, A, A_sf, A_global_scale, W_image, B_global_scale, bias=None) -> None:
+    """linear_nvfp4 on a weight image made by prepack_weight_nvfp4 (N = D.size(1), K = 2 * A.size(1))."""
+    _check(isinstance(D, torch.Tensor) and D.dim() == 2, "d must be a 2d matrix")
+    _check(D.dtype in _DTYPE_TAG, "d must be bfloat16, half or float")
+    _check(D.is_cuda and D.is_contiguous(), "d must be contiguous")
+    M, N = D.shape
+    _check(A.dim() == 2 and A.size(0) == M, "A size(0) must be {}", M)
+    K = _check_linear_operand(A, A_sf, A_global_scale, M, "a")
+    _check_tensor(W_image, torch.uint8, "w_image")
+    _check(N > 0 and W_image.numel() == _L.ac4k_prepack_weight_nvfp4_bytes(N, K) and W_image.numel() > 0,
+           "w_image is not the weight image of a [{}, {}] weight", N, K)
+    _check_tensor(B_global_scale, torch.float32, "global_scale_", "b")
+    _check(B_global_scale.dim() == 0, "b_global_scale must be a scalar")
+    bias_ptr, bias_tag = _bias_args(bias, N)
+    if M == 0:
+        return
+    nbytes = _L.ac4k_linear_nvfp4_prepacked_workspace_bytes(M, N, K)
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=D.device) if nbytes > 0 else None
+    _lib.check(_L.ac4k_linear_nvfp4_prepacked(D.data_ptr(), _DTYPE_TAG[D.dtype], A.data_ptr(), A_sf.data_ptr(),
+                                              A_global_scale.data_ptr(), W_image.data_ptr(),
+                                              B_global_scale.data_ptr(), bias_ptr, bias_tag, M, N, K,
+                                              None if ws is None else ws.data_ptr(), nbytes, _stream()))
+
+
 def linear_nvfp4_fused(D, X, X_q, X_sf, X_global_scale, B, B_sf, B_global_scale, bias=None) -> None:
     """quantize(X, 0, 1) + linear_nvfp4 for a bf16 activation X [M, K], 1 <= M <= 32;
     X_q / X_sf / X_global_scale receive the quantized activation."""

@@ -28,7 +28,19 @@ struct LinearArgs {
   const float *A_gs, *B_gs;
   const void *bias;
   int64_t M, N, K, Mp, Np;
+  int prepacked = 0;  // B points at a weight image (W_BLOCK_BYTES blocks, see below) and B_sf is unused
 };
+
+// --- pre-packed weight image -----------------------------------------------------
+// Static weights can be re-laid once into the order the kernels fetch them: one block per
+// (128 rows, 128 k), blocks of a 128-row band consecutive along k, bands consecutive along n (N is
+// padded with zero rows to a whole band).  A block is the LDS stage picture of those rows: 128 rows x
+// 64 packed bytes with the 16-byte piece p of row r at position p ^ ((r >> 1) & 3), followed by the
+// scale dwords [2 chunks][128 rows].  Every LDS-DMA transfer of a stage then reads one contiguous
+// kilobyte, and a stage of the decode-sized kernel (256 k) is one contiguous run of two blocks.
+constexpr int W_BLOCK_ROWS = 128, W_BLOCK_K = 128;
+constexpr int W_BLOCK_DATA = W_BLOCK_ROWS * W_BLOCK_K / 2;            // 8192
+constexpr int W_BLOCK_BYTES = W_BLOCK_DATA + 2 * W_BLOCK_ROWS * 4;    // 9216
 
 // --- output / bias element types -------------------------------------------
 template <int DT>
@@ -86,6 +98,27 @@ __device__ __forceinline__ void decode8(uint32_t w, f16x2 sp, f16x2 (&h)[4]) {
   h[1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 256.0f, 1) * sp;
   h[2] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 256.0f, 2) * sp;
   h[3] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 256.0f, 3) * sp;
+}
+
+// --- workgroup -> output tile ---------------------------------------------------
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Workgroup `pid` is first
+// renumbered so that every XCD owns one contiguous run of the tile sequence, and the sequence walks
+// the tiles in bands of GROUP_M tile-rows, column by column inside a band: the workgroups resident
+// on one XCD at a time then cover a compact GROUP_M x (CUs / GROUP_M) patch and share its operand
+// panels through that L2.
+struct TileCoord {
+  int64_t m, n;
+};
+template <int GROUP_M>
+__device__ __forceinline__ TileCoord tile_of_workgroup(int64_t pid, int64_t tiles_m, int64_t tiles_n) {
+  const int64_t ntiles = tiles_m * tiles_n;
+  const int64_t per = ntiles / 8, rem = ntiles % 8;
+  const int64_t xcd = pid % 8, idx = pid / 8;
+  pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
+  const int64_t band = pid / (GROUP_M * tiles_n), in_band = pid % (GROUP_M * tiles_n);
+  const int64_t first_m = band * GROUP_M;
+  const int64_t rows = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+  return {first_m + in_band % rows, in_band / rows};
 }
 
 // ===========================================================================
@@ -149,22 +182,8 @@ __global__ __launch_bounds__(256) void linear_nvfp4_tile128_kernel(LinearArgs a)
   __shared__ __attribute__((aligned(16))) _Float16 sA[T_BM * T_BK];
   __shared__ __attribute__((aligned(16))) _Float16 sB[T_BN * T_BK];
 
-  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of tiles so
-  // its L2 sees neighbouring tiles, then walk tiles in groups of 8 tile-rows.
-  const int64_t tiles_m = ceil_div(a.M, T_BM), tiles_n = ceil_div(a.N, T_BN);
-  const int64_t ntiles = tiles_m * tiles_n;
-  int64_t pid = blockIdx.x;
-  {
-    const int64_t per = ntiles / 8, rem = ntiles % 8;
-    const int64_t xcd = pid % 8, idx = pid / 8;
-    pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
-  }
-  constexpr int GROUP_M = 8;
-  const int64_t group = pid / (GROUP_M * tiles_n);
-  const int64_t first_m = group * GROUP_M;
-  const int64_t gsize = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
-  const int64_t tm = first_m + (pid % (GROUP_M * tiles_n)) % gsize;
-  const int64_t tn = (pid % (GROUP_M * tiles_n)) / gsize;
+  const TileCoord tc = tile_of_workgroup<8>(blockIdx.x, ceil_div(a.M, T_BM), ceil_div(a.N, T_BN));
+  const int64_t tm = tc.m, tn = tc.n;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -232,253 +251,6 @@ __global__ __launch_bounds__(256) void linear_nvfp4_tile128_kernel(LinearArgs a)
     }
   }
 }
-
-// ===========================================================================
-// 256x256x64 tile kernel for large problems: 4 waves (2x2), each wave 128x128 = 4x4 MFMA
-// 32x32x16 tiles (256 fp32 accumulators per lane).  A wave tile this large halves the LDS
-// fragment traffic per flop against 64x64 wave tiles.  LDS is double buffered (2 x 64 KiB):
-// while the MFMAs consume K-step kt from one buffer, the packed slice of step kt+1 (already
-// in registers) is decoded into the other and the packed slice of step kt+2 is fetched.
-// Thread t owns row t of the A tile and row t of the B tile: 32 packed bytes + one scale
-// dword per K-step each.  Requires K % 64 == 0.
-// ===========================================================================
-constexpr int L_BM = 256, L_BN = 256, L_BK = 64;
-constexpr int L_TILE_HALVES = L_BM * L_BK;  // fp16 elements per operand tile
-
-struct PackedRow {
-  uint4 lo, hi;  // 64 nibbles: four 16-blocks
-  uint32_t sf;   // their four scale bytes
-};
-
-// `row` is clamped by the caller: rows past the matrix read the last valid row and feed
-// accumulators whose outputs are never stored, so the load needs no predicate.
-__device__ __forceinline__ PackedRow load_row(const uint8_t *base, const uint32_t *sf, int64_t rows_p,
-                                              int64_t K, int64_t row, int64_t kt) {
-  PackedRow r;
-  const uint4 *p = reinterpret_cast<const uint4 *>(base + row * (K >> 1) + kt * 32);
-  r.lo = p[0];
-  r.hi = p[1];
-  r.sf = sf[kt * rows_p + row];
-  return r;
-}
-
-// decode 16-block `q` (0..3) of a packed row into its two 16-byte LDS chunks
-__device__ __forceinline__ void decode_block_to_lds(_Float16 *tile, int row, int q, uint32_t w0, uint32_t w1,
-                                                    uint32_t sfw) {
-  f16x2 sp = scale_pattern(sfw >> (8 * q));
-  f16x2 lo[4], hi[4];
-  decode8(w0, sp, lo);
-  decode8(w1, sp, hi);
-  uint4 v0 = make_uint4(__builtin_bit_cast(uint32_t, lo[0]), __builtin_bit_cast(uint32_t, lo[1]),
-                        __builtin_bit_cast(uint32_t, lo[2]), __builtin_bit_cast(uint32_t, lo[3]));
-  uint4 v1 = make_uint4(__builtin_bit_cast(uint32_t, hi[0]), __builtin_bit_cast(uint32_t, hi[1]),
-                        __builtin_bit_cast(uint32_t, hi[2]), __builtin_bit_cast(uint32_t, hi[3]));
-  *reinterpret_cast<uint4 *>(tile + row * 64 + (((2 * q) ^ LDS_SWZ(row)) << 3)) = v0;
-  *reinterpret_cast<uint4 *>(tile + row * 64 + (((2 * q + 1) ^ LDS_SWZ(row)) << 3)) = v1;
-}
-
-__device__ __forceinline__ void decode_row_quarter(_Float16 *tile, int row, int q, const PackedRow &r) {
-  const uint32_t w[8] = {r.lo.x, r.lo.y, r.lo.z, r.lo.w, r.hi.x, r.hi.y, r.hi.z, r.hi.w};
-  decode_block_to_lds(tile, row, q, w[2 * q], w[2 * q + 1], r.sf);
-}
-
-struct Frags {
-  f16x8 a[4], b[4];
-};
-
-__device__ __forceinline__ void load_frags(Frags &f, const _Float16 *cA, const _Float16 *cB, int arow, int brow,
-                                           int chunk) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) f.a[i] = lds_frag(cA, arow + i * 32, chunk);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) f.b[j] = lds_frag(cB, brow + j * 32, chunk);
-}
-
-template <int D_DT, int BIAS_DT>
-__global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256_kernel(LinearArgs a) {
-  extern __shared__ __attribute__((aligned(16))) _Float16 lds[];  // [2 buffers][A tile | B tile]
-
-  const int64_t tiles_m = ceil_div(a.M, L_BM), tiles_n = ceil_div(a.N, L_BN);
-  const int64_t ntiles = tiles_m * tiles_n;
-  int64_t pid = blockIdx.x;
-  {  // contiguous run of tiles per XCD (workgroups are dealt round-robin to the 8 XCDs)
-    const int64_t per = ntiles / 8, rem = ntiles % 8;
-    const int64_t xcd = pid % 8, idx = pid / 8;
-    pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
-  }
-  constexpr int GROUP_M = 4;
-  const int64_t group = pid / (GROUP_M * tiles_n);
-  const int64_t first_m = group * GROUP_M;
-  const int64_t gsize = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
-  const int64_t tm = first_m + (pid % (GROUP_M * tiles_n)) % gsize;
-  const int64_t tn = (pid % (GROUP_M * tiles_n)) / gsize;
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  int64_t arow = tm * L_BM + tid, brow = tn * L_BN + tid;
-  arow = arow < a.M ? arow : a.M - 1;
-  brow = brow < a.N ? brow : a.N - 1;
-  const int nk = (int)(a.K / L_BK);
-  const int fa_row = wm * 128 + (lane & 31), fb_row = wn * 128 + (lane & 31), half = lane >> 5;
-
-  f32x16 acc[4][4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-
-  // Software pipeline.  Step kt multiplies LDS buffer kt&1 while it decodes the packed slice of
-  // step kt+1 (held in registers since the previous step) into the other buffer; the packed
-  // slices of steps kt+2 / kt+3 are in flight in the second register set.  The decode is done
-  // in sub-steps 0..2, the workgroup barrier sits before sub-step 3, and sub-step 3's MFMAs
-  // cover the barrier skew, the first fragment loads of step kt+1 and the next global loads.
-  PackedRow ra0 = load_row(a.A, a.A_sf, a.Mp, a.K, arow, 0);
-  PackedRow rb0 = load_row(a.B, a.B_sf, a.Np, a.K, brow, 0);
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    decode_row_quarter(lds, tid, q, ra0);
-    decode_row_quarter(lds + L_TILE_HALVES, tid, q, rb0);
-  }
-  const int klast = nk - 1;
-  ra0 = load_row(a.A, a.A_sf, a.Mp, a.K, arow, 1 < klast ? 1 : klast);
-  rb0 = load_row(a.B, a.B_sf, a.Np, a.K, brow, 1 < klast ? 1 : klast);
-  PackedRow ra1 = load_row(a.A, a.A_sf, a.Mp, a.K, arow, 2 < klast ? 2 : klast);
-  PackedRow rb1 = load_row(a.B, a.B_sf, a.Np, a.K, brow, 2 < klast ? 2 : klast);
-  __syncthreads();
-
-  Frags f[2];
-  load_frags(f[0], lds, lds + L_TILE_HALVES, fa_row, fb_row, half);
-
-  auto mfma16 = [&](const Frags &c) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(c.a[i], c.b[j], acc[i][j], 0, 0, 0);
-  };
-  // one K-step; da/db hold the packed slice of step kt+1 and are refilled with step kt+3
-  auto kstep = [&](int kt, PackedRow &da, PackedRow &db) {
-    const _Float16 *cA = lds + (kt & 1) * (2 * L_TILE_HALVES);
-    const _Float16 *cB = cA + L_TILE_HALVES;
-    _Float16 *nA = lds + ((kt + 1) & 1) * (2 * L_TILE_HALVES);
-    _Float16 *nB = nA + L_TILE_HALVES;
-    // sub-step 0
-    load_frags(f[1], cA, cB, fa_row, fb_row, 2 + half);
-    decode_row_quarter(nA, tid, 0, da);
-    decode_row_quarter(nA, tid, 1, da);
-    decode_row_quarter(nA, tid, 2, da);
-    mfma16(f[0]);
-#pragma unroll
-    for (int g = 0; g < 16; ++g) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-      if (g < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if (g >= 10) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    // sub-step 1
-    load_frags(f[0], cA, cB, fa_row, fb_row, 4 + half);
-    decode_row_quarter(nA, tid, 3, da);
-    decode_row_quarter(nB, tid, 0, db);
-    decode_row_quarter(nB, tid, 1, db);
-    mfma16(f[1]);
-#pragma unroll
-    for (int g = 0; g < 16; ++g) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-      if (g < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if (g >= 10) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    // sub-step 2
-    load_frags(f[1], cA, cB, fa_row, fb_row, 6 + half);
-    decode_row_quarter(nB, tid, 2, db);
-    decode_row_quarter(nB, tid, 3, db);
-    mfma16(f[0]);
-#pragma unroll
-    for (int g = 0; g < 16; ++g) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
-      if (g < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if (g >= 12) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    __syncthreads();  // buffer (kt+1)&1 is complete, buffer kt&1 has been read by everyone
-    // sub-step 3
-    load_frags(f[0], nA, nB, fa_row, fb_row, half);
-    const int kn = kt + 3 < klast ? kt + 3 : klast;
-    da = load_row(a.A, a.A_sf, a.Mp, a.K, arow, kn);
-    db = load_row(a.B, a.B_sf, a.Np, a.K, brow, kn);
-    mfma16(f[1]);
-#pragma unroll
-    for (int g = 0; g < 16; ++g) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-      if (g < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if (g >= 8 && g < 14) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  };
-  for (int kt = 0; kt < nk; ++kt) {
-    PackedRow na = ra1, nb = rb1;
-    kstep(kt, ra0, rb0);   // consumes ra0/rb0 (step kt+1), refills them with step kt+3
-    ra1 = ra0; rb1 = rb0;  // rotate: next step decodes the old ra1/rb1 (step kt+2)
-    ra0 = na; rb0 = nb;
-  }
-
-  const float scale = (*a.A_gs) * (*a.B_gs);
-  using DE = Elem<D_DT>;
-  typename DE::T *D = static_cast<typename DE::T *>(a.D);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int64_t n = tn * L_BN + wn * 128 + j * 32 + (lane & 31);
-    float bv = 0.0f;
-    if constexpr (BIAS_DT != BIAS_NONE) {
-      if (n < a.N) bv = Elem<BIAS_DT>::load(a.bias, n);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int64_t m = tm * L_BM + wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (m < a.M && n < a.N) {
-          float v = acc[i][j][e] * scale;
-          if constexpr (BIAS_DT != BIAS_NONE) v += bv;
-          D[m * a.N + n] = DE::cvt(v);
-        }
-      }
-    }
-  }
-}
-
-// ===========================================================================
-// 256x256x64 tile, 8 waves (2 x 4), each wave 128x64 = 4x2 MFMA tiles (128 accumulators).
-// Two waves share every SIMD, so one wave's decode VALU work, LDS stores and fragment loads
-// issue while the other wave's MFMAs run; a single wave per SIMD cannot overlap them because
-// it issues in order and an LDS store alone holds its issue port for ~32 cycles.
-// Thread t owns half a row (32 nibbles = two 16-blocks) of the A tile and of the B tile.
-// ===========================================================================
-struct PackedHalfRow {
-  uint4 d;      // 32 nibbles: two 16-blocks
-  uint32_t sf;  // scale dword of the row's 64-chunk (this thread uses two of its bytes)
-};
-
-__device__ __forceinline__ PackedHalfRow load_half_row(const uint8_t *base, const uint32_t *sf, int64_t rows_p,
-                                                       int64_t K, int64_t row, int half, int kt) {
-  PackedHalfRow r;
-  r.d = *reinterpret_cast<const uint4 *>(base + row * (K >> 1) + (int64_t)kt * 32 + half * 16);
-  r.sf = sf[(int64_t)kt * rows_p + row];
-  return r;
-}
-
-// block b (0/1) of a thread's half row -> its two 16-byte LDS chunks
-__device__ __forceinline__ void decode_half_block(_Float16 *tile, int row, int half, int b, const PackedHalfRow &r) {
-  const uint32_t w0 = b ? r.d.z : r.d.x, w1 = b ? r.d.w : r.d.y;
-  decode_block_to_lds(tile, row, half * 2 + b, w0, w1, r.sf);
-}
-
 
 // ===========================================================================
 // (64 MI) x (64 NJ) tile, packed operands in LDS, decode after the fragment load.
@@ -713,20 +485,8 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   constexpr int NS = (NSA + NSB + 3) / 4;  // scale transfers per wave (a remainder repeats the last one)
   constexpr int NPIECES = NDA + NDB + NS;
 
-  const int64_t tiles_m = ceil_div(a.M, BM), tiles_n = ceil_div(a.N, BN);
-  const int64_t ntiles = tiles_m * tiles_n;
-  int64_t pid = blockIdx.x;
-  {  // contiguous run of tiles per XCD (workgroups are dealt round-robin to the 8 XCDs)
-    const int64_t per = ntiles / 8, rem = ntiles % 8;
-    const int64_t xcd = pid % 8, idx = pid / 8;
-    pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
-  }
-  constexpr int GROUP_M = 4;
-  const int64_t group = pid / (GROUP_M * tiles_n);
-  const int64_t first_m = group * GROUP_M;
-  const int64_t gsize = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
-  const int64_t tm = first_m + (pid % (GROUP_M * tiles_n)) % gsize;
-  const int64_t tn = (pid % (GROUP_M * tiles_n)) / gsize;
+  const TileCoord tc = tile_of_workgroup<4>(blockIdx.x, ceil_div(a.M, BM), ceil_div(a.N, BN));
+  const int64_t tm = tc.m, tn = tc.n;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -752,19 +512,34 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     ra = tm * BM + ra < a.M ? ra : a.M - 1 - tm * BM;  // rows past the matrix read the last valid row
     offA[q] = (uint32_t)(ra * kb + dma_piece * 16);
   }
+  // weight image: a transfer's 16 rows are one contiguous kilobyte of a block (the swizzle is part of
+  // the image); bands past the last one read the last band, whose outputs are never stored
+  const int64_t w_band_bytes = (int64_t)nkt_all * W_BLOCK_BYTES, w_last_band = (a.N - 1) / W_BLOCK_ROWS;
+  auto w_band_of = [&](int64_t row, int64_t &within) {
+    int64_t band = row / W_BLOCK_ROWS;
+    within = row % W_BLOCK_ROWS;
+    return band < w_last_band ? band : w_last_band;
+  };
 #pragma unroll
   for (int q = 0; q < NDB; ++q) {
-    int64_t rb = (swave * NDB + q) * 16 + (lane >> 2);
-    rb = tn * BN + rb < a.N ? rb : a.N - 1 - tn * BN;
-    offB[q] = (uint32_t)(rb * kb + dma_piece * 16);
+    if (a.prepacked) {
+      int64_t within;
+      const int64_t band = w_band_of(tn * BN + (swave * NDB + q) * 16, within);
+      offB[q] = (uint32_t)(band * w_band_bytes + within * P_ROW + lane * 16);
+    } else {
+      int64_t rb = (swave * NDB + q) * 16 + (lane >> 2);
+      rb = tn * BN + rb < a.N ? rb : a.N - 1 - tn * BN;
+      offB[q] = (uint32_t)(rb * kb + dma_piece * 16);
+    }
   }
+  const int64_t strideB = a.prepacked ? W_BLOCK_BYTES : P_ROW;  // bytes per stage along k
   auto uniform_ptr = [](const void *p) {  // pin a wave-uniform pointer to scalar registers
     const uint64_t v = (uint64_t)p;
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
     return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
   };
   const uint8_t *baseA = uniform_ptr(a.A + tm * BM * kb + (int64_t)kt0 * P_ROW);
-  const uint8_t *baseB = uniform_ptr(a.B + tn * BN * kb + (int64_t)kt0 * P_ROW);
+  const uint8_t *baseB = uniform_ptr(a.prepacked ? a.B + (int64_t)kt0 * W_BLOCK_BYTES : a.B + tn * BN * kb + (int64_t)kt0 * P_ROW);
   // scale transfers: piece g = swave * NS + p (past the last piece: the last piece again, which
   // lands the same bytes in the same place).  g < NSA: operand A, chunk g / (BM/64), 64-row block
   // g % (BM/64); otherwise operand B, chunk (g-NSA) / (BN/64), block (g-NSA) % (BN/64).  Source
@@ -781,11 +556,19 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     const int gl = isB ? gq - NSA : gq, nb = isB ? BN / 64 : BM / 64;
     const int c = gl / nb, rb = gl % nb;
     const int64_t rows = isB ? a.Np : a.Mp;
-    int64_t sr = (isB ? tn * BN : tm * BM) + rb * 64 + lane;
-    sr = sr < rows ? sr : rows - 1;
-    offS[p2] = (uint32_t)sr * 4u;  // byte offset inside a scale plane
-    strideS[p2] = 2 * rows * 4;    // two planes (chunks) per stage
-    baseS[p2] = uniform_ptr((isB ? sfB8 : sfA8) + c * rows * 4 + kt0 * strideS[p2]);
+    if (isB && a.prepacked) {  // the scale dwords follow the packed rows of the block
+      int64_t within;
+      const int64_t band = w_band_of(tn * BN + rb * 64, within);
+      offS[p2] = (uint32_t)(band * w_band_bytes + W_BLOCK_DATA + c * (W_BLOCK_ROWS * 4) + (within + lane) * 4);
+      strideS[p2] = W_BLOCK_BYTES;
+      baseS[p2] = uniform_ptr(a.B + (int64_t)kt0 * W_BLOCK_BYTES);
+    } else {
+      int64_t sr = (isB ? tn * BN : tm * BM) + rb * 64 + lane;
+      sr = sr < rows ? sr : rows - 1;
+      offS[p2] = (uint32_t)sr * 4u;  // byte offset inside a scale plane
+      strideS[p2] = 2 * rows * 4;    // two planes (chunks) per stage
+      baseS[p2] = uniform_ptr((isB ? sfB8 : sfA8) + c * rows * 4 + kt0 * strideS[p2]);
+    }
     ldsS[p2] = (uint32_t)__builtin_amdgcn_readfirstlane((isB ? PL::OFF_SFB + c * BN * 4 : PL::OFF_SFA + c * BM * 4) + rb * 256);
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)plds;
@@ -804,7 +587,7 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
   auto src_at = [&](int kt) {
     Src p;
     p.a = baseA + (int64_t)kt * P_ROW;
-    p.b = baseB + (int64_t)kt * P_ROW;
+    p.b = baseB + (int64_t)kt * strideB;
 #pragma unroll
     for (int p2 = 0; p2 < NS; ++p2) p.s[p2] = baseS[p2] + kt * strideS[p2];
     return p;
@@ -975,7 +758,7 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     st_dma = ring_next(st_dma);
     const bool adv = kt + PS <= last;
     src.a += adv ? P_ROW : 0;
-    src.b += adv ? P_ROW : 0;
+    src.b += adv ? strideB : 0;
 #pragma unroll
     for (int p2 = 0; p2 < NS; ++p2) src.s[p2] += adv ? strideS[p2] : 0;
   }
@@ -1103,31 +886,6 @@ static int launch_tile256p(const LinearArgs &a, hipStream_t st) {
   return launch_tile_plan<D_DT, BIAS_DT>(a, tile_plan(a.M, a.N, a.K, false), one, st);
 }
 
-constexpr int L_LDS_BYTES = 2 * 2 * L_TILE_HALVES * (int)sizeof(_Float16);  // 128 KiB
-
-enum class LinearKernel { AUTO, TILE128, TILE256, TILE256P };
-
-static LinearKernel forced_kernel() {  // benchmarking aid: AC4K_LINEAR_KERNEL=tile128|tile256
-  static const LinearKernel k = [] {
-    const char *e = getenv("AC4K_LINEAR_KERNEL");
-    if (e && !strcmp(e, "tile128")) return LinearKernel::TILE128;
-    if (e && !strcmp(e, "tile256")) return LinearKernel::TILE256;
-    if (e && !strcmp(e, "tile256p")) return LinearKernel::TILE256P;
-    return LinearKernel::AUTO;
-  }();
-  return k;
-}
-
-template <int D_DT, int BIAS_DT>
-static int launch_tile256(const LinearArgs &a, hipStream_t st) {
-  auto *kern = linear_nvfp4_tile256_kernel<D_DT, BIAS_DT>;
-  static std::atomic<uint32_t> lds_ok{0};
-  if (int rc = allow_dynamic_lds(kern, lds_ok, L_LDS_BYTES)) return rc;
-  const int64_t ntiles = ceil_div(a.M, L_BM) * ceil_div(a.N, L_BN);
-  hipLaunchKernelGGL(kern, dim3((unsigned)ntiles), dim3(256), L_LDS_BYTES, st, a);
-  return 0;
-}
-
 // ===========================================================================
 // Decode-sized linear (1 <= M <= 32): bound by streaming the weights once.
 //
@@ -1156,6 +914,7 @@ struct SkinnyArgs {
   float *partial;      // [splitK][M][N]
   int64_t M, N, K, Np;
   int ks_len, split_k;
+  int prepacked = 0;  // B is a weight image (LDS-ring kernel only), B_sf unused
 };
 
 constexpr int SK_ROWS = 128;   // weight rows per workgroup
@@ -1393,7 +1152,7 @@ constexpr int ST_THREADS = 512;
 constexpr int ST_BK = 256;        // k per stage (four 64-chunks)
 constexpr int ST_ROW = ST_BK / 2; // packed bytes per row per stage
 constexpr int ST_PS = 6;
-constexpr int ST_NPIECES = 4;     // LDS-DMA instructions per wave per stage
+constexpr int ST_NPIECES = 4;     // LDS-DMA instructions per wave per stage (three from a weight image)
 constexpr int ST_OFF_B = 0;
 constexpr int ST_OFF_A = ST_OFF_B + ST_BN * ST_ROW;     // 32 packed activation rows
 constexpr int ST_OFF_SFB = ST_OFF_A + 32 * ST_ROW;      // weight scale dwords [chunk][128 rows]
@@ -1403,9 +1162,19 @@ constexpr int ST_LDS_BYTES = ST_PS * ST_STAGE_BYTES;
 static_assert(ST_LDS_BYTES <= 160 * 1024, "the ring must fit in the CU's LDS");
 static_assert((ST_PS - 3) * ST_NPIECES <= 63, "the wait counts must fit the 6-bit counter");
 static_assert(ST_LDS_BYTES >= 4 * 64 * 16 * 4, "the ring doubles as the exchange buffer of the two k halves");
+// From a weight image (PRE) a stage's weights and weight scales are ONE contiguous run of two blocks,
+// copied as it lies to the head of the LDS stage by 18 one-kilobyte transfers; with the four transfers
+// of the activation rows and the two of their scales that is three per wave.  The activation part of
+// the stage keeps its layout.
+constexpr int ST_PRE_W_BYTES = 2 * W_BLOCK_BYTES;  // 18432
+static_assert(ST_PRE_W_BYTES == ST_OFF_A + 4 * ST_BN * 4, "both layouts must give the same stage size");
+constexpr int ST_PRE_OFF_A = ST_PRE_W_BYTES, ST_PRE_OFF_SFA = ST_PRE_OFF_A + 32 * ST_ROW;
+constexpr int ST_PRE_NPIECES = 3;
 
-template <int D_DT, int BIAS_DT>
+template <int D_DT, int BIAS_DT, bool PRE>
 __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(SkinnyArgs a) {
+  constexpr int NPIECES = PRE ? ST_PRE_NPIECES : ST_NPIECES;
+  constexpr int OFF_A = PRE ? ST_PRE_OFF_A : ST_OFF_A, OFF_SFA = PRE ? ST_PRE_OFF_SFA : ST_OFF_SFA;
   extern __shared__ __attribute__((aligned(16))) char stlds[];
   const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, r32 = lane & 31;
   const int swave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1426,56 +1195,89 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
   // (one piece of each of 32 rows) over all LDS banks.  Unswizzled those reads fall on a quarter of the
   // banks and, issued by eight waves every stage, held the transfers back (40 us against 31 us on
   // N = 28672, K = 8192).
-  // --- this wave's four transfers of a stage: lane offsets (loop invariant), LDS destinations, sources
-  // (1, 2) weight rows swave * 16 + {0..7}, {8..15}, 128 B each
-  uint32_t offW[2];
+  // --- this wave's transfers of a stage: lane offsets (loop invariant), LDS destinations, sources
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)stlds;
+  // weights (and, from an image, their scales)
+  uint32_t offW[3];
+  const uint8_t *srcW;
+  int64_t strideW;
+  uint32_t ldsW;
+  if constexpr (PRE) {
+    // transfers 2 swave, 2 swave + 1 of the stage's 18 contiguous kilobytes; waves 0 and 1 also 16, 17
+    offW[0] = (uint32_t)(swave * 2048 + lane * 16);
+    offW[1] = offW[0] + 1024;
+    offW[2] = (uint32_t)((16 + swave) * 1024 + lane * 16);
+    strideW = ST_PRE_W_BYTES;
+    srcW = uniform_ptr(a.B + ((int64_t)blockIdx.x * (a.K / W_BLOCK_K) + 2 * (int64_t)s0) * W_BLOCK_BYTES);
+    ldsW = (uint32_t)__builtin_amdgcn_readfirstlane(swave * 2048);
+  } else {
+    // weight rows swave * 16 + {0..7}, {8..15}, 128 B each
 #pragma unroll
-  for (int q = 0; q < 2; ++q) {
-    const int loc = swave * 16 + q * 8 + (lane >> 3);
-    int64_t row = n0 + loc;
-    row = row < a.N ? row : a.N - 1;  // rows past N read the last row; their outputs are never stored
-    offW[q] = (uint32_t)((row - n0) * kb + ((lane & 7) ^ (loc & 7)) * 16);
+    for (int q = 0; q < 2; ++q) {
+      const int loc = swave * 16 + q * 8 + (lane >> 3);
+      int64_t row = n0 + loc;
+      row = row < a.N ? row : a.N - 1;  // rows past N read the last row; their outputs are never stored
+      offW[q] = (uint32_t)((row - n0) * kb + ((lane & 7) ^ (loc & 7)) * 16);
+    }
+    offW[2] = 0;
+    strideW = ST_ROW;
+    srcW = uniform_ptr(a.B + n0 * kb + (int64_t)s0 * ST_ROW);
+    ldsW = (uint32_t)__builtin_amdgcn_readfirstlane(ST_OFF_B + swave * 2048);
   }
-  const uint8_t *srcW = uniform_ptr(a.B + n0 * kb + (int64_t)s0 * ST_ROW);
-  const uint32_t ldsW = (uint32_t)__builtin_amdgcn_readfirstlane(ST_OFF_B + swave * 2048);
-  // (3) weight scales: chunk swave / 2, rows (swave % 2) * 64 + lane of the tile
-  int64_t srow = n0 + (swave & 1) * 64 + lane;
-  srow = srow < a.Np ? srow : a.Np - 1;
-  const uint32_t offS = (uint32_t)(srow * 4);
-  const int64_t strideS = 4 * a.Np * 4;  // bytes per stage (four chunk planes)
-  const uint8_t *srcS = uniform_ptr(reinterpret_cast<const uint8_t *>(a.B_sf) + (int64_t)(swave >> 1) * a.Np * 4 + s0 * strideS);
-  const uint32_t ldsS = (uint32_t)__builtin_amdgcn_readfirstlane(ST_OFF_SFB + (swave >> 1) * (ST_BN * 4) + (swave & 1) * 256);
-  // (4) waves 0..3: packed activation rows swave * 8 + {0..7}; waves 4, 5: activation scales of chunks
-  //     2 (swave - 4) + {0, 1}; waves 6, 7 repeat those of waves 4, 5 (every wave issues the same count)
-  uint32_t off4, lds4;
-  const uint8_t *src4;
-  int64_t stride4;
-  if (swave < 4) {
-    const int loc = swave * 8 + (lane >> 3);
+  // weight scales from the scale tensor: chunk swave / 2, rows (swave % 2) * 64 + lane of the tile
+  uint32_t offS = 0, ldsS = 0;
+  int64_t strideS = 0;
+  const uint8_t *srcS = nullptr;
+  if constexpr (!PRE) {
+    int64_t srow = n0 + (swave & 1) * 64 + lane;
+    srow = srow < a.Np ? srow : a.Np - 1;
+    offS = (uint32_t)(srow * 4);
+    strideS = 4 * a.Np * 4;  // bytes per stage (four chunk planes)
+    srcS = uniform_ptr(reinterpret_cast<const uint8_t *>(a.B_sf) + (int64_t)(swave >> 1) * a.Np * 4 + s0 * strideS);
+    ldsS = (uint32_t)__builtin_amdgcn_readfirstlane(ST_OFF_SFB + (swave >> 1) * (ST_BN * 4) + (swave & 1) * 256);
+  }
+  // activation: four waves take the packed rows w * 8 + {0..7}, two the scales of chunks 2 p + {0, 1};
+  // without an image waves 6 and 7 repeat the scale transfers (every wave issues the same count), with
+  // one waves 0 and 1 have their third weight transfer instead
+  constexpr int A_FIRST = PRE ? 2 : 0;  // first wave of the four that move the rows
+  const bool moves_rows = swave >= A_FIRST && swave < A_FIRST + 4;
+  uint32_t off4 = 0, lds4 = 0;
+  const uint8_t *src4 = nullptr;
+  int64_t stride4 = 0;
+  if (moves_rows) {
+    const int loc = (swave - A_FIRST) * 8 + (lane >> 3);
     const int64_t row = loc < a.M ? loc : a.M - 1;  // rows past M read row M - 1; their outputs are never stored
     off4 = (uint32_t)(row * kb + ((lane & 7) ^ (loc & 7)) * 16);
     stride4 = ST_ROW;
     src4 = uniform_ptr(a.Aq + (int64_t)s0 * ST_ROW);
-    lds4 = (uint32_t)__builtin_amdgcn_readfirstlane(ST_OFF_A + swave * 1024);
-  } else {
+    lds4 = (uint32_t)__builtin_amdgcn_readfirstlane(OFF_A + (swave - A_FIRST) * 1024);
+  } else if (!PRE || swave >= 6) {
     const int pair = swave & 1;  // chunks 2 pair, 2 pair + 1
     const int64_t row = r32 < a.Mp ? r32 : a.Mp - 1;
     off4 = (uint32_t)(((2 * pair + half) * a.Mp + row) * 4);
     stride4 = 4 * a.Mp * 4;
     src4 = uniform_ptr(a.A_sf + s0 * stride4);
-    lds4 = (uint32_t)__builtin_amdgcn_readfirstlane(ST_OFF_SFA + pair * 256);
+    lds4 = (uint32_t)__builtin_amdgcn_readfirstlane(OFF_SFA + pair * 256);
   }
-  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)stlds;
   auto issue_stage = [&](int slot, int st) {  // st: stage index inside this workgroup's range
     const uint32_t base = lds_base + slot * ST_STAGE_BYTES;
-    const uint8_t *pw = srcW + (int64_t)st * ST_ROW;
+    const uint8_t *pw = srcW + (int64_t)st * strideW;
     dma16(pw, offW[0], base, ldsW);
     dma16(pw, offW[1], base, ldsW + 1024);
-    dma4(srcS + st * strideS, offS, base, ldsS);
-    if (swave < 4)
-      dma16(src4 + st * stride4, off4, base, lds4);
-    else
-      dma4(src4 + st * stride4, off4, base, lds4);
+    if constexpr (PRE) {
+      if (swave < 2)
+        dma16(pw, offW[2], base, (uint32_t)__builtin_amdgcn_readfirstlane((16 + swave) * 1024));
+      else if (swave < 6)
+        dma16(src4 + st * stride4, off4, base, lds4);
+      else
+        dma4(src4 + st * stride4, off4, base, lds4);
+    } else {
+      dma4(srcS + st * strideS, offS, base, ldsS);
+      if (swave < 4)
+        dma16(src4 + st * stride4, off4, base, lds4);
+      else
+        dma4(src4 + st * stride4, off4, base, lds4);
+    }
   };
 
   // this wave's fragments of one stage: for each of its two 64-chunks (2 kh, 2 kh + 1) 32 packed
@@ -1490,11 +1292,16 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
 #pragma unroll
   for (int c = 0; c < 2; ++c) {
     const int piece = kh * 4 + c * 2 + half;
-    wf_off[c] = ST_OFF_B + wrow_l * ST_ROW + ((piece ^ (wrow_l & 7)) * 16);
-    xf_off[c] = ST_OFF_A + r32 * ST_ROW + ((piece ^ (r32 & 7)) * 16);
+    if constexpr (PRE)  // block kh of the stage; 64-byte rows, piece p of a chunk pair at p ^ ((r >> 1) & 3)
+      wf_off[c] = kh * W_BLOCK_BYTES + wrow_l * 64 + (((c * 2 + half) ^ ((wrow_l >> 1) & 3)) * 16);
+    else
+      wf_off[c] = ST_OFF_B + wrow_l * ST_ROW + ((piece ^ (wrow_l & 7)) * 16);
+    xf_off[c] = OFF_A + r32 * ST_ROW + ((piece ^ (r32 & 7)) * 16);
   }
-  const int ws_off = ST_OFF_SFB + (kh * 2) * (ST_BN * 4) + wrow_l * 4 + half * 2;
-  const int xs_off = ST_OFF_SFA + (kh * 2) * (32 * 4) + r32 * 4 + half * 2;
+  // scale planes of the wave's two chunks: `ws_pitch` bytes apart
+  constexpr int ws_pitch = PRE ? W_BLOCK_ROWS * 4 : ST_BN * 4;
+  const int ws_off = (PRE ? kh * W_BLOCK_BYTES + W_BLOCK_DATA : ST_OFF_SFB + (kh * 2) * (ST_BN * 4)) + wrow_l * 4 + half * 2;
+  const int xs_off = OFF_SFA + (kh * 2) * (32 * 4) + r32 * 4 + half * 2;
   auto load_frags = [&](int slot) {
     const char *st = stlds + slot * ST_STAGE_BYTES;
     StageFrags f;
@@ -1502,7 +1309,7 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
     for (int c = 0; c < 2; ++c) {
       f.w[c] = *reinterpret_cast<const uint4 *>(st + wf_off[c]);
       f.x[c] = *reinterpret_cast<const uint4 *>(st + xf_off[c]);
-      f.ws[c] = *reinterpret_cast<const uint16_t *>(st + ws_off + c * (ST_BN * 4));
+      f.ws[c] = *reinterpret_cast<const uint16_t *>(st + ws_off + c * ws_pitch);
       f.xs[c] = *reinterpret_cast<const uint16_t *>(st + xs_off + c * (32 * 4));
     }
     return f;
@@ -1519,7 +1326,7 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
   const int last = nst - 1;
 #pragma unroll
   for (int d = 0; d < ST_PS - 1; ++d) issue_stage(d, d < last ? d : last);
-  wait_vmcnt<(ST_PS - 3) * ST_NPIECES>();
+  wait_vmcnt<(ST_PS - 3) * NPIECES>();
   __syncthreads();
   StageFrags cur = load_frags(0);
 
@@ -1540,7 +1347,7 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
     // refill the slot of the stage before this one (everybody read it before the previous barrier)
     const int sd = s + ST_PS - 1;
     issue_stage(slot_dma, sd < last ? sd : last);
-    wait_vmcnt<(ST_PS - 3) * ST_NPIECES>();  // own transfers of stage s + 2 have landed
+    wait_vmcnt<(ST_PS - 3) * NPIECES>();  // own transfers of stage s + 2 have landed
     __syncthreads();
     cur = nxt;
     slot_next = slot_next + 1 == ST_PS ? 0 : slot_next + 1;
@@ -1677,8 +1484,13 @@ static int launch_skinny_it(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_
 
 template <int D_DT, int BIAS_DT>
 static int launch_skinny(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_t st) {
-  if (p.kind == DECODE_LDS_RING) {
-    auto *kern = linear_nvfp4_stream_kernel<D_DT, BIAS_DT>;
+  if (p.kind == DECODE_LDS_RING && a.prepacked) {
+    auto *kern = linear_nvfp4_stream_kernel<D_DT, BIAS_DT, true>;
+    static std::atomic<uint32_t> lds_ok{0};
+    if (int rc = allow_dynamic_lds(kern, lds_ok, ST_LDS_BYTES)) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)p.groups, (unsigned)p.split_k), dim3(ST_THREADS), ST_LDS_BYTES, st, a);
+  } else if (p.kind == DECODE_LDS_RING) {
+    auto *kern = linear_nvfp4_stream_kernel<D_DT, BIAS_DT, false>;
     static std::atomic<uint32_t> lds_ok{0};
     if (int rc = allow_dynamic_lds(kern, lds_ok, ST_LDS_BYTES)) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)p.groups, (unsigned)p.split_k), dim3(ST_THREADS), ST_LDS_BYTES, st, a);
@@ -1720,21 +1532,11 @@ static bool packed_kernel_ok(const LinearArgs &a) {
          a.N < (1ll << 27);
 }
 
+// M > 32 goes to the packed-operand tile kernel whenever its layout conditions hold; the
+// 128x128 kernel, which has no condition beyond K % 64 == 0, takes everything else.
 template <int D_DT, int BIAS_DT>
 static int launch_linear(const LinearArgs &a, hipStream_t st) {
-  LinearKernel k = forced_kernel();
-  const bool big_ok = a.K % L_BK == 0 && (((uintptr_t)a.A | (uintptr_t)a.B) & 15) == 0;
-  const bool packed_ok = packed_kernel_ok(a);
-  if (k == LinearKernel::AUTO) {
-    if (a.M > 32 && a.N >= 128 && packed_ok)
-      k = LinearKernel::TILE256P;
-    else if (a.M > 128 && a.N > 128 && big_ok)
-      k = LinearKernel::TILE256;
-    else
-      k = LinearKernel::TILE128;
-  }
-  if (k == LinearKernel::TILE256P && packed_ok) return launch_tile256p<D_DT, BIAS_DT>(a, st);
-  if (k == LinearKernel::TILE256 && big_ok) return launch_tile256<D_DT, BIAS_DT>(a, st);
+  if (a.M > 32 && a.N >= 128 && packed_kernel_ok(a)) return launch_tile256p<D_DT, BIAS_DT>(a, st);
   const int64_t ntiles = ceil_div(a.M, T_BM) * ceil_div(a.N, T_BN);
   hipLaunchKernelGGL((linear_nvfp4_tile128_kernel<D_DT, BIAS_DT>), dim3((unsigned)ntiles), dim3(256), 0, st, a);
   return 0;
@@ -1832,6 +1634,19 @@ static int dispatch_mid(const LinearArgs &a, const TilePlan &p, float *partial, 
     case AC4K_DTYPE_FP32: return dispatch_mid_bias<AC4K_DTYPE_FP32>(a, p, partial, bias_dtype, st);
   }
   return set_error("d must be bfloat16, half or float (dtype tag %d)", d_dtype);
+}
+
+// one K range of the tile kernel with a given plan (the entry point of the weight image)
+template <int D_DT>
+static int dispatch_prepacked_bias(const LinearArgs &a, const TilePlan &p, int bias_dtype, hipStream_t st) {
+  const SplitK one{nullptr, 1};
+  if (!a.bias) return launch_tile_plan<D_DT, BIAS_NONE>(a, p, one, st);
+  switch (bias_dtype) {
+    case AC4K_DTYPE_BF16: return launch_tile_plan<D_DT, AC4K_DTYPE_BF16>(a, p, one, st);
+    case AC4K_DTYPE_FP16: return launch_tile_plan<D_DT, AC4K_DTYPE_FP16>(a, p, one, st);
+    case AC4K_DTYPE_FP32: return launch_tile_plan<D_DT, AC4K_DTYPE_FP32>(a, p, one, st);
+  }
+  return set_error("bias must be bfloat16, half or float (dtype tag %d)", bias_dtype);
 }
 
 // shared tail of the two decode-sized entry points: packed activation in, partial sums in the workspace
@@ -1956,6 +1771,123 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_skinny_s
   // the partial sums are written before they are read: nothing in the array has to start at zero
   return linear_skinny_impl(D, d_dtype, A, A_sf, A_gs, B, B_sf, B_gs, bias, bias_dtype, M, N, K, ws,
                             STATIC_SCRATCH_BYTES, (hipStream_t)stream, "ac4k_linear_nvfp4_skinny_static");
+}
+
+namespace ac4k {
+
+// One workgroup writes one block of the weight image: 128 rows x 64 packed bytes (rows past N zero),
+// piece p of row r at position p ^ ((r >> 1) & 3), then the scale dwords [2 chunks][128 rows].
+__global__ __launch_bounds__(256) void prepack_weight_kernel(uint8_t *image, const uint8_t *B, const uint32_t *B_sf,
+                                                             int64_t N, int64_t K, int64_t Np) {
+  const int64_t kt = blockIdx.x, band = blockIdx.y;
+  uint8_t *blk = image + (band * gridDim.x + kt) * W_BLOCK_BYTES;
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int r = (t + i * 256) >> 2, pc = t & 3;
+    const int64_t row = band * W_BLOCK_ROWS + r;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (row < N) v = *reinterpret_cast<const uint4 *>(B + row * (K >> 1) + kt * (W_BLOCK_K / 2) + pc * 16);
+    *reinterpret_cast<uint4 *>(blk + r * (W_BLOCK_K / 2) + ((pc ^ ((r >> 1) & 3)) * 16)) = v;
+  }
+  const int c = t >> 7, r = t & 127;
+  const int64_t row = band * W_BLOCK_ROWS + r;
+  reinterpret_cast<uint32_t *>(blk + W_BLOCK_DATA)[c * W_BLOCK_ROWS + r] = row < N ? B_sf[(kt * 2 + c) * Np + row] : 0u;
+}
+
+static int64_t weight_image_bytes(int64_t N, int64_t K) {
+  if (N < 1 || K < W_BLOCK_K || K % W_BLOCK_K != 0) return 0;
+  return ceil_div(N, W_BLOCK_ROWS) * (K / W_BLOCK_K) * W_BLOCK_BYTES;
+}
+
+// How a linear on a weight image runs: the LDS-ring kernel for decode-sized M (K % 256 == 0), the tile
+// kernel otherwise, split along K when the workspace entry point of the plain layout would split too.
+struct PrepackedPlan {
+  bool ring;
+  SkinnyPlan sp;
+  TilePlan tp;
+  int64_t partial_bytes;
+};
+static bool prepacked_plan(int64_t M, int64_t N, int64_t K, PrepackedPlan &p) {
+  const int64_t bytes = weight_image_bytes(N, K);
+  if (M < 1 || bytes == 0 || bytes >= (1ll << 32) || (K >> 1) * 256 >= (1ll << 31) || N >= (1ll << 27)) return false;
+  p.ring = M <= 32 && K % ST_BK == 0;
+  if (p.ring) {
+    plan_lds_ring(M, N, K, p.sp);
+    p.partial_bytes = p.sp.partial_bytes;
+  } else {
+    p.tp = tile_plan(M, N, K, true);
+    p.partial_bytes = p.tp.partial_bytes;
+  }
+  return true;
+}
+
+}  // namespace ac4k
+
+extern "C" __attribute__((visibility("default"))) int64_t ac4k_prepack_weight_nvfp4_bytes(int64_t N, int64_t K) {
+  const int64_t bytes = weight_image_bytes(N, K);
+  return bytes < (1ll << 32) ? bytes : 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int ac4k_prepack_weight_nvfp4(void *image, const void *B, const void *B_sf, int64_t N, int64_t K,
+                                                                                ac4k_stream_t stream) {
+  AC4K_REQUIRE(image && B && B_sf, "null pointer argument");
+  const int64_t bytes = ac4k_prepack_weight_nvfp4_bytes(N, K);
+  AC4K_REQUIRE(bytes > 0, "no weight image for N = %lld, K = %lld: K must be a multiple of 128 and the image smaller than 4 GiB",
+               (long long)N, (long long)K);
+  AC4K_REQUIRE((((uintptr_t)image | (uintptr_t)B) & 15) == 0 && ((uintptr_t)B_sf & 3) == 0,
+               "image and B must be 16-byte aligned, B_sf 4-byte aligned");
+  hipLaunchKernelGGL(prepack_weight_kernel, dim3((unsigned)(K / W_BLOCK_K), (unsigned)ceil_div(N, W_BLOCK_ROWS)), dim3(256), 0,
+                     (hipStream_t)stream, static_cast<uint8_t *>(image), static_cast<const uint8_t *>(B),
+                     static_cast<const uint32_t *>(B_sf), N, K, align_up(N, 16));
+  return check_launch("ac4k_prepack_weight_nvfp4");
+}
+
+extern "C" __attribute__((visibility("default"))) int64_t ac4k_linear_nvfp4_prepacked_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  PrepackedPlan p;
+  return prepacked_plan(M, N, K, p) ? p.partial_bytes : 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_prepacked(void *D, int d_dtype, const void *A, const void *A_sf, const float *A_gs,
+                                                                                  const void *W_image, const float *B_gs, const void *bias,
+                                                                                  int bias_dtype, int64_t M, int64_t N, int64_t K, void *workspace,
+                                                                                  int64_t workspace_bytes, ac4k_stream_t stream) {
+  AC4K_REQUIRE(D && A && A_sf && A_gs && W_image && B_gs, "null pointer argument");
+  AC4K_REQUIRE(M >= 1 && N >= 1, "M and N must be positive (M = %lld, N = %lld)", (long long)M, (long long)N);
+  PrepackedPlan p;
+  AC4K_REQUIRE(prepacked_plan(M, N, K, p), "no weight image for N = %lld, K = %lld (ac4k_prepack_weight_nvfp4_bytes returns 0)",
+               (long long)N, (long long)K);
+  AC4K_REQUIRE((((uintptr_t)A | (uintptr_t)W_image) & 15) == 0 && ((uintptr_t)A_sf & 3) == 0,
+               "A and the weight image must be 16-byte aligned, A_sf 4-byte aligned");
+  AC4K_REQUIRE(ceil_div(M, 128) * ceil_div(N, 64) < (1ll << 31), "problem too large");
+  if (p.partial_bytes > 0) {
+    AC4K_REQUIRE(workspace && ((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
+    AC4K_REQUIRE(workspace_bytes >= p.partial_bytes, "workspace too small: %lld bytes needed", (long long)p.partial_bytes);
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (p.ring) {
+    SkinnyArgs a{D, static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(A_sf), align_up(M, 16),
+                 static_cast<const uint8_t *>(W_image), nullptr, A_gs, B_gs, bias, static_cast<float *>(workspace),
+                 M, N, K, align_up(N, 16), 0, p.sp.split_k, 1};
+    if (int rc = dispatch_skinny(a, p.sp, d_dtype, bias_dtype, st)) return rc;
+    return check_launch("ac4k_linear_nvfp4_prepacked");
+  }
+  LinearArgs la{D, static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(W_image),
+                static_cast<const uint32_t *>(A_sf), nullptr, A_gs, B_gs, bias,
+                M, N, K, align_up(M, 16), align_up(N, 16), 1};
+  int rc;
+  if (p.tp.splits > 1) {
+    rc = dispatch_mid(la, p.tp, static_cast<float *>(workspace), d_dtype, bias_dtype, st);
+  } else {
+    switch (d_dtype) {
+      case AC4K_DTYPE_BF16: rc = dispatch_prepacked_bias<AC4K_DTYPE_BF16>(la, p.tp, bias_dtype, st); break;
+      case AC4K_DTYPE_FP16: rc = dispatch_prepacked_bias<AC4K_DTYPE_FP16>(la, p.tp, bias_dtype, st); break;
+      case AC4K_DTYPE_FP32: rc = dispatch_prepacked_bias<AC4K_DTYPE_FP32>(la, p.tp, bias_dtype, st); break;
+      default: return set_error("d must be bfloat16, half or float (dtype tag %d)", d_dtype);
+    }
+  }
+  if (rc) return rc;
+  return check_launch("ac4k_linear_nvfp4_prepacked");
 }
 
 extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_fused_bf16(void *D, int d_dtype, const void *X, void *X_q, void *X_sf,

@@ -1,10 +1,10 @@
 """NVFP4-path operators with the names of the reference's ac4k_kernel.ops
 (python/ac4k_kernel/ops/__init__.py:5-26); the attention, RoPE and sparse-attention
 operators of the reference are not part of this library."""
-from .linear import fused_linear, linear, linear_nvfp4
+from .linear import fused_linear, linear, linear_nvfp4, linear_prepacked, prepack_weight
 from .quant import quantize, quantize_fp8, quantize_int8, quantize_nvfp4
 
 __all__ = [
-    "quantize", "linear", "fused_linear",
+    "quantize", "linear", "fused_linear", "prepack_weight", "linear_prepacked",
     "quantize_nvfp4", "quantize_fp8", "quantize_int8", "linear_nvfp4",
 ]

@@ -8,6 +8,7 @@ from .. import _rocm_ops
 from .utils import align_up
 
 linear_nvfp4 = _rocm_ops.linear_nvfp4
+prepack_weight = _rocm_ops.prepack_weight_nvfp4
 
 
 class Ac4kLinearOp(torch.nn.Module):
@@ -52,4 +53,20 @@ def fused_linear(x, weight, weight_scale, weight_global_scale, bias=None, out=No
     _rocm_ops.linear_nvfp4_fused(out, x, x_q, x_sf, x_gs, weight, weight_scale, weight_global_scale, bias)
     if return_quantized:
         return out, (x_q, x_sf, x_gs)
+    return out
+
+
+def linear_prepacked(x, x_scale, x_global_scale, weight_image, weight_global_scale, bias=None, out=None, n=None):
+    """`linear` on a weight image from `prepack_weight(weight, weight_scale)`: same result as
+    linear(x, x_scale, x_global_scale, weight, weight_scale, weight_global_scale, bias, out).  The image
+    does not carry N: pass `out` or `n`."""
+    if (bias is not None) and (bias.ndim == 1):
+        bias = bias.reshape(1, -1)
+    if out is None:
+        if n is None:
+            if bias is None:
+                raise RuntimeError("linear_prepacked needs out, n or bias to know N")
+            n = bias.shape[-1]
+        out = torch.empty((x.shape[0], n), dtype=torch.bfloat16, device=x.device)
+    _rocm_ops.linear_nvfp4_prepacked(out, x, x_scale, x_global_scale, weight_image, weight_global_scale, bias)
     return out

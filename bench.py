@@ -197,7 +197,8 @@ def linear_bytes(m, n, k):
     return (m + n) * k // 2 + ((m + 15) // 16 * 16 + (n + 15) // 16 * 16) * k // 16 + m * n * 2 + 8
 
 
-def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True, key=None, with_quantize=False, gen_on_gpu=False):
+def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True, key=None, with_quantize=False, gen_on_gpu=False,
+                 with_image=False):
     if gen_on_gpu:  # very large operands: the host generator would take longer than the measurement
         g = torch.Generator(device="cuda").manual_seed(0)
         a = torch.empty((m, k), dtype=torch.float32, device="cuda").normal_(generator=g).to(torch.bfloat16)
@@ -235,6 +236,20 @@ def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True, key=None, wi
         else:
             _, ms_with_quantize = time_gpu(lambda: ops.linear(*ops.quantize(xa, 0, 1), *weights(), out=out), steps, warmup)
         del xa
+    image = None
+    if with_image and k % 128 == 0:  # the same linear on pre-packed weight images of the same weights
+        imgs = [ops.prepack_weight(w[0], w[1]) for w in bqs]
+        out_i = torch.empty_like(out)
+        ops.linear_prepacked(*aq, imgs[0], bq[2], out=out_i)
+        ops.linear(*aq, *bq, out=out)
+        same = bool(torch.equal(out, out_i))
+        _, ms_i = time_gpu(lambda: (turn.__setitem__(0, turn[0] + 1),
+                                    ops.linear_prepacked(*aq, imgs[turn[0] % ncopy], bq[2], out=out_i)), steps, warmup)
+        _, ms_p = time_gpu(lambda: ops.linear(*aq, *weights(), out=out), steps, warmup)  # plain layout again, after it
+        image = {"ms": ms_i, "plain_layout_ms_before": ms, "plain_layout_ms_after": ms_p,
+                 "bit_identical_to_plain_layout": same,
+                 "TFLOP/s": 2.0 * m * n * k / (ms_i * 1e-3) / 1e12, "GB/s": linear_bytes(m, n, k) / (ms_i * 1e-3) / 1e9}
+        del imgs, out_i
     del bqs
     tflops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
     gbs = linear_bytes(m, n, k) / (ms * 1e-3) / 1e9
@@ -242,7 +257,8 @@ def bench_linear(ops, m, n, k, steps, warmup, wstd=1.0, check=True, key=None, wi
     rl = roofline("mfma", tflops, key) if t_flops >= t_bytes else roofline("hbm", gbs, key)
     return {"workload": f"NVFP4 linear M={m} N={n} K={k}, bf16 out, operands pre-quantized", "ms": ms,
             "total_ms": total, "TFLOP/s": tflops, "GB/s": gbs, "within_1e-2_of_fp32_dequant_matmul": ok,
-            "roofline": rl, "ms_with_activation_quantize": ms_with_quantize, "rotating_weight_copies": ncopy}
+            "roofline": rl, "ms_with_activation_quantize": ms_with_quantize, "rotating_weight_copies": ncopy,
+            "weight_image": image}
 
 
 def _read_sclk_mhz():
@@ -319,7 +335,7 @@ def vendor_gemm_yardstick(steps, warmup, n=8192):
     return res
 
 
-def bench_decode(ops, m, n, k, steps, warmup, check=True, ncopy=3):
+def bench_decode(ops, m, n, k, steps, warmup, check=True, ncopy=3, key=None):
     """Fused decode-sized linear: bf16 activation in, on-the-fly NVFP4 quantize + GEMM.  The calls
     rotate over `ncopy` copies of the weights (3 x 132 MB: more than the 256 MB memory-side cache holds),
     so that the weights are streamed from HBM."""
@@ -343,7 +359,7 @@ def bench_decode(ops, m, n, k, steps, warmup, check=True, ncopy=3):
     gbs = nbytes / (ms * 1e-3) / 1e9
     return {"workload": f"fused decode linear M={m} N={n} K={k} (bf16 activation quantized on the fly)", "ms": ms,
             "bytes": nbytes, "GB/s": gbs, "equals_quantize_then_linear_within_1e-2": ok,
-            "roofline": roofline("hbm", gbs), "rotating_weight_copies": ncopy}
+            "roofline": roofline("hbm", gbs, key), "rotating_weight_copies": ncopy}
 
 
 def bench_quantize_layouts(ops, steps, warmup):
@@ -417,6 +433,24 @@ def run_traffic(ops):
     out = torch.empty((8192, 8192), dtype=torch.bfloat16, device="cuda")
     for _ in range(3):
         ops.linear(*aq, *bq, out=out)
+    img = ops.prepack_weight(bq[0], bq[1])
+    for _ in range(3):
+        ops.linear_prepacked(*aq, img, bq[2], out=out)
+    del aq, bq, out, img, a
+    # decode-sized kernels: configuration 5 at M = 1 / 8 / 32 and configuration 4 at M = 16, linear alone
+    # (activation already quantized), then the same on weight images; the kernels are told apart by
+    # their names and grids in the counter output
+    for (n, k, ms_) in ((28672, 8192, (1, 8, 32)), (14336, 4096, (16,))):
+        wq = ops.quantize(make_input((n, k), seed=3, std=0.02).cuda(), 0, 1)
+        wimg = ops.prepack_weight(wq[0], wq[1])
+        for m in ms_:
+            xq = ops.quantize(make_input((m, k), seed=2).cuda(), 0, 1)
+            o = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+            for _ in range(3):
+                ops.linear(*xq, *wq, out=o)
+            for _ in range(3):
+                ops.linear_prepacked(*xq, wimg, wq[2], out=o)
+        del wq, wimg
     x = make_input((8192, 4096), seed=0, outliers=True).cuda()
     for prec in ("nvfp4", "fp8e4m3", "int8"):
         for _ in range(3):
@@ -525,9 +559,16 @@ def main():
             log(f"[bench] cpu quantize oracle: {quant['cpu_baseline']['value']:.2f} GB/s on "
                 f"{quant['cpu_baseline']['cores']} threads")
     if args.workload in ("all", "linear"):
-        lin = bench_linear(ops, 8192, 8192, 8192, S, W, check=check, key="linear_8192")
+        lin = bench_linear(ops, 8192, 8192, 8192, S, W, check=check, key="linear_8192", with_image=True)
         log(f"[bench] {lin['workload']}: {lin['ms']:.3f} ms  {lin['TFLOP/s']:.1f} TFLOP/s "
             f"({100 * lin['roofline']['frac']:.1f}% of MFMA peak)  ok={lin['within_1e-2_of_fp32_dequant_matmul']}")
+        wi = lin["weight_image"]
+        log(f"[bench]   same linear on a pre-packed weight image: {wi['ms']:.3f} ms  {wi['TFLOP/s']:.1f} TFLOP/s "
+            f"({100 * wi['TFLOP/s'] / MFMA_PEAK_TFLOPS:.1f}% of MFMA peak; plain layout re-timed after it: "
+            f"{wi['plain_layout_ms_after']:.3f} ms)  bit-identical={wi['bit_identical_to_plain_layout']}")
+        line["linear_8192_weight_image_tflops"] = wi["TFLOP/s"]
+        line["linear_8192_weight_image_frac"] = wi["TFLOP/s"] / MFMA_PEAK_TFLOPS
+        line["linear_8192_weight_image_bit_identical"] = wi["bit_identical_to_plain_layout"]
         line.update({"metric": "nvfp4_linear_tflops", "value": lin["TFLOP/s"], "unit": "TFLOP/s",
                      "ms_per_step": lin["ms"], "dtype": "fp4 x e4m3 decoded exactly to fp16, fp32 accumulate",
                      "config": {"workload": lin["workload"]}, "roofline": lin["roofline"],
@@ -549,19 +590,26 @@ def main():
             log(f"[bench] yardstick, torch.matmul 8192^3 on already dense operands: "
                 f"{line['vendor_dense_gemm']['bf16_TFLOP/s']:.0f} TFLOP/s bf16, "
                 f"{line['vendor_dense_gemm']['fp16_TFLOP/s']:.0f} TFLOP/s fp16")
-            shapes = {"cfg3_4096": bench_linear(ops, 4096, 4096, 4096, S, W, check=check)}
+            shapes = {"cfg3_4096": bench_linear(ops, 4096, 4096, 4096, S, W, check=check, with_image=True)}
             for (n, k) in ((14336, 4096), (4096, 14336)):
                 for m in (16, 128, 2048, 8192):
                     shapes[f"cfg4_M{m}_N{n}_K{k}"] = bench_linear(ops, m, n, k, S, W, wstd=0.02, check=check,
-                                                                  with_quantize=True)
+                                                                  with_quantize=True, with_image=True,
+                                                                  key=f"decode_linear_M{m}_N{n}_K{k}" if m <= 32 else None)
+            for m in (1, 8, 32):  # configuration 5 with the activation already quantized (linear alone)
+                shapes[f"cfg5_M{m}_linear_alone"] = bench_linear(ops, m, 28672, 8192, S, W, wstd=0.02, check=check,
+                                                                 with_image=True, key=f"decode_linear_M{m}")
             for k_, v in shapes.items():
                 wq_ = v["ms_with_activation_quantize"]
                 log(f"[bench] {k_}: {v['ms'] * 1e3:.1f} us  {v['TFLOP/s']:.1f} TFLOP/s  {v['GB/s']:.0f} GB/s  "
                     f"{100 * v['roofline']['frac']:.1f}% of {v['roofline']['bound']} peak  "
                     f"ok={v['within_1e-2_of_fp32_dequant_matmul']}"
-                    + ("" if wq_ is None else f"  with activation quantize {wq_ * 1e3:.1f} us"))
+                    + ("" if wq_ is None else f"  with activation quantize {wq_ * 1e3:.1f} us")
+                    + ("" if v["weight_image"] is None else
+                       f"  on a weight image {v['weight_image']['ms'] * 1e3:.1f} us "
+                       f"(bit-identical={v['weight_image']['bit_identical_to_plain_layout']})"))
             line["linear_shapes"] = shapes
-            dec = {f"cfg5_M{m}": bench_decode(ops, m, 28672, 8192, S, W, check) for m in (1, 8, 32)}
+            dec = {f"cfg5_M{m}": bench_decode(ops, m, 28672, 8192, S, W, check, key=f"decode_fused_M{m}") for m in (1, 8, 32)}
             for k_, v in dec.items():
                 log(f"[bench] {k_}: {v['ms'] * 1e3:.1f} us  {v['GB/s']:.0f} GB/s "
                     f"({100 * v['roofline']['frac']:.1f}% of HBM peak)  ok={v['equals_quantize_then_linear_within_1e-2']}")
@@ -625,6 +673,14 @@ def main():
         if k_ in line:
             summary.append(k_ + ": " + "  ".join(f"{n_.split('_', 1)[1]} {v['ms'] * 1e3:.1f}us/{v['roofline']['frac']:.2f}"
                                                  for n_, v in line[k_].items()))
+    if "linear_shapes" in line:
+        summary.append("weight image / plain layout, us: " + "  ".join(
+            f"{n_.split('_', 1)[1]} {v['weight_image']['ms'] * 1e3:.1f}/{v['ms'] * 1e3:.1f}"
+            for n_, v in line["linear_shapes"].items() if v.get("weight_image")))
+    if "linear_8192_weight_image_tflops" in line:
+        summary.append(f"linear 8192^3 on a weight image: {line['linear_8192_weight_image_tflops']:.1f} TFLOP/s  "
+                       f"frac {line['linear_8192_weight_image_frac']:.3f}  "
+                       f"bit_identical={line['linear_8192_weight_image_bit_identical']}")
     if "ref_shapes" in line:
         summary.append("ref shapes: " + "  ".join(f"{n_} {v['TFLOP/s']:.0f}TF/{v['roofline']['frac']:.2f}"
                                                   for n_, v in line["ref_shapes"].items()))

@@ -156,6 +156,34 @@ int ac4k_linear_nvfp4_skinny_static(void *D, int d_dtype, const void *A, const v
  * Process-wide; returns non-zero on values outside these sets. */
 int ac4k_set_linear_tuning(int mi, int nj, int splits, int skinny_ks, int decode_kernel);
 
+/* Pre-packed weight image.  No counterpart in the reference, which fetches the weights in their
+ * tensor layout on every call (lib/cuda/sm120/linear_nvfp4.cu:586-633); it would sit beside
+ * ac4k::linear_nvfp4 (lib/cuda/sm120/linear_nvfp4.cu:753-901).  Static weights are re-laid ONCE into
+ * the order the kernels fetch them, and the linear then reads the image instead of B and B_sf.
+ * The arithmetic is untouched: same nibbles, same scale bytes, same order of accumulation, so the
+ * output is bit-identical to the entry point of the plain layout that runs the same kernel
+ * (ac4k_linear_nvfp4, or ac4k_linear_nvfp4_skinny for the shapes it splits along K or streams
+ * through the LDS ring).
+ * Image: one block of 9216 bytes per (128 rows, 128 k), blocks of a 128-row band consecutive along
+ * k, bands consecutive along n, N padded with zero rows to a whole band.  A block holds 128 rows x
+ * 64 packed bytes, the 16-byte piece p of row r at position p ^ ((r >> 1) & 3) of its row, then the
+ * scale dwords of the block's two 64-chunks, [2][128 rows].
+ * ac4k_prepack_weight_nvfp4_bytes: size of the image, 0 when there is none (K % 128 != 0, or an
+ * image of 4 GiB and more).  ac4k_prepack_weight_nvfp4: B [N,K/2], B_sf [K/64,align_up(N,16),4] ->
+ * image (16-byte aligned).
+ * ac4k_linear_nvfp4_prepacked: contract of ac4k_linear_nvfp4 with W_image in place of B and B_sf;
+ * `workspace` as for ac4k_linear_nvfp4_skinny, of ac4k_linear_nvfp4_prepacked_workspace_bytes(M,N,K)
+ * bytes (may be NULL when that is 0).  M <= 32 with K % 256 == 0 streams the image through the LDS
+ * ring; everything else runs the tile kernel, split along K when there are too few tiles. */
+int64_t ac4k_prepack_weight_nvfp4_bytes(int64_t N, int64_t K);
+int ac4k_prepack_weight_nvfp4(void *image, const void *B, const void *B_sf, int64_t N, int64_t K,
+                              ac4k_stream_t stream);
+int64_t ac4k_linear_nvfp4_prepacked_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int ac4k_linear_nvfp4_prepacked(void *D, int d_dtype, const void *A, const void *A_sf,
+                                const float *A_gs, const void *W_image, const float *B_gs,
+                                const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K,
+                                void *workspace, int64_t workspace_bytes, ac4k_stream_t stream);
+
 /* Fused decode-sized linear: quantize(X,0,1) followed by linear(...) in one call.  No single
  * reference function: it equals the composition the reference's tests make
  * (test/test_linear_bench.py:128-137) — the activation bytes, scales and global scale it
