@@ -123,4 +123,52 @@ __device__ __forceinline__ uint32_t f32x8_to_e2m1x8(const float (&f)[8]) {
   return r;
 }
 
+// ---------------------------------------------------------------------------
+// nvfp4 block arithmetic shared by the quantizers and the linear kernel that quantizes its activation
+// ---------------------------------------------------------------------------
+// Correctly rounded fp32 reciprocals of the 128 non-negative E4M3 codes (entry 0 is 0, entry
+// 0x7F is NaN): the block scale takes one of these values, so the IEEE division of the spec
+// (about a dozen VALU instructions) becomes one LDS read.  The table is folded at compile time
+// (constant folding of `/` is correctly rounded).
+struct RcpE4M3Table {
+  float v[128];
+  constexpr RcpE4M3Table() : v() {
+    for (int c = 0; c < 128; ++c) {
+      const int e = c >> 3, m = c & 7;
+      float val = 0.0f;
+      if (e == 0) {
+        val = (float)m * 0.001953125f;  // m * 2^-9
+      } else {
+        val = 1.0f + (float)m * 0.125f;
+        for (int i = 7; i < e; ++i) val *= 2.0f;
+        for (int i = e; i < 7; ++i) val *= 0.5f;
+      }
+      v[c] = c == 0 ? 0.0f : (c == 127 ? __builtin_nanf("") : 1.0f / val);
+    }
+  }
+};
+static __constant__ RcpE4M3Table g_rcp_e4m3;  // one copy per translation unit
+
+// Fills the block's LDS copy of the table (every thread must call it; ends with a barrier).
+__device__ __forceinline__ void load_rcp_table(float *lut) {
+  if (threadIdx.x < 128) lut[threadIdx.x] = g_rcp_e4m3.v[threadIdx.x];
+  __syncthreads();
+}
+
+// Scale of one 16-block.  Returns the multiplier alpha * (1 / fp32(sf)) and the e4m3 code.
+// With code 0 the table gives 0 (alpha is finite then: alpha = inf makes every code 0x7E/0x7F).
+__device__ __forceinline__ float nvfp4_block_scale(float amax, float alpha, const float *lut, uint32_t &code) {
+  float s32 = alpha * (amax * 0.16666666666666666f);
+  code = f32_to_ue4m3_satfinite(s32);
+  return alpha * lut[code];
+}
+
+__device__ __forceinline__ uint32_t nvfp4_pack8(uint4 v, float o) {
+  float f[8] = {bf16_lo(v.x) * o, bf16_hi(v.x) * o, bf16_lo(v.y) * o, bf16_hi(v.y) * o,
+                bf16_lo(v.z) * o, bf16_hi(v.z) * o, bf16_lo(v.w) * o, bf16_hi(v.w) * o};
+  // A NaN multiplier (global scale 0: inf * 0) makes every product NaN; cvt.satfinite maps NaN
+  // to +6 whatever its sign, the gfx950 converter keeps the sign, so this case is spelled out.
+  return (o != o) ? 0x77777777u : f32x8_to_e2m1x8(f);
+}
+
 }  // namespace ac4k

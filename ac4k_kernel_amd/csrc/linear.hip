@@ -1171,6 +1171,81 @@ static_assert(ST_PRE_W_BYTES == ST_OFF_A + 4 * ST_BN * 4, "both layouts must giv
 constexpr int ST_PRE_OFF_A = ST_PRE_W_BYTES, ST_PRE_OFF_SFA = ST_PRE_OFF_A + 32 * ST_ROW;
 constexpr int ST_PRE_NPIECES = 3;
 
+// a wave's fragments of one stage: for each of its two 64-chunks (2 kh, 2 kh + 1) 32 packed elements
+// of a weight row and of an activation row (the lane's half of the chunk) and the two block scales of each
+struct StageFrags {
+  uint4 w[2], x[2];
+  uint32_t ws[2], xs[2];
+};
+
+// acc[c] += W . Xhat^T over the wave's two chunks of a stage (decode in registers)
+__device__ __forceinline__ void stream_multiply(const StageFrags &cur, f32x16 (&acc)[2]) {
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const f16x2 wsc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(cur.ws[c], 1.0f, false);
+    const f16x2 xsc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(cur.xs[c], 1.0f, false);
+    acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<false>(cur.w[c].x, wsc), decode_dword<false>(cur.x[c].x, xsc), acc[c], 0, 0, 0);
+    acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<false>(cur.w[c].y, wsc), decode_dword<false>(cur.x[c].y, xsc), acc[c], 0, 0, 0);
+    acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<true>(cur.w[c].z, wsc), decode_dword<true>(cur.x[c].z, xsc), acc[c], 0, 0, 0);
+    acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<true>(cur.w[c].w, wsc), decode_dword<true>(cur.x[c].w, xsc), acc[c], 0, 0, 0);
+  }
+}
+
+// End of the LDS-ring kernels, after the last LDS-DMA has landed and every wave has passed a barrier:
+// the two chunk sums of a wave, then the two k halves (through `xch_base`, always in this order), then
+// either the fp32 partial sums of this K range or the finished outputs (times gsA * gsB, plus bias).
+template <int D_DT, int BIAS_DT>
+__device__ __forceinline__ void stream_finish(f32x16 (&acc)[2], const SkinnyArgs &a, char *xch_base, float gs_a, int wn, int kh,
+                                              int lane, int64_t n0) {
+  const int half = lane >> 5, r32 = lane & 31;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[0][e] += acc[1][e];
+  float4 *xch = reinterpret_cast<float4 *>(xch_base) + (wn * 64 + lane) * 4;
+  if (kh == 1) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) xch[g] = make_float4(acc[0][4 * g], acc[0][4 * g + 1], acc[0][4 * g + 2], acc[0][4 * g + 3]);
+  }
+  __syncthreads();
+  if (kh == 1) return;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const float4 o = xch[g];
+    acc[0][4 * g] += o.x; acc[0][4 * g + 1] += o.y; acc[0][4 * g + 2] += o.z; acc[0][4 * g + 3] += o.w;
+  }
+
+  // acc: lane <-> m = r32, element e <-> n = (e >> 2) * 8 + half * 4 + (e & 3): four consecutive n per group
+  const int m = r32;
+  if (m >= (int)a.M) return;
+  const int64_t nw = n0 + wn * 32;
+  if (a.split_k > 1) {
+    float *pp = a.partial + ((int64_t)blockIdx.y * a.M + m) * a.N;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int64_t n = nw + g * 8 + half * 4;
+      if (n + 3 < a.N && (a.N & 3) == 0) {
+        *reinterpret_cast<float4 *>(pp + n) = make_float4(acc[0][4 * g], acc[0][4 * g + 1], acc[0][4 * g + 2], acc[0][4 * g + 3]);
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (n + q < a.N) pp[n + q] = acc[0][4 * g + q];
+      }
+    }
+    return;
+  }
+  using DE = Elem<D_DT>;
+  typename DE::T *Dp = static_cast<typename DE::T *>(a.D);
+  const float scale = gs_a * (*a.B_gs);
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int64_t n = nw + (e >> 2) * 8 + half * 4 + (e & 3);
+    if (n < a.N) {
+      float v = acc[0][e] * scale;
+      if constexpr (BIAS_DT != BIAS_NONE) v += Elem<BIAS_DT>::load(a.bias, n);
+      Dp[(int64_t)m * a.N + n] = DE::cvt(v);
+    }
+  }
+}
+
 template <int D_DT, int BIAS_DT, bool PRE>
 __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(SkinnyArgs a) {
   constexpr int NPIECES = PRE ? ST_PRE_NPIECES : ST_NPIECES;
@@ -1184,6 +1259,14 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
   const int s0 = (int)((int64_t)nst_all * blockIdx.y / a.split_k);
   const int nst = (int)((int64_t)nst_all * (blockIdx.y + 1) / a.split_k) - s0;  // >= 1: split_k <= stages
   const int64_t kb = a.K >> 1;
+  // Workgroup b walks its stages starting at stage b % nst and wraps around.  In step, every workgroup
+  // would ask for the same 128-byte column of its rows at the same time; with a row pitch that is a
+  // power of two (K = 8192: 4096 bytes) all those addresses fall on the same few memory channels.
+  const int rot = (int)(blockIdx.x % (unsigned)nst);
+  auto stage_of = [&](int step) {
+    const int p = step + rot;
+    return p >= nst ? p - nst : p;
+  };
 
   auto uniform_ptr = [](const void *p) {  // pin a wave-uniform pointer to scalar registers
     const uint64_t v = (uint64_t)p;
@@ -1259,7 +1342,8 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
     src4 = uniform_ptr(a.A_sf + s0 * stride4);
     lds4 = (uint32_t)__builtin_amdgcn_readfirstlane(OFF_SFA + pair * 256);
   }
-  auto issue_stage = [&](int slot, int st) {  // st: stage index inside this workgroup's range
+  auto issue_stage = [&](int slot, int step) {  // step: position in this workgroup's order of stages
+    const int st = stage_of(step);
     const uint32_t base = lds_base + slot * ST_STAGE_BYTES;
     const uint8_t *pw = srcW + (int64_t)st * strideW;
     dma16(pw, offW[0], base, ldsW);
@@ -1280,13 +1364,6 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
     }
   };
 
-  // this wave's fragments of one stage: for each of its two 64-chunks (2 kh, 2 kh + 1) 32 packed
-  // elements of a weight row and of an activation row (the lane's half of the chunk) and the two block
-  // scales of each
-  struct StageFrags {
-    uint4 w[2], x[2];
-    uint32_t ws[2], xs[2];
-  };
   const int wrow_l = wn * 32 + r32;
   int wf_off[2], xf_off[2];
 #pragma unroll
@@ -1335,15 +1412,7 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
     // fragments of the next stage (it landed before the previous barrier) travel from LDS while this
     // stage is decoded and multiplied (past the range: a stage nobody uses)
     const StageFrags nxt = load_frags(slot_next);
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      const f16x2 wsc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(cur.ws[c], 1.0f, false);
-      const f16x2 xsc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(cur.xs[c], 1.0f, false);
-      acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<false>(cur.w[c].x, wsc), decode_dword<false>(cur.x[c].x, xsc), acc[c], 0, 0, 0);
-      acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<false>(cur.w[c].y, wsc), decode_dword<false>(cur.x[c].y, xsc), acc[c], 0, 0, 0);
-      acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<true>(cur.w[c].z, wsc), decode_dword<true>(cur.x[c].z, xsc), acc[c], 0, 0, 0);
-      acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<true>(cur.w[c].w, wsc), decode_dword<true>(cur.x[c].w, xsc), acc[c], 0, 0, 0);
-    }
+    stream_multiply(cur, acc);
     // refill the slot of the stage before this one (everybody read it before the previous barrier)
     const int sd = s + ST_PS - 1;
     issue_stage(slot_dma, sd < last ? sd : last);
@@ -1355,53 +1424,7 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-DMA may land after this point: the ring is reused
   __syncthreads();
-#pragma unroll
-  for (int e = 0; e < 16; ++e) acc[0][e] += acc[1][e];
-  // the sums of the upper k half join those of the lower one (always in this order)
-  float4 *xch = reinterpret_cast<float4 *>(stlds) + (wn * 64 + lane) * 4;
-  if (kh == 1) {
-#pragma unroll
-    for (int g = 0; g < 4; ++g) xch[g] = make_float4(acc[0][4 * g], acc[0][4 * g + 1], acc[0][4 * g + 2], acc[0][4 * g + 3]);
-  }
-  __syncthreads();
-  if (kh == 1) return;
-#pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const float4 o = xch[g];
-    acc[0][4 * g] += o.x; acc[0][4 * g + 1] += o.y; acc[0][4 * g + 2] += o.z; acc[0][4 * g + 3] += o.w;
-  }
-
-  // acc: lane <-> m = r32, element e <-> n = (e >> 2) * 8 + half * 4 + (e & 3): four consecutive n per group
-  const int m = r32;
-  if (m >= (int)a.M) return;
-  const int64_t nw = n0 + wn * 32;
-  if (a.split_k > 1) {
-    float *pp = a.partial + ((int64_t)blockIdx.y * a.M + m) * a.N;
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int64_t n = nw + g * 8 + half * 4;
-      if (n + 3 < a.N && (a.N & 3) == 0) {
-        *reinterpret_cast<float4 *>(pp + n) = make_float4(acc[0][4 * g], acc[0][4 * g + 1], acc[0][4 * g + 2], acc[0][4 * g + 3]);
-      } else {
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-          if (n + q < a.N) pp[n + q] = acc[0][4 * g + q];
-      }
-    }
-    return;
-  }
-  using DE = Elem<D_DT>;
-  typename DE::T *Dp = static_cast<typename DE::T *>(a.D);
-  const float scale = (*a.A_gs) * (*a.B_gs);
-#pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const int64_t n = nw + (e >> 2) * 8 + half * 4 + (e & 3);
-    if (n < a.N) {
-      float v = acc[0][e] * scale;
-      if constexpr (BIAS_DT != BIAS_NONE) v += Elem<BIAS_DT>::load(a.bias, n);
-      Dp[(int64_t)m * a.N + n] = DE::cvt(v);
-    }
-  }
+  stream_finish<D_DT, BIAS_DT>(acc, a, stlds, *a.A_gs, wn, kh, lane, n0);
 }
 
 // Plan of a decode-sized linear: which of the two kernels, its K split and the fp32 scratch it needs.
@@ -1453,19 +1476,21 @@ static void plan_lds_ring(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
   p.lds_bytes = ST_LDS_BYTES;
 }
 
-// Shapes of the decode-sized kernels (both need K % 256 == 0) and the choice between them: the
-// register kernel streams a little faster at small M (all its loads are in flight at once, four
-// workgroups per CU) but pays for partial sums and a second launch, and its registers run out as M
-// grows; the LDS-ring kernel takes nearly the same time for every M <= 32 and needs no second launch
-// when N alone fills the GPU.  Measured, linear alone, register / LDS-ring kernel in us:
-//   N = 28672, K = 8192:  M = 1 30.9 / 34.0, M = 8 34.7 / 34.5, M = 12 37.2 / 35.9, M = 16 41.0 / 37.0, M = 32 45.2 / 37.9
-//   N = 14336, K = 4096:  M = 8 14.3 / 16.2, M = 12 16.1 / 16.2, M = 16 17.0 / 16.2, M = 32 21.8 / 16.8
-//   N = 4096, K = 14336:  M = 8 16.2 / 17.3, M = 12 17.2 / 17.5, M = 16 18.2 / 17.4, M = 32 22.2 / 17.9
+// Shapes of the decode-sized kernels (both need K % 256 == 0) and the choice between them.  The
+// register kernel has all its loads in flight at once and four workgroups per CU, which wins while M
+// is small and the problem needs a K split anyway (few row tiles, long K); it pays for partial sums
+// and a second launch, and its registers run out as M grows.  The LDS-ring kernel takes nearly the
+// same time for every M <= 32 and needs no second launch when the row tiles alone fill the GPU.
+// Measured on one box, linear alone, register / LDS-ring kernel in us:
+//   N = 28672, K = 8192 (224 tiles):  M = 1 31.3 / 32.6, M = 4 31.4 / 31.7, M = 8 32.8 / 32.6, M = 12 34.8 / 33.7, M = 16 36.6 / 34.9, M = 32 44.7 / 35.8
+//   N = 14336, K = 4096 (112 tiles):  M = 1 13.8 / 14.4, M = 8 13.9 / 14.5, M = 12 14.0 / 14.5, M = 16 14.0 / 14.6, M = 32 16.7 / 15.0
+//   N = 4096, K = 14336 (32 tiles):   M = 1 13.9 / 15.6, M = 8 13.8 / 15.8, M = 12 14.5 / 15.9, M = 16 14.8 / 15.9, M = 32 17.6 / 16.2
+// Hence: with 192 row tiles and more the ring kernel from M = 8 on, with fewer from M = 17 on.
 static bool skinny_plan(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
   if (M < 1 || M > 32 || K % SK_STEP != 0 || N < 1) return false;
   const bool ring_ok = (K >> 1) * ST_BN < (1ll << 31) && N < (1ll << 27);  // 32-bit lane offsets
   int kind = g_forced_decode_kernel.load(std::memory_order_relaxed);
-  if (kind == 0) kind = M >= 12 ? DECODE_LDS_RING : DECODE_REGISTERS;
+  if (kind == 0) kind = M >= (ceil_div(N, ST_BN) >= 192 ? 8 : 17) ? DECODE_LDS_RING : DECODE_REGISTERS;
   if (kind == DECODE_LDS_RING && ring_ok)
     plan_lds_ring(M, N, K, p);
   else

@@ -117,7 +117,8 @@ int ac4k_linear_nvfp4(void *D, int d_dtype, const void *A, const void *A_sf, con
  * (lib/cuda/sm120/linear_nvfp4.cu:753-901; the reference runs every shape through its one
  * 128x128 tile kernel).  Two families:
  *   - decode-sized, 1 <= M <= 32 and K % 256 == 0: kernels that stream the weights once (into
- *     registers for M < 12, through an LDS ring above); the workspace receives the fp32 partial sums
+ *     registers for small M, through an LDS ring for larger M; the switch is at M = 8 when N / 128 >= 192
+ *     and at M = 17 otherwise); the workspace receives the fp32 partial sums
  *     of their K ranges when they split K; A and B 16-byte aligned;
  *   - 32 < M with too few output tiles to fill the GPU and K % 128 == 0: split-K over the tile
  *     kernel (tile shape and number of K ranges chosen by a cost model); the workspace receives

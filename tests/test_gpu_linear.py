@@ -204,7 +204,7 @@ def test_decode_sized_shapes(m, n, k):
     run_case(m, n, k, bias_dtype=torch.bfloat16, o_dtype=torch.float16, seed=n, wstd=0.02)
 
 
-# both decode-sized kernels at every M class (the library picks by M; here each is forced): ragged N,
+# both decode-sized kernels at every M class (the library picks by M and N; here each is forced): ragged N,
 # one K range and several, every output / bias type
 @pytest.mark.parametrize("kind", [1, 2])
 @pytest.mark.parametrize("m", [1, 5, 8, 11, 12, 16, 17, 31, 32])
@@ -339,3 +339,37 @@ def test_error_behaviour():
         o.linear(aq[0][:, :60], aq[1], aq[2], *bq)       # non-contiguous / K mismatch
     with pytest.raises(RuntimeError):
         o.linear(aq[0], aq[1], aq[2].reshape(1), *bq)    # global scale must be 0-dim
+
+
+@pytest.mark.parametrize("m,n,k", [(5, 7, 48), (70, 130, 80), (3, 4, 16), (33, 140, 208)])
+def test_k_not_a_multiple_of_64(m, n, k):
+    """The quantizer pads K to 64, so operands with a K % 64 tail are built by hand: random nibbles, random
+    finite block scales for the K/16 blocks that exist and 0x7E (448) in the unused slots of the last
+    scale dword, which the kernel must not read into the sum.  Checked against the C oracle (fp64 sum)
+    and against a dequantize-matmul written out here."""
+    g = torch.Generator().manual_seed(k * 1000 + m)
+    nb, nc = k // 16, (k + 63) // 64
+
+    def operand(rows):
+        packed = torch.randint(0, 256, (rows, k // 2), generator=g, dtype=torch.uint8)
+        rp = (rows + 15) // 16 * 16
+        sf = torch.full((nc, rp, 4), 0x7E, dtype=torch.uint8)
+        codes = torch.randint(0x20, 0x48, (rows, nb), generator=g, dtype=torch.uint8)  # 2^-3 .. 3.5
+        for j in range(nb):
+            sf[j // 4, :rows, j % 4] = codes[:, j]
+        return packed, sf, torch.tensor(0.5 + rows / 256.0, dtype=torch.float32)
+
+    a, b = operand(m), operand(n)
+    d = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    ops().linear(a[0].cuda(), a[1].cuda().view(torch.float8_e4m3fn), a[2].cuda(),
+                 b[0].cuda(), b[1].cuda().view(torch.float8_e4m3fn), b[2].cuda(), out=d)
+    ref_c = C.linear_nvfp4(*a, *b)
+
+    def dequant(q, rows):
+        v = T.e2m1_unpack(q[0]).float().reshape(rows, nb, 16)
+        s = T.sf_to_linear(q[1], rows)[:, :nb] * q[2]
+        return (v * s.unsqueeze(-1)).reshape(rows, k).double()
+
+    ref_t = (dequant(a, m) @ dequant(b, n).t()).float()
+    torch.testing.assert_close(ref_c, ref_t, atol=1e-4, rtol=1e-5)
+    torch.testing.assert_close(d.cpu(), ref_c, atol=1e-4, rtol=1e-5)
