@@ -887,15 +887,16 @@ static int launch_tile256p(const LinearArgs &a, hipStream_t st) {
 }
 
 // ===========================================================================
-// Decode-sized linear (1 <= M <= 32): bound by streaming the weights once.
+// Decode-sized linear (1 <= M <= 32): bound by streaming the weights once.  Two kernels; this one
+// streams the weights into registers, linear_nvfp4_stream_kernel below through an LDS ring, and
+// skinny_plan chooses between them by shape.
 //
 // A workgroup (4 waves) owns 128 weight rows and one K-slice; every wave one 32-row tile.  It
 // first decodes its slice of the packed activation to fp16 (exact, without the global scale)
 // into LDS, shared by the four waves (with more than 16 activation rows, 512 k at a time, so that
 // the LDS footprint stays at 33 KB).  Lane (row r, half h) streams 64 contiguous bytes of its weight row per 256-k step
-// (elements [128h, 128h+128) of the step) and decodes them dword by dword into MFMA operands;
-// The MFMA is issued as
-// D^T = W . Ahat^T so a lane ends up with 4 consecutive n for one m.  K-slices of one row
+// (elements [128h, 128h+128) of the step) and decodes them dword by dword into MFMA operands; the
+// MFMA is issued as D^T = W . Ahat^T so a lane ends up with 4 consecutive n for one m.  K-slices of one row
 // group meet through fp32 partial tiles in a caller-provided workspace; a small second kernel
 // adds them in slice order (deterministic), applies gsA*gsB and the bias, converts and stores.
 // (A last-arriver reduction inside the kernel needs device-scope fences, which write back the
