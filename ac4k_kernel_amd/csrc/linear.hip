@@ -1193,25 +1193,31 @@ __device__ __forceinline__ void stream_multiply(const StageFrags &cur, f32x16 (&
 }
 
 // End of the LDS-ring kernels, after the last LDS-DMA has landed and every wave has passed a barrier:
-// the two chunk sums of a wave, then the two k halves (through `xch_base`, always in this order), then
-// either the fp32 partial sums of this K range or the finished outputs (times gsA * gsB, plus bias).
-template <int D_DT, int BIAS_DT>
+// the two chunk sums of a wave, then the NK k parts of each of the NWN row groups (through `xch_base`,
+// always in this order), then either the fp32 partial sums of this K range or the finished outputs
+// (times gsA * gsB, plus bias).
+template <int D_DT, int BIAS_DT, int NK = 2, int NWN = 4>
 __device__ __forceinline__ void stream_finish(f32x16 (&acc)[2], const SkinnyArgs &a, char *xch_base, float gs_a, int wn, int kh,
                                               int lane, int64_t n0) {
   const int half = lane >> 5, r32 = lane & 31;
 #pragma unroll
   for (int e = 0; e < 16; ++e) acc[0][e] += acc[1][e];
-  float4 *xch = reinterpret_cast<float4 *>(xch_base) + (wn * 64 + lane) * 4;
-  if (kh == 1) {
+  // the NK k parts of a row group meet in the waves of part 0, added in the order of the parts
+  if (kh != 0) {
+    float4 *xch = reinterpret_cast<float4 *>(xch_base) + (((kh - 1) * NWN + wn) * 64 + lane) * 4;
 #pragma unroll
     for (int g = 0; g < 4; ++g) xch[g] = make_float4(acc[0][4 * g], acc[0][4 * g + 1], acc[0][4 * g + 2], acc[0][4 * g + 3]);
   }
   __syncthreads();
-  if (kh == 1) return;
+  if (kh != 0) return;
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const float4 o = xch[g];
-    acc[0][4 * g] += o.x; acc[0][4 * g + 1] += o.y; acc[0][4 * g + 2] += o.z; acc[0][4 * g + 3] += o.w;
+  for (int k = 1; k < NK; ++k) {
+    const float4 *xch = reinterpret_cast<const float4 *>(xch_base) + (((k - 1) * NWN + wn) * 64 + lane) * 4;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const float4 o = xch[g];
+      acc[0][4 * g] += o.x; acc[0][4 * g + 1] += o.y; acc[0][4 * g + 2] += o.z; acc[0][4 * g + 3] += o.w;
+    }
   }
 
   // acc: lane <-> m = r32, element e <-> n = (e >> 2) * 8 + half * 4 + (e & 3): four consecutive n per group
@@ -1428,10 +1434,161 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
   stream_finish<D_DT, BIAS_DT>(acc, a, stlds, *a.A_gs, wn, kh, lane, n0);
 }
 
+// ===========================================================================
+// The LDS-ring kernel with 64 weight rows per workgroup, for weights with so few rows that 128-row
+// tiles leave CUs idle or force a K split with partial sums and a second launch (N = 14336: 112
+// tiles of 128 rows, 224 of 64).  Same ring, swizzle, stage order and arithmetic; wave (wn, kq) =
+// (wave % 2, wave / 2) takes weight rows 32 wn .. 32 wn + 31 and chunk kq of every stage, and the four
+// k parts of a row group meet through LDS at the end.  A stage is 13.5 KB (64 weight rows, 32
+// activation rows, their scales), ten of them make the ring; three transfers per wave per stage.
+// Plain layout only.
+// ===========================================================================
+constexpr int S6_BN = 64;
+constexpr int S6_PS = 10;
+constexpr int S6_NPIECES = 3;
+constexpr int S6_OFF_B = 0;
+constexpr int S6_OFF_A = S6_OFF_B + S6_BN * ST_ROW;      // 32 packed activation rows
+constexpr int S6_OFF_SFB = S6_OFF_A + 32 * ST_ROW;       // weight scale dwords [chunk][64 rows]
+constexpr int S6_OFF_SFA = S6_OFF_SFB + 4 * S6_BN * 4;   // activation scale dwords [chunk][32 rows]
+constexpr int S6_STAGE_BYTES = S6_OFF_SFA + 4 * 32 * 4;  // 13824
+constexpr int S6_LDS_BYTES = S6_PS * S6_STAGE_BYTES;
+static_assert(S6_LDS_BYTES <= 160 * 1024, "the ring must fit in the CU's LDS");
+static_assert((S6_PS - 3) * S6_NPIECES <= 63, "the wait counts must fit the 6-bit counter");
+static_assert(S6_LDS_BYTES >= 3 * 2 * 64 * 16 * 4, "the ring doubles as the exchange buffer of the four k parts");
+
+template <int D_DT, int BIAS_DT>
+__global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream64_kernel(SkinnyArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char stlds[];
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, r32 = lane & 31;
+  const int swave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wn = swave & 1, kq = swave >> 1;
+  const int64_t n0 = (int64_t)blockIdx.x * S6_BN;
+  const int nst_all = (int)(a.K / ST_BK);
+  const int s0 = (int)((int64_t)nst_all * blockIdx.y / a.split_k);
+  const int nst = (int)((int64_t)nst_all * (blockIdx.y + 1) / a.split_k) - s0;  // >= 1: split_k <= stages
+  const int64_t kb = a.K >> 1;
+  const int rot = (int)(blockIdx.x % (unsigned)nst);  // stages are walked from stage b % nst on (see linear_nvfp4_stream_kernel)
+  auto stage_of = [&](int step) {
+    const int p = step + rot;
+    return p >= nst ? p - nst : p;
+  };
+  auto uniform_ptr = [](const void *p) {  // pin a wave-uniform pointer to scalar registers
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
+  };
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)stlds;
+  // (1) weight rows swave * 8 + {0..7}, 128 B each, piece p of row r at position p ^ (r & 7)
+  uint32_t offW;
+  {
+    const int loc = swave * 8 + (lane >> 3);
+    int64_t row = n0 + loc;
+    row = row < a.N ? row : a.N - 1;  // rows past N read the last row; their outputs are never stored
+    offW = (uint32_t)((row - n0) * kb + ((lane & 7) ^ (loc & 7)) * 16);
+  }
+  const uint8_t *srcW = uniform_ptr(a.B + n0 * kb + (int64_t)s0 * ST_ROW);
+  const uint32_t ldsW = (uint32_t)__builtin_amdgcn_readfirstlane(S6_OFF_B + swave * 1024);
+  // (2) waves 0..3: weight scale dwords of chunk swave, rows n0 + lane; waves 4..7: packed activation
+  //     rows (swave - 4) * 8 + {0..7}
+  uint32_t off2, lds2;
+  const uint8_t *src2;
+  int64_t stride2;
+  if (swave < 4) {
+    int64_t srow = n0 + lane;
+    srow = srow < a.Np ? srow : a.Np - 1;
+    off2 = (uint32_t)(srow * 4);
+    stride2 = 4 * a.Np * 4;  // bytes per stage (four chunk planes)
+    src2 = uniform_ptr(reinterpret_cast<const uint8_t *>(a.B_sf) + (int64_t)swave * a.Np * 4 + s0 * stride2);
+    lds2 = (uint32_t)__builtin_amdgcn_readfirstlane(S6_OFF_SFB + swave * (S6_BN * 4));
+  } else {
+    const int loc = (swave - 4) * 8 + (lane >> 3);
+    const int64_t row = loc < a.M ? loc : a.M - 1;  // rows past M read row M - 1; their outputs are never stored
+    off2 = (uint32_t)(row * kb + ((lane & 7) ^ (loc & 7)) * 16);
+    stride2 = ST_ROW;
+    src2 = uniform_ptr(a.Aq + (int64_t)s0 * ST_ROW);
+    lds2 = (uint32_t)__builtin_amdgcn_readfirstlane(S6_OFF_A + (swave - 4) * 1024);
+  }
+  // (3) activation scales of chunks 2 p + {0, 1}, p = swave % 2 (waves 2..7 repeat the transfers of waves
+  //     0 and 1: every wave issues the same count)
+  const int pair = swave & 1;
+  const int64_t arow = r32 < a.Mp ? r32 : a.Mp - 1;
+  const uint32_t off3 = (uint32_t)(((2 * pair + half) * a.Mp + arow) * 4);
+  const int64_t stride3 = 4 * a.Mp * 4;
+  const uint8_t *src3 = uniform_ptr(a.A_sf + s0 * stride3);
+  const uint32_t lds3 = (uint32_t)__builtin_amdgcn_readfirstlane(S6_OFF_SFA + pair * 256);
+  auto issue_stage = [&](int slot, int step) {  // step: position in this workgroup's order of stages
+    const int st = stage_of(step);
+    const uint32_t base = lds_base + slot * S6_STAGE_BYTES;
+    dma16(srcW + (int64_t)st * ST_ROW, offW, base, ldsW);
+    if (swave < 4)
+      dma4(src2 + st * stride2, off2, base, lds2);
+    else
+      dma16(src2 + st * stride2, off2, base, lds2);
+    dma4(src3 + st * stride3, off3, base, lds3);
+  };
+
+  // this wave's fragments of a stage: chunk kq, 32 packed elements of a weight row and of an activation
+  // row (the lane's half of the chunk) and the two block scales of each
+  struct Frags {
+    uint4 w, x;
+    uint32_t ws, xs;
+  };
+  const int wrow_l = wn * 32 + r32;
+  const int piece = kq * 2 + half;
+  const int wf_off = S6_OFF_B + wrow_l * ST_ROW + ((piece ^ (wrow_l & 7)) * 16);
+  const int xf_off = S6_OFF_A + r32 * ST_ROW + ((piece ^ (r32 & 7)) * 16);
+  const int ws_off = S6_OFF_SFB + kq * (S6_BN * 4) + wrow_l * 4 + half * 2;
+  const int xs_off = S6_OFF_SFA + kq * (32 * 4) + r32 * 4 + half * 2;
+  auto load_frags = [&](int slot) {
+    const char *st = stlds + slot * S6_STAGE_BYTES;
+    Frags f;
+    f.w = *reinterpret_cast<const uint4 *>(st + wf_off);
+    f.x = *reinterpret_cast<const uint4 *>(st + xf_off);
+    f.ws = *reinterpret_cast<const uint16_t *>(st + ws_off);
+    f.xs = *reinterpret_cast<const uint16_t *>(st + xs_off);
+    return f;
+  };
+
+  f32x16 acc[2];  // two independent accumulation chains: the first and the second half of the chunk
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[c][e] = 0.0f;
+
+  const int last = nst - 1;
+#pragma unroll
+  for (int d = 0; d < S6_PS - 1; ++d) issue_stage(d, d < last ? d : last);
+  wait_vmcnt<(S6_PS - 3) * S6_NPIECES>();
+  __syncthreads();
+  Frags cur = load_frags(0);
+
+  int slot_next = 1, slot_dma = S6_PS - 1;
+  for (int s = 0; s < nst; ++s) {
+    const Frags nxt = load_frags(slot_next);  // it landed before the previous barrier
+    const f16x2 wsc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(cur.ws, 1.0f, false);
+    const f16x2 xsc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(cur.xs, 1.0f, false);
+    acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<false>(cur.w.x, wsc), decode_dword<false>(cur.x.x, xsc), acc[0], 0, 0, 0);
+    acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<false>(cur.w.y, wsc), decode_dword<false>(cur.x.y, xsc), acc[0], 0, 0, 0);
+    acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<true>(cur.w.z, wsc), decode_dword<true>(cur.x.z, xsc), acc[1], 0, 0, 0);
+    acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(decode_dword<true>(cur.w.w, wsc), decode_dword<true>(cur.x.w, xsc), acc[1], 0, 0, 0);
+    const int sd = s + S6_PS - 1;
+    issue_stage(slot_dma, sd < last ? sd : last);
+    wait_vmcnt<(S6_PS - 3) * S6_NPIECES>();  // own transfers of stage s + 2 have landed
+    __syncthreads();
+    cur = nxt;
+    slot_next = slot_next + 1 == S6_PS ? 0 : slot_next + 1;
+    slot_dma = slot_dma + 1 == S6_PS ? 0 : slot_dma + 1;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-DMA may land after this point: the ring is reused
+  __syncthreads();
+  stream_finish<D_DT, BIAS_DT, 4, 2>(acc, a, stlds, *a.A_gs, wn, kq, lane, n0);
+}
+
 // Plan of a decode-sized linear: which of the two kernels, its K split and the fp32 scratch it needs.
-enum { DECODE_REGISTERS = 1, DECODE_LDS_RING = 2 };
+enum { DECODE_REGISTERS = 1, DECODE_LDS_RING = 2, DECODE_LDS_RING64 = 3 };
 struct SkinnyPlan {
-  int kind;                // DECODE_REGISTERS: linear_nvfp4_skinny_kernel; DECODE_LDS_RING: linear_nvfp4_stream_kernel
+  int kind;                // DECODE_REGISTERS: linear_nvfp4_skinny_kernel; DECODE_LDS_RING: linear_nvfp4_stream_kernel;
+                           // DECODE_LDS_RING64: linear_nvfp4_stream64_kernel
   int ks_len;              // register kernel: k per workgroup (256, 512 or 1024)
   int split_k;             // K ranges; > 1 needs `partial_bytes` of fp32 scratch
   int64_t partial_bytes, groups;
@@ -1457,9 +1614,9 @@ static void plan_registers(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
 
 // LDS-ring kernel: one K range per 128-row tile when the tiles alone fill the GPU; otherwise the
 // smallest number of ranges that gives about 200 workgroups, each range at least two stages long.
-static void plan_lds_ring(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
-  p.kind = DECODE_LDS_RING;
-  p.groups = ceil_div(N, ST_BN);
+static void plan_lds_ring(int64_t M, int64_t N, int64_t K, SkinnyPlan &p, int rows = ST_BN) {
+  p.kind = rows == ST_BN ? DECODE_LDS_RING : DECODE_LDS_RING64;
+  p.groups = ceil_div(N, rows);
   const int64_t stages = K / ST_BK;
   int64_t splits = 1;
   if (const int f = g_forced_skinny_ks.load(std::memory_order_relaxed)) {  // forced length of a K range
@@ -1474,25 +1631,34 @@ static void plan_lds_ring(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
   p.ks_len = 0;
   p.split_k = (int)splits;
   p.partial_bytes = splits > 1 ? splits * M * N * 4 : 0;
-  p.lds_bytes = ST_LDS_BYTES;
+  p.lds_bytes = rows == ST_BN ? ST_LDS_BYTES : S6_LDS_BYTES;
 }
 
-// Shapes of the decode-sized kernels (both need K % 256 == 0) and the choice between them.  The
+// Shapes of the decode-sized kernels (all need K % 256 == 0) and the choice between them.  The
 // register kernel has all its loads in flight at once and four workgroups per CU, which wins while M
 // is small and the problem needs a K split anyway (few row tiles, long K); it pays for partial sums
-// and a second launch, and its registers run out as M grows.  The LDS-ring kernel takes nearly the
-// same time for every M <= 32 and needs no second launch when the row tiles alone fill the GPU.
-// Measured on one box, linear alone, register / LDS-ring kernel in us:
-//   N = 28672, K = 8192 (224 tiles):  M = 1 31.3 / 32.6, M = 4 31.4 / 31.7, M = 8 32.8 / 32.6, M = 12 34.8 / 33.7, M = 16 36.6 / 34.9, M = 32 44.7 / 35.8
-//   N = 14336, K = 4096 (112 tiles):  M = 1 13.8 / 14.4, M = 8 13.9 / 14.5, M = 12 14.0 / 14.5, M = 16 14.0 / 14.6, M = 32 16.7 / 15.0
-//   N = 4096, K = 14336 (32 tiles):   M = 1 13.9 / 15.6, M = 8 13.8 / 15.8, M = 12 14.5 / 15.9, M = 16 14.8 / 15.9, M = 32 17.6 / 16.2
-// Hence: with 192 row tiles and more the ring kernel from M = 8 on, with fewer from M = 17 on.
+// and a second launch, and its registers run out as M grows.  The LDS-ring kernels take nearly the
+// same time for every M <= 32 and need no second launch when their row tiles alone fill the GPU:
+// 128-row tiles when there are 192 of them, 64-row tiles for narrower weights.
+// Measured on one box, linear alone, weights from HBM, register / ring 128 / ring 64 in us:
+//   N = 28672, K = 8192 (224 / 448 tiles):  M = 1 31.0 / 32.4 / 41.3, M = 8 35.1 / 33.6 / 41.6, M = 16 40.4 / 35.5 / 42.7, M = 32 45.5 / 37.3 / 44.3
+//   N = 14336, K = 4096 (112 / 224 tiles):  M = 1 14.0 / 15.5 / 13.8, M = 8 14.5 / 15.8 / 14.2, M = 16 17.6 / 16.4 / 13.9, M = 32 22.1 / 17.2 / 14.9
+//   N = 4096, K = 14336 (32 / 64 tiles):    M = 1 15.1 / 16.8 / 16.2, M = 8 16.3 / 17.3 / 16.3, M = 16 18.7 / 17.5 / 16.9, M = 32 22.9 / 17.8 / 17.1
+// Hence: with 192 tiles of 128 rows and more, 128-row tiles from M = 8 on; otherwise 64-row tiles when
+// there are 192 of those, or from M = 8 on; the register kernel in the remaining cases.
 static bool skinny_plan(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
   if (M < 1 || M > 32 || K % SK_STEP != 0 || N < 1) return false;
   const bool ring_ok = (K >> 1) * ST_BN < (1ll << 31) && N < (1ll << 27);  // 32-bit lane offsets
   int kind = g_forced_decode_kernel.load(std::memory_order_relaxed);
-  if (kind == 0) kind = M >= (ceil_div(N, ST_BN) >= 192 ? 8 : 17) ? DECODE_LDS_RING : DECODE_REGISTERS;
-  if (kind == DECODE_LDS_RING && ring_ok)
+  if (kind == 0) {
+    if (ceil_div(N, ST_BN) >= 192)
+      kind = M >= 8 ? DECODE_LDS_RING : DECODE_REGISTERS;
+    else
+      kind = (M >= 8 || ceil_div(N, S6_BN) >= 192) ? DECODE_LDS_RING64 : DECODE_REGISTERS;
+  }
+  if (kind == DECODE_LDS_RING64 && ring_ok)
+    plan_lds_ring(M, N, K, p, S6_BN);
+  else if (kind == DECODE_LDS_RING && ring_ok)
     plan_lds_ring(M, N, K, p);
   else
     plan_registers(M, N, K, p);
@@ -1515,6 +1681,11 @@ static int launch_skinny(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_t s
     static std::atomic<uint32_t> lds_ok{0};
     if (int rc = allow_dynamic_lds(kern, lds_ok, ST_LDS_BYTES)) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)p.groups, (unsigned)p.split_k), dim3(ST_THREADS), ST_LDS_BYTES, st, a);
+  } else if (p.kind == DECODE_LDS_RING64) {
+    auto *kern = linear_nvfp4_stream64_kernel<D_DT, BIAS_DT>;
+    static std::atomic<uint32_t> lds_ok{0};
+    if (int rc = allow_dynamic_lds(kern, lds_ok, S6_LDS_BYTES)) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)p.groups, (unsigned)p.split_k), dim3(ST_THREADS), S6_LDS_BYTES, st, a);
   } else if (p.kind == DECODE_LDS_RING) {
     auto *kern = linear_nvfp4_stream_kernel<D_DT, BIAS_DT, false>;
     static std::atomic<uint32_t> lds_ok{0};
@@ -1936,8 +2107,9 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_fused_bf
 
 extern "C" __attribute__((visibility("default"))) int ac4k_set_linear_tuning(int mi, int nj, int splits, int skinny_ks,
                                                                           int decode_kernel) {
-  AC4K_REQUIRE(decode_kernel >= 0 && decode_kernel <= 2,
-               "decode_kernel must be 0 (by shape), 1 (register kernel) or 2 (LDS-ring kernel) (got %d)", decode_kernel);
+  AC4K_REQUIRE(decode_kernel >= 0 && decode_kernel <= 3,
+               "decode_kernel must be 0 (by shape), 1 (register kernel), 2 (LDS-ring kernel) or 3 (LDS-ring kernel with "
+               "64-row tiles) (got %d)", decode_kernel);
   ac4k::g_forced_decode_kernel.store(decode_kernel);
   if (mi == 0 && nj == 0 && splits == 0) {
     ac4k::g_forced_tile_plan.store(0);

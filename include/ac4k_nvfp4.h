@@ -117,8 +117,8 @@ int ac4k_linear_nvfp4(void *D, int d_dtype, const void *A, const void *A_sf, con
  * (lib/cuda/sm120/linear_nvfp4.cu:753-901; the reference runs every shape through its one
  * 128x128 tile kernel).  Two families:
  *   - decode-sized, 1 <= M <= 32 and K % 256 == 0: kernels that stream the weights once (into
- *     registers for small M, through an LDS ring for larger M; the switch is at M = 8 when N / 128 >= 192
- *     and at M = 17 otherwise); the workspace receives the fp32 partial sums
+ *     registers for small M, through an LDS ring with 128- or 64-row tiles for larger M and for
+ *     weights of 12288 to 24575 rows); the workspace receives the fp32 partial sums
  *     of their K ranges when they split K; A and B 16-byte aligned;
  *   - 32 < M with too few output tiles to fill the GPU and K % 128 == 0: split-K over the tile
  *     kernel (tile shape and number of K ranges chosen by a cost model); the workspace receives
@@ -153,7 +153,7 @@ int ac4k_linear_nvfp4_skinny_static(void *D, int d_dtype, const void *A, const v
  * ranges (mi in {2,4}, nj in {1,2,4}, not (4,1); splits > 1 only takes effect in the workspace entry
  * points), the length of a K range of the decode-sized kernels (a multiple of 256; the register
  * kernel takes 256, 512 or 1024) and which decode-sized kernel runs (1 = weights streamed into
- * registers, 2 = weights streamed through an LDS ring).  Zeros give each choice back to the library.
+ * registers, 2 = weights streamed through an LDS ring in 128-row tiles, 3 = in 64-row tiles).  Zeros give each choice back to the library.
  * Process-wide; returns non-zero on values outside these sets. */
 int ac4k_set_linear_tuning(int mi, int nj, int splits, int skinny_ks, int decode_kernel);
 

@@ -65,7 +65,7 @@ def test_argument_rejection_without_gpu():
     # tuning values outside the instantiated kernels are refused, zeros are accepted
     assert lib.ac4k_set_linear_tuning(4, 1, 1, 0, 0) != 0 and b"tile plan" in lib.ac4k_last_error()
     assert lib.ac4k_set_linear_tuning(0, 0, 0, 100, 0) != 0 and b"skinny_ks" in lib.ac4k_last_error()
-    assert lib.ac4k_set_linear_tuning(0, 0, 0, 0, 3) != 0 and b"decode_kernel" in lib.ac4k_last_error()
+    assert lib.ac4k_set_linear_tuning(0, 0, 0, 0, 4) != 0 and b"decode_kernel" in lib.ac4k_last_error()
     assert lib.ac4k_set_linear_tuning(0, 0, 0, 0, 0) == 0
     assert lib.ac4k_debug_last_quantize_path() in (0, 1, 2, 3)
     rc = lib.ac4k_linear_nvfp4_fused_bf16(one, 0, one, one, one, one, one, one, one, None, 0, 64, 4, 64, one, 0, None)

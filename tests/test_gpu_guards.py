@@ -120,7 +120,7 @@ def test_linear_stays_inside_its_output(m, n, k, plan, odt, linear_tuning):
         assert same_bytes(w.t, ref), (m, n, k, plan, shift)
 
 
-@pytest.mark.parametrize("kind", [0, 1, 2])  # decode-sized shapes: the library's choice, register kernel, LDS-ring kernel
+@pytest.mark.parametrize("kind", [0, 1, 2, 3])  # decode-sized shapes: the library's choice, register kernel, LDS ring (128, 64 rows)
 @pytest.mark.parametrize("m,n,k", [(1, 1000, 1024), (5, 136, 2048), (32, 520, 512), (16, 130, 3584), (128, 1024, 4096),
                                    (96, 300, 2048)])
 def test_workspace_linear_stays_inside_workspace_and_output(m, n, k, kind, linear_tuning):

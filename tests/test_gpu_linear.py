@@ -204,9 +204,10 @@ def test_decode_sized_shapes(m, n, k):
     run_case(m, n, k, bias_dtype=torch.bfloat16, o_dtype=torch.float16, seed=n, wstd=0.02)
 
 
-# both decode-sized kernels at every M class (the library picks by M and N; here each is forced): ragged N,
-# one K range and several, every output / bias type
-@pytest.mark.parametrize("kind", [1, 2])
+# the decode-sized kernels at every M class (the library picks by M and N; here each is forced: 1 registers,
+# 2 LDS ring with 128-row tiles, 3 LDS ring with 64-row tiles): ragged N, one K range and several, every
+# output / bias type
+@pytest.mark.parametrize("kind", [1, 2, 3])
 @pytest.mark.parametrize("m", [1, 5, 8, 11, 12, 16, 17, 31, 32])
 def test_decode_kernels_forced(kind, m, linear_tuning):
     linear_tuning(decode_kernel=kind)
