@@ -1242,13 +1242,27 @@ __device__ __forceinline__ void stream_finish(f32x16 (&acc)[2], const SkinnyArgs
   using DE = Elem<D_DT>;
   typename DE::T *Dp = static_cast<typename DE::T *>(a.D);
   const float scale = gs_a * (*a.B_gs);
+  // a lane's four consecutive outputs of a group leave as one 8- or 16-byte store where the rows allow it
+  const bool vec_ok = (a.N & 3) == 0 && ((uintptr_t)a.D & 15) == 0;
 #pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const int64_t n = nw + (e >> 2) * 8 + half * 4 + (e & 3);
-    if (n < a.N) {
-      float v = acc[0][e] * scale;
-      if constexpr (BIAS_DT != BIAS_NONE) v += Elem<BIAS_DT>::load(a.bias, n);
-      Dp[(int64_t)m * a.N + n] = DE::cvt(v);
+  for (int g = 0; g < 4; ++g) {
+    const int64_t n = nw + g * 8 + half * 4;
+    float v[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      v[q] = acc[0][4 * g + q] * scale;
+      if constexpr (BIAS_DT != BIAS_NONE) v[q] += n + q < a.N ? Elem<BIAS_DT>::load(a.bias, n + q) : 0.0f;
+    }
+    typename DE::T *dst = Dp + (int64_t)m * a.N + n;
+    if (vec_ok && n + 3 < a.N) {
+      if constexpr (sizeof(typename DE::T) == 2)
+        *reinterpret_cast<uint2 *>(dst) = make_uint2(DE::cvt2(v[0], v[1]), DE::cvt2(v[2], v[3]));
+      else
+        *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (n + q < a.N) dst[q] = DE::cvt(v[q]);
     }
   }
 }
