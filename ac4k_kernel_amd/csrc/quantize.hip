@@ -554,9 +554,14 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_small_kernel(
     OnePassGeom g, float max_scale) {
   __shared__ float lut[128];
   __shared__ uint32_t red[OP_THREADS / 64];
+  // Only every eighth workgroup works (NSEG > 1): workgroups are dealt round-robin to the 8 XCDs, so the
+  // working ones share ONE L2 and their reads of the whole tensor meet there instead of crossing the
+  // fabric eight times.
+  if (NSEG > 1 && (blockIdx.x & 7)) return;
+  const uint32_t seg = NSEG > 1 ? blockIdx.x >> 3 : blockIdx.x;
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t nvec = g.total_chunks * 8;
-  const uint32_t lv = blockIdx.x * OP_THREADS + tid;  // this lane's vector of the workgroup's own segment
+  const uint32_t lv = seg * OP_THREADS + tid;  // this lane's vector of the workgroup's own segment
   uint4 own = make_uint4(0, 0, 0, 0);
   if (lv < nvec) own = in[lv];
   uint4 v[NSEG];
@@ -575,7 +580,7 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_small_kernel(
   __syncthreads();
   const uint32_t gm = group_umax<16>(red[lane & 15]);
   const float gs = bf16_bits_to_f32(gm) / max_scale;
-  if (blockIdx.x == 0 && tid == 0) *gs_out = gs;
+  if (seg == 0 && tid == 0) *gs_out = gs;
   const float alpha = 1.0f / gs;
   if (g.swizzle) own = swizzle_nvfp4_quad(own, (int)lane);  // the maximum above does not depend on the order
   uint32_t bm = absmax_bf16x8(own);
@@ -593,7 +598,7 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_small_kernel(
       sf[((uint64_t)l * g.ncc + cc) * g.Rp + r] = sfw;
     }
   }
-  if (g.Rp > g.R && blockIdx.x == 0) {  // zero scales of the pad rows R..Rp-1
+  if (g.Rp > g.R && seg == 0) {  // zero scales of the pad rows R..Rp-1
     const uint32_t pad = g.Rp - g.R, npad = g.lead * g.ncc * pad;
     for (uint32_t i = tid; i < npad; i += OP_THREADS) sf[(uint64_t)(i / pad) * g.Rp + g.R + i % pad] = 0u;
   }
@@ -1122,7 +1127,7 @@ constexpr int SMALL_MAX_SEGS = 16;
 static void launch_small(uint32_t *out, uint32_t *sf, const uint4 *in, float *gs, const OnePassGeom &g,
                          float max_scale, hipStream_t st) {
   const unsigned nseg = (unsigned)ceil_div((int64_t)g.total_chunks, 128);
-  const dim3 grid(nseg), block(OP_THREADS);
+  const dim3 grid(nseg <= 1 ? 1 : nseg * 8), block(OP_THREADS);  // NSEG > 1: one working workgroup in eight, all on one XCD
   if (nseg <= 1) hipLaunchKernelGGL(quantize_nvfp4_small_kernel<1>, grid, block, 0, st, out, sf, in, gs, g, max_scale);
   else if (nseg <= 2) hipLaunchKernelGGL(quantize_nvfp4_small_kernel<2>, grid, block, 0, st, out, sf, in, gs, g, max_scale);
   else if (nseg <= 4) hipLaunchKernelGGL(quantize_nvfp4_small_kernel<4>, grid, block, 0, st, out, sf, in, gs, g, max_scale);
@@ -1145,7 +1150,10 @@ static int try_quantize_nvfp4_onepass(void *out, void *sf, float *gs, const void
   if (nwg < 8 || chunks > (int64_t)nwg * 128 * OP_MAX_NV) return QPATH_NONE;
   const OnePassGeom g{(uint32_t)chunks, (uint32_t)(K / 64), (uint32_t)R, (uint32_t)align_up(R, 16), (uint32_t)lead,
                       swizzle ? 1u : 0u};
-  if (chunks <= 128 * SMALL_MAX_SEGS) {  // small: one launch, no grid wait, no state
+  // small: one launch, no grid wait, no state.  Above eight segments the kernel with the grid wait is
+  // faster (256 KB: 5.0 against 6.1 us in front of a dependent kernel), but it is not available under
+  // capture, where the stateless kernel keeps the call at one launch.
+  if (chunks <= 128 * 8 || (chunks <= 128 * SMALL_MAX_SEGS && stream_is_capturing(st))) {
     launch_small(static_cast<uint32_t *>(out), static_cast<uint32_t *>(sf), static_cast<const uint4 *>(in), gs, g,
                  max_scale, st);
     return QPATH_SMALL;
