@@ -67,7 +67,8 @@ int ac4k_quantize_nvfp4(void *out, void *sf, const void *in, const float *global
  * input, then ac4k_quantize_nvfp4 with it.  `in` must be dense: the four dims, in any order, tile
  * d0*d1*R*K contiguous elements (the reference op makes its input contiguous, :201); other strides
  * are rejected.  Nothing to initialise, no host synchronisation.
- *   - dense row-major tensors (sK == 1, K % 64 == 0, 16-byte aligned) of up to 256 KB: one launch;
+ *   - dense row-major tensors (sK == 1, K % 64 == 0, 16-byte aligned) of up to 128 KB (256 KB while
+ *     `stream` is capturing): one launch;
  *   - the same up to 64 MiB: one launch of a kernel whose workgroups exchange their maxima through
  *     synchronisation words inside the library (32 sets per GPU, handed to the most recently used
  *     streams), see ac4k_set_quantize_sync_timeout_us;
