@@ -69,3 +69,41 @@ def test_static_scratch_entry_rejects_what_does_not_fit():
     # shapes that take no scratch are refused like ac4k_linear_nvfp4_skinny refuses them
     rc = L.ac4k_linear_nvfp4_skinny_static(one, 0, one, one, one, one, one, one, None, 0, 8192, 8192, 8192, None)
     assert rc != 0 and b"no workspace-assisted path" in L.ac4k_last_error()
+
+
+def test_static_scratch_entry_under_graph_capture(linear_tuning):
+    """The callers the entry point is for: a decode step captured into a HIP graph (quantize, then the
+    linear on the library's own scratch; no allocation inside the capture), replayed on fresh activations
+    with eager work in between, equals the eager result every time.  A shape that splits K is used, so
+    the replays really go through the scratch array."""
+    from ac4k_kernel_amd import _lib, _rocm_ops, ops
+    L = _lib.load()
+    m, n, k = 4, 1024, 4096
+    need = L.ac4k_linear_nvfp4_skinny_workspace_bytes(m, n, k)
+    assert 256 < need <= STATIC_BYTES  # more than the marker value: partial sums go through the scratch
+    wq = ops.quantize(make_input((n, k), seed=91, std=0.02).cuda(), 0, 1)
+    x_static = make_input((m, k), seed=92).cuda()
+    xq = ops.quantize(x_static, 0, 1)  # output buffers of the captured quantize
+    d_static = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    d_eager = torch.zeros_like(d_static)
+    st = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
+
+    def linear_static(dst):
+        _lib.check(L.ac4k_linear_nvfp4_skinny_static(dst.data_ptr(), 0, xq[0].data_ptr(), xq[1].data_ptr(),
+                                                     xq[2].data_ptr(), wq[0].data_ptr(), wq[1].data_ptr(),
+                                                     wq[2].data_ptr(), None, 0, m, n, k, st()))
+
+    linear_static(d_eager)  # first call on this GPU outside capture: it looks up the array's address
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _rocm_ops.quantize_nvfp4_with_global_scale(xq[0], xq[1], xq[2], x_static, 0, 1, False, 2688.0)
+        linear_static(d_static)
+    for seed in (101, 102, 103):
+        x = make_input((m, k), seed=seed, outliers=True).cuda()
+        x_static.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = d_static.clone()
+        ref = ops.linear(*ops.quantize(x, 0, 1), *wq)  # eager work between the replays, and the expected value
+        assert torch.equal(got, ref), f"replay with seed {seed}: {(got != ref).sum().item()} outputs differ"
