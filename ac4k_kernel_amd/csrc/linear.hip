@@ -1133,10 +1133,11 @@ static void launch_reduce(const SkinnyArgs &a, hipStream_t st) {
 //
 // A workgroup (8 waves) owns 128 weight rows and a contiguous range of 256-k stages.  Weights, weight
 // scales, the packed activation rows and their scales go from global memory straight into an LDS ring
-// of ST_PS stages with LDS-DMA loads: lane l of a transfer fetches piece l % 8 of row l / 8, so eight
+// of six or seven stages with LDS-DMA loads: lane l of a transfer fetches piece l % 8 of row l / 8, so eight
 // lanes read one 128-byte run of a row, and every request is a full 64-byte line.  (With loads into
 // registers in the MFMA operand layout every lane reads from a different row: four times the address
-// work per byte, and the partial sums of a K split on top.)  Wave (wn, kh) = (wave % 4, wave / 4) takes
+// work per byte, and the partial sums of a K split on top; the same pattern with 16 bytes per lane, as a
+// wave's fragment of one stage would need, measured 2 TB/s.)  Wave (wn, kh) = (wave % 4, wave / 4) takes
 // weight rows 32 wn .. 32 wn + 31 and the 64-chunks 2 kh, 2 kh + 1 of every stage: its packed
 // fragments of the NEXT stage travel from LDS to registers while it decodes the current ones in
 // registers (weights and activation alike: 4 converts + 4 packed multiplies per 8 elements) and
@@ -1152,24 +1153,25 @@ constexpr int ST_BN = 128;        // weight rows per workgroup
 constexpr int ST_THREADS = 512;
 constexpr int ST_BK = 256;        // k per stage (four 64-chunks)
 constexpr int ST_ROW = ST_BK / 2; // packed bytes per row per stage
-constexpr int ST_PS = 6;
 constexpr int ST_NPIECES = 4;     // LDS-DMA instructions per wave per stage (three from a weight image)
+// A stage: the weight rows, their scale dwords [chunk][128 rows], MR packed activation rows and their scale
+// dwords [chunk][MR rows].  MR is 32, or 16 when M <= 16: the smaller stage leaves room for a seventh one
+// in the ring, i.e. one more stage of weights in flight.
 constexpr int ST_OFF_B = 0;
-constexpr int ST_OFF_A = ST_OFF_B + ST_BN * ST_ROW;     // 32 packed activation rows
-constexpr int ST_OFF_SFB = ST_OFF_A + 32 * ST_ROW;      // weight scale dwords [chunk][128 rows]
-constexpr int ST_OFF_SFA = ST_OFF_SFB + 4 * ST_BN * 4;  // activation scale dwords [chunk][32 rows]
-constexpr int ST_STAGE_BYTES = ST_OFF_SFA + 4 * 32 * 4;
-constexpr int ST_LDS_BYTES = ST_PS * ST_STAGE_BYTES;
-static_assert(ST_LDS_BYTES <= 160 * 1024, "the ring must fit in the CU's LDS");
-static_assert((ST_PS - 3) * ST_NPIECES <= 63, "the wait counts must fit the 6-bit counter");
-static_assert(ST_LDS_BYTES >= 4 * 64 * 16 * 4, "the ring doubles as the exchange buffer of the two k halves");
-// From a weight image (PRE) a stage's weights and weight scales are ONE contiguous run of two blocks,
-// copied as it lies to the head of the LDS stage by 18 one-kilobyte transfers; with the four transfers
-// of the activation rows and the two of their scales that is three per wave.  The activation part of
-// the stage keeps its layout.
+constexpr int ST_OFF_SFB = ST_OFF_B + ST_BN * ST_ROW;
+constexpr int ST_OFF_A = ST_OFF_SFB + 4 * ST_BN * 4;  // 18432
+__host__ __device__ constexpr int st_off_sfa(int mr) { return ST_OFF_A + mr * ST_ROW; }
+__host__ __device__ constexpr int st_stage_bytes(int mr) { return st_off_sfa(mr) + 4 * mr * 4; }
+__host__ __device__ constexpr int st_stages(int mr) { return mr == 32 ? 6 : 7; }
+__host__ __device__ constexpr int st_lds_bytes(int mr) { return st_stages(mr) * st_stage_bytes(mr); }
+static_assert(st_lds_bytes(32) <= 160 * 1024 && st_lds_bytes(16) <= 160 * 1024, "the ring must fit in the CU's LDS");
+static_assert((st_stages(16) - 3) * ST_NPIECES <= 63, "the wait counts must fit the 6-bit counter");
+static_assert(st_lds_bytes(16) >= 4 * 64 * 16 * 4, "the ring doubles as the exchange buffer of the two k halves");
+// From a weight image (PRE) the weights and weight scales of a stage are ONE contiguous run of two blocks,
+// copied as it lies to the head of the LDS stage by 18 one-kilobyte transfers; with the transfers of the
+// activation rows and of their scales that is three per wave.  The activation part of the stage is the same.
 constexpr int ST_PRE_W_BYTES = 2 * W_BLOCK_BYTES;  // 18432
-static_assert(ST_PRE_W_BYTES == ST_OFF_A + 4 * ST_BN * 4, "both layouts must give the same stage size");
-constexpr int ST_PRE_OFF_A = ST_PRE_W_BYTES, ST_PRE_OFF_SFA = ST_PRE_OFF_A + 32 * ST_ROW;
+static_assert(ST_PRE_W_BYTES == ST_OFF_A, "both layouts put the activation behind 18 KB of weights and scales");
 constexpr int ST_PRE_NPIECES = 3;
 
 // a wave's fragments of one stage: for each of its two 64-chunks (2 kh, 2 kh + 1) 32 packed elements
@@ -1267,10 +1269,12 @@ __device__ __forceinline__ void stream_finish(f32x16 (&acc)[2], const SkinnyArgs
   }
 }
 
-template <int D_DT, int BIAS_DT, bool PRE>
+template <int D_DT, int BIAS_DT, bool PRE, int MR>
 __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(SkinnyArgs a) {
+  static_assert(MR == 32 || MR == 16, "activation rows per stage");
   constexpr int NPIECES = PRE ? ST_PRE_NPIECES : ST_NPIECES;
-  constexpr int OFF_A = PRE ? ST_PRE_OFF_A : ST_OFF_A, OFF_SFA = PRE ? ST_PRE_OFF_SFA : ST_OFF_SFA;
+  constexpr int OFF_A = ST_OFF_A, OFF_SFA = st_off_sfa(MR);
+  constexpr int ST_PS = st_stages(MR), ST_STAGE_BYTES = st_stage_bytes(MR);
   extern __shared__ __attribute__((aligned(16))) char stlds[];
   const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, r32 = lane & 31;
   const int swave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1340,11 +1344,13 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
     srcS = uniform_ptr(reinterpret_cast<const uint8_t *>(a.B_sf) + (int64_t)(swave >> 1) * a.Np * 4 + s0 * strideS);
     ldsS = (uint32_t)__builtin_amdgcn_readfirstlane(ST_OFF_SFB + (swave >> 1) * (ST_BN * 4) + (swave & 1) * 256);
   }
-  // activation: four waves take the packed rows w * 8 + {0..7}, two the scales of chunks 2 p + {0, 1};
-  // without an image waves 6 and 7 repeat the scale transfers (every wave issues the same count), with
-  // one waves 0 and 1 have their third weight transfer instead
-  constexpr int A_FIRST = PRE ? 2 : 0;  // first wave of the four that move the rows
-  const bool moves_rows = swave >= A_FIRST && swave < A_FIRST + 4;
+  // activation: MR / 8 waves take the packed rows w * 8 + {0..7}; the scale dwords are one transfer for
+  // MR = 16 (lane = chunk x row) and two for MR = 32 (chunks 2 p + {0, 1}, p = 0, 1).  From an image waves
+  // 0 and 1 have their third weight transfer first.  The waves left over repeat a scale transfer: every wave
+  // issues the same count.
+  constexpr int A_FIRST = PRE ? 2 : 0;  // first wave of those that move the rows
+  constexpr int A_WAVES = MR / 8;
+  const bool moves_rows = swave >= A_FIRST && swave < A_FIRST + A_WAVES;
   uint32_t off4 = 0, lds4 = 0;
   const uint8_t *src4 = nullptr;
   int64_t stride4 = 0;
@@ -1355,13 +1361,18 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
     stride4 = ST_ROW;
     src4 = uniform_ptr(a.Aq + (int64_t)s0 * ST_ROW);
     lds4 = (uint32_t)__builtin_amdgcn_readfirstlane(OFF_A + (swave - A_FIRST) * 1024);
-  } else if (!PRE || swave >= 6) {
-    const int pair = swave & 1;  // chunks 2 pair, 2 pair + 1
-    const int64_t row = r32 < a.Mp ? r32 : a.Mp - 1;
-    off4 = (uint32_t)(((2 * pair + half) * a.Mp + row) * 4);
+  } else if (!PRE || swave >= 2) {
     stride4 = 4 * a.Mp * 4;
     src4 = uniform_ptr(a.A_sf + s0 * stride4);
-    lds4 = (uint32_t)__builtin_amdgcn_readfirstlane(OFF_SFA + pair * 256);
+    if constexpr (MR == 32) {
+      const int pair = swave & 1;  // chunks 2 pair, 2 pair + 1
+      const int64_t row = r32 < a.Mp ? r32 : a.Mp - 1;
+      off4 = (uint32_t)(((2 * pair + half) * a.Mp + row) * 4);
+      lds4 = (uint32_t)__builtin_amdgcn_readfirstlane(OFF_SFA + pair * 256);
+    } else {
+      off4 = (uint32_t)(((lane >> 4) * a.Mp + (lane & 15)) * 4);  // Mp >= 16
+      lds4 = (uint32_t)__builtin_amdgcn_readfirstlane(OFF_SFA);
+    }
   }
   auto issue_stage = [&](int slot, int step) {  // step: position in this workgroup's order of stages
     const int st = stage_of(step);
@@ -1372,13 +1383,13 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
     if constexpr (PRE) {
       if (swave < 2)
         dma16(pw, offW[2], base, (uint32_t)__builtin_amdgcn_readfirstlane((16 + swave) * 1024));
-      else if (swave < 6)
+      else if (moves_rows)
         dma16(src4 + st * stride4, off4, base, lds4);
       else
         dma4(src4 + st * stride4, off4, base, lds4);
     } else {
       dma4(srcS + st * strideS, offS, base, ldsS);
-      if (swave < 4)
+      if (moves_rows)
         dma16(src4 + st * stride4, off4, base, lds4);
       else
         dma4(src4 + st * stride4, off4, base, lds4);
@@ -1386,6 +1397,7 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
   };
 
   const int wrow_l = wn * 32 + r32;
+  const int xrow = r32 & (MR - 1);  // lanes of rows past MR read a staged row; their outputs are never stored
   int wf_off[2], xf_off[2];
 #pragma unroll
   for (int c = 0; c < 2; ++c) {
@@ -1394,12 +1406,12 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
       wf_off[c] = kh * W_BLOCK_BYTES + wrow_l * 64 + (((c * 2 + half) ^ ((wrow_l >> 1) & 3)) * 16);
     else
       wf_off[c] = ST_OFF_B + wrow_l * ST_ROW + ((piece ^ (wrow_l & 7)) * 16);
-    xf_off[c] = OFF_A + r32 * ST_ROW + ((piece ^ (r32 & 7)) * 16);
+    xf_off[c] = OFF_A + xrow * ST_ROW + ((piece ^ (xrow & 7)) * 16);
   }
   // scale planes of the wave's two chunks: `ws_pitch` bytes apart
   constexpr int ws_pitch = PRE ? W_BLOCK_ROWS * 4 : ST_BN * 4;
   const int ws_off = (PRE ? kh * W_BLOCK_BYTES + W_BLOCK_DATA : ST_OFF_SFB + (kh * 2) * (ST_BN * 4)) + wrow_l * 4 + half * 2;
-  const int xs_off = OFF_SFA + (kh * 2) * (32 * 4) + r32 * 4 + half * 2;
+  const int xs_off = OFF_SFA + (kh * 2) * (MR * 4) + xrow * 4 + half * 2;
   auto load_frags = [&](int slot) {
     const char *st = stlds + slot * ST_STAGE_BYTES;
     StageFrags f;
@@ -1408,7 +1420,7 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
       f.w[c] = *reinterpret_cast<const uint4 *>(st + wf_off[c]);
       f.x[c] = *reinterpret_cast<const uint4 *>(st + xf_off[c]);
       f.ws[c] = *reinterpret_cast<const uint16_t *>(st + ws_off + c * ws_pitch);
-      f.xs[c] = *reinterpret_cast<const uint16_t *>(st + xs_off + c * (32 * 4));
+      f.xs[c] = *reinterpret_cast<const uint16_t *>(st + xs_off + c * (MR * 4));
     }
     return f;
   };
@@ -1645,7 +1657,7 @@ static void plan_lds_ring(int64_t M, int64_t N, int64_t K, SkinnyPlan &p, int ro
   p.ks_len = 0;
   p.split_k = (int)splits;
   p.partial_bytes = splits > 1 ? splits * M * N * 4 : 0;
-  p.lds_bytes = rows == ST_BN ? ST_LDS_BYTES : S6_LDS_BYTES;
+  p.lds_bytes = rows == ST_BN ? st_lds_bytes(M <= 16 ? 16 : 32) : S6_LDS_BYTES;
 }
 
 // Shapes of the decode-sized kernels (all need K % 256 == 0) and the choice between them.  The
@@ -1688,23 +1700,29 @@ static int launch_skinny_it(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_
   return 0;
 }
 
+template <int D_DT, int BIAS_DT, bool PRE, int MR>
+static int launch_ring(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_t st) {
+  auto *kern = linear_nvfp4_stream_kernel<D_DT, BIAS_DT, PRE, MR>;
+  static std::atomic<uint32_t> lds_ok{0};
+  if (int rc = allow_dynamic_lds(kern, lds_ok, st_lds_bytes(MR))) return rc;
+  hipLaunchKernelGGL(kern, dim3((unsigned)p.groups, (unsigned)p.split_k), dim3(ST_THREADS), st_lds_bytes(MR), st, a);
+  return 0;
+}
+
 template <int D_DT, int BIAS_DT>
 static int launch_skinny(const SkinnyArgs &a, const SkinnyPlan &p, hipStream_t st) {
-  if (p.kind == DECODE_LDS_RING && a.prepacked) {
-    auto *kern = linear_nvfp4_stream_kernel<D_DT, BIAS_DT, true>;
-    static std::atomic<uint32_t> lds_ok{0};
-    if (int rc = allow_dynamic_lds(kern, lds_ok, ST_LDS_BYTES)) return rc;
-    hipLaunchKernelGGL(kern, dim3((unsigned)p.groups, (unsigned)p.split_k), dim3(ST_THREADS), ST_LDS_BYTES, st, a);
+  if (p.kind == DECODE_LDS_RING) {
+    int rc;
+    if (a.M <= 16)
+      rc = a.prepacked ? launch_ring<D_DT, BIAS_DT, true, 16>(a, p, st) : launch_ring<D_DT, BIAS_DT, false, 16>(a, p, st);
+    else
+      rc = a.prepacked ? launch_ring<D_DT, BIAS_DT, true, 32>(a, p, st) : launch_ring<D_DT, BIAS_DT, false, 32>(a, p, st);
+    if (rc) return rc;
   } else if (p.kind == DECODE_LDS_RING64) {
     auto *kern = linear_nvfp4_stream64_kernel<D_DT, BIAS_DT>;
     static std::atomic<uint32_t> lds_ok{0};
     if (int rc = allow_dynamic_lds(kern, lds_ok, S6_LDS_BYTES)) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)p.groups, (unsigned)p.split_k), dim3(ST_THREADS), S6_LDS_BYTES, st, a);
-  } else if (p.kind == DECODE_LDS_RING) {
-    auto *kern = linear_nvfp4_stream_kernel<D_DT, BIAS_DT, false>;
-    static std::atomic<uint32_t> lds_ok{0};
-    if (int rc = allow_dynamic_lds(kern, lds_ok, ST_LDS_BYTES)) return rc;
-    hipLaunchKernelGGL(kern, dim3((unsigned)p.groups, (unsigned)p.split_k), dim3(ST_THREADS), ST_LDS_BYTES, st, a);
   } else {
     int rc;
     if (a.M <= 8) rc = launch_skinny_it<D_DT, BIAS_DT, 1>(a, p, st);
