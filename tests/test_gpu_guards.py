@@ -160,3 +160,32 @@ def test_fused_linear_stays_inside_every_buffer(m, n, k):
     torch.cuda.synchronize()
     assert all(w.intact() for w in (d, ws, xq, xs, xg))
     assert same_bytes(d.t, ref) and same_bytes(xq.t, rq) and same_bytes(xs.t, rs) and xg.t.item() == rg.item()
+
+
+# the weight image and the linear that reads it: tile kernel (edge tiles, split along K), LDS-ring kernel (one and
+# several K ranges, 16- and 32-row activation stages), ragged N inside the last 128-row band
+@pytest.mark.parametrize("m,n,k", [(1, 1000, 1024), (12, 136, 2048), (32, 520, 512), (128, 1024, 4096), (96, 300, 2048),
+                                   (300, 130, 384), (20, 64, 128)])
+def test_prepacked_linear_stays_inside_image_workspace_and_output(m, n, k):
+    from ac4k_kernel_amd import _lib
+    L = _lib.load()
+    aq = ops().quantize(make_input((m, k), seed=m + 3).cuda(), 0, 1)
+    bq = ops().quantize(make_input((n, k), seed=n + 3, std=0.02).cuda(), 0, 1)
+    st = torch.cuda.current_stream().cuda_stream
+    nimg = L.ac4k_prepack_weight_nvfp4_bytes(n, k)
+    assert nimg == -(-n // 128) * (k // 128) * 9216
+    img = Window((nimg,), torch.uint8)
+    _lib.check(L.ac4k_prepack_weight_nvfp4(img.t.data_ptr(), bq[0].data_ptr(), bq[1].data_ptr(), n, k, st))
+    torch.cuda.synchronize()
+    assert img.intact()
+    assert same_bytes(img.t, ops().prepack_weight(bq[0], bq[1]))
+    nws = L.ac4k_linear_nvfp4_prepacked_workspace_bytes(m, n, k)
+    ref = ops().linear_prepacked(*aq, img.t, bq[2], n=n)
+    for shift in (0, 2):  # 256-byte aligned, and aligned to the element only
+        d, ws = Window((m, n), torch.bfloat16, shift=shift), Window((max(nws, 16),), torch.uint8)
+        _lib.check(L.ac4k_linear_nvfp4_prepacked(d.t.data_ptr(), 0, aq[0].data_ptr(), aq[1].data_ptr(), aq[2].data_ptr(),
+                                                 img.t.data_ptr(), bq[2].data_ptr(), None, 0, m, n, k,
+                                                 ws.t.data_ptr() if nws else None, nws, st))
+        torch.cuda.synchronize()
+        assert d.intact() and ws.intact() and img.intact(), (m, n, k, shift)
+        assert same_bytes(d.t, ref), (m, n, k, shift)
