@@ -290,6 +290,14 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+// Pins a wave-uniform pointer to scalar registers (the halves are taken as unsigned: readfirstlane
+// returns a signed int, and a sign-extended low half would corrupt the high one).
+__device__ __forceinline__ const uint8_t *uniform_ptr(const void *p) {
+  const uint64_t v = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
+}
+
 // LDS-DMA: global_load_lds with a scalar 64-bit base, a 32-bit lane offset and the LDS
 // destination of lane 0 in M0 (lane l lands at M0 + size * l).  Issued through inline asm so
 // that the compiler's wait-count insertion does not see these loads: with the builtin it puts
@@ -533,11 +541,6 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_tile256p_kernel(LinearArg
     }
   }
   const int64_t strideB = a.prepacked ? W_BLOCK_BYTES : P_ROW;  // bytes per stage along k
-  auto uniform_ptr = [](const void *p) {  // pin a wave-uniform pointer to scalar registers
-    const uint64_t v = (uint64_t)p;
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
-  };
   const uint8_t *baseA = uniform_ptr(a.A + tm * BM * kb + (int64_t)kt0 * P_ROW);
   const uint8_t *baseB = uniform_ptr(a.prepacked ? a.B + (int64_t)kt0 * W_BLOCK_BYTES : a.B + tn * BN * kb + (int64_t)kt0 * P_ROW);
   // scale transfers: piece g = swave * NS + p (past the last piece: the last piece again, which
@@ -1293,11 +1296,6 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream_kernel(Skin
     return p >= nst ? p - nst : p;
   };
 
-  auto uniform_ptr = [](const void *p) {  // pin a wave-uniform pointer to scalar registers
-    const uint64_t v = (uint64_t)p;
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
-  };
   // LDS holds row-major 128-byte rows (lane l of a transfer lands at 16 l: eight rows per transfer);
   // the eight 16-byte pieces of row r sit at positions piece ^ (r & 7), which spreads a fragment read
   // (one piece of each of 32 rows) over all LDS banks.  Unswizzled those reads fall on a quarter of the
@@ -1497,11 +1495,6 @@ __global__ __launch_bounds__(ST_THREADS, 1) void linear_nvfp4_stream64_kernel(Sk
   auto stage_of = [&](int step) {
     const int p = step + rot;
     return p >= nst ? p - nst : p;
-  };
-  auto uniform_ptr = [](const void *p) {  // pin a wave-uniform pointer to scalar registers
-    const uint64_t v = (uint64_t)p;
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
   };
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)stlds;
   // (1) weight rows swave * 8 + {0..7}, 128 B each, piece p of row r at position p ^ (r & 7)
