@@ -83,8 +83,8 @@ TIMELINE_LIB_PATH = os.path.join(PKG_DIR, "libac4k_nvfp4_timeline.so")
 
 def build_timeline(verbose: bool = True) -> str:
     """The same sources with the kernels' clock stamps compiled in (profiling aid, not the product):
-    load it with AC4K_NVFP4_LIB=<path> for `bench.py --workload quantize-timeline`."""
-    return build(force=True, verbose=verbose, extra_flags=["-DAC4K_ONEPASS_TIMELINE"], out=TIMELINE_LIB_PATH)
+    load it with AC4K_NVFP4_LIB=<path> for `bench.py --workload quantize-timeline` / `linear-timeline`."""
+    return build(force=True, verbose=verbose, extra_flags=["-DAC4K_ONEPASS_TIMELINE", "-DAC4K_LINEAR_TIMELINE"], out=TIMELINE_LIB_PATH)
 
 
 if __name__ == "__main__":

@@ -333,9 +333,10 @@ __device__ __forceinline__ uint32_t dword_of(const uint4 &v) {
   return S == 0 ? v.x : S == 1 ? v.y : S == 2 ? v.z : v.w;
 }
 
-// Build with -DAC4K_LINEAR_TIMELINE to record per workgroup the 100 MHz clock at kernel entry,
-// loop entry, loop exit and kernel exit plus the shader cycles spent in the loop (a profiling
-// aid; not compiled into the library).
+// Build with -DAC4K_LINEAR_TIMELINE (`build.py --timeline`) to record per workgroup the 100 MHz clock at
+// kernel entry, loop entry, loop exit and kernel exit plus the shader cycles spent in the loop of the
+// tile kernel and of the K-split-waves kernel; ac4k_debug_linear_timeline copies the stamps out
+// (a profiling aid; not compiled into the library).
 #ifdef AC4K_LINEAR_TIMELINE
 __device__ uint64_t g_linear_timeline[8192][6];
 #define AC4K_LTL(i, v)                                                     \
@@ -887,6 +888,407 @@ template <int D_DT, int BIAS_DT>
 static int launch_tile256p(const LinearArgs &a, hipStream_t st) {
   const SplitK one{nullptr, 1};
   return launch_tile_plan<D_DT, BIAS_DT>(a, tile_plan(a.M, a.N, a.K, false), one, st);
+}
+
+// ===========================================================================
+// Mid-sized M (33 .. 128): every weight byte is used by at most four 32-row activation fragments, so
+// the problem is bound by streaming the weights and by decode instructions, not by the MFMA rate, and
+// there are too few 256-wide tiles to fill the GPU.  Tile (32 MI) x (32 NJ) with ALL of M in one tile
+// (MI = 4, NJ = 2: 128 x 64) and the four waves of the workgroup splitting K, not the tile: a stage is
+// 256 k = four 64-chunks, wave w multiplies the whole tile over chunk w.  Every packed fragment of the
+// stage is then decoded exactly once per workgroup (the 2 x 2 wave grid of the tile kernel decodes each
+// one twice): (MI + NJ) * 8 decode instructions per MI * NJ MFMAs, 6 per MFMA for 128 x 64, with one
+// wave per SIMD.  Packed rows and scale dwords of a stage travel by LDS-DMA into a ring (128-byte rows,
+// 16-byte pieces at position piece ^ (row & 7), scales as [chunk][row] dwords); one workgroup barrier
+// per stage.  The four k parts of the tile meet through LDS at the end: wave w receives the sums of a
+// quarter of the tile from the other three, adds them in wave order, and stores its quarter
+// (times gsA * gsB, plus bias), or the raw fp32 sums of this K range when K is split over workgroups.
+// Requires K % 256 == 0 and 16-byte aligned operands and scale tensors.
+// ===========================================================================
+constexpr int KW_BK = 256;          // k per stage
+constexpr int KW_ROW = KW_BK / 2;   // packed bytes per row per stage
+
+template <int MI, int NJ>
+struct KWLayout {
+  static constexpr int BM = 32 * MI, BN = 32 * NJ;
+  static_assert(BM % 64 == 0 && BN % 64 == 0, "a scale transfer covers 64-row blocks");
+  static constexpr int OFF_W = 0;                         // BN weight rows, then BM activation rows
+  static constexpr int OFF_A = BN * KW_ROW;
+  static constexpr int OFF_SFW = OFF_A + BM * KW_ROW;     // scale dwords [4 chunks][BN rows]
+  static constexpr int OFF_SFA = OFF_SFW + 4 * BN * 4;    // [4 chunks][BM rows]
+  static constexpr int STAGE_BYTES = OFF_SFA + 4 * BM * 4;
+  static constexpr int PS = (159 * 1024) / STAGE_BYTES < 8 ? (159 * 1024) / STAGE_BYTES : 8;  // ring slots
+  static constexpr int LDS_BYTES = PS * STAGE_BYTES;      // the ring; one spare kilobyte follows it
+  static constexpr int LDS_ALLOC = LDS_BYTES + 1024;
+  static constexpr int NROW = (BM + BN) / 8 / 4;          // 8-row transfers per wave per stage
+  static constexpr int NSCW = BN / 64, NSCA = BM / 64;    // scale transfers per stage (1 KB each)
+  static constexpr int NPIECES = NROW + 1;                // every wave issues the same count
+  static constexpr int PPW = MI * NJ / 4;                 // 32 x 32 output blocks a wave finishes
+  static_assert((BM + BN) % 32 == 0 && NSCW + NSCA <= 4 && MI * NJ % 4 == 0, "transfers are dealt evenly to four waves");
+  static_assert(PS >= 3 && (PS - 2) * NPIECES <= 63, "the wait counts must fit the 6-bit counter");
+  static_assert(LDS_BYTES >= 16 * PPW * 4096, "the ring doubles as the exchange buffer of the four k parts");
+};
+
+template <int D_DT, int BIAS_DT, int MI, int NJ>
+__global__ __launch_bounds__(256, 1) void linear_nvfp4_ksplit_kernel(LinearArgs a, SplitK sk) {
+  using L = KWLayout<MI, NJ>;
+  constexpr int BM = L::BM, BN = L::BN, PS = L::PS, NP = L::NPIECES;
+  extern __shared__ __attribute__((aligned(16))) char kwlds[];
+  AC4K_LTL(0, wall_clock64());
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, r32 = lane & 31;
+  const int swave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t tiles_n = ceil_div(a.N, BN);
+  const int64_t tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+  const int64_t m0 = tm * BM, n0 = tn * BN;
+  const int nst_all = (int)(a.K / KW_BK);
+  const int s0 = (int)((int64_t)nst_all * blockIdx.y / sk.splits);
+  const int nst = (int)((int64_t)nst_all * (blockIdx.y + 1) / sk.splits) - s0;  // >= 1: splits <= stages
+  const int64_t kb = a.K >> 1;
+  // workgroup b starts at stage b % nst of its range and wraps around, so that the workgroups of a
+  // launch do not all ask for the same column of their rows at the same time (memory channels)
+  const int rot = (int)(blockIdx.x % (unsigned)nst);
+  const int last = nst - 1;
+  auto stage_of = [&](int step) {
+    const int p = (step < last ? step : last) + rot;
+    return p >= nst ? p - nst : p;
+  };
+
+  // --- this wave's transfers of a stage
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)kwlds;
+  // rows: transfer t = swave * NROW + q moves rows 8 t .. 8 t + 7 of the stage (weight rows first), lane l
+  // the piece of row l / 8 that belongs at position l % 8
+  uint32_t offR[L::NROW], ldsR[L::NROW];
+  const uint8_t *srcR[L::NROW];
+#pragma unroll
+  for (int q = 0; q < L::NROW; ++q) {
+    const int t = swave * L::NROW + q;
+    const bool isW = t < BN / 8;
+    const int loc = (isW ? t : t - BN / 8) * 8 + (lane >> 3);
+    const int64_t rows = isW ? a.N : a.M, first = isW ? n0 : m0;
+    const int64_t row = first + loc < rows ? loc : rows - 1 - first;  // rows past the matrix read its last row
+    offR[q] = (uint32_t)(row * kb + ((lane & 7) ^ (loc & 7)) * 16);
+    srcR[q] = uniform_ptr((isW ? a.B + n0 * kb : a.A + m0 * kb) + (int64_t)s0 * KW_ROW);
+    ldsR[q] = (uint32_t)__builtin_amdgcn_readfirstlane(t * 1024);
+  }
+  // scales: one transfer is 256 dwords of the [chunk][row] picture, a lane the four dwords of rows
+  // 4 g .. 4 g + 3 of one chunk (16 bytes of the scale tensor).  Transfers 0 .. NSCW - 1 are the weights',
+  // the others the activation's; a wave past the last transfer repeats the last one.
+  uint32_t offS, ldsS;
+  const uint8_t *srcS;
+  int64_t strideS;
+  {
+    const int t = swave < L::NSCW + L::NSCA ? swave : L::NSCW + L::NSCA - 1;
+    const bool isW = t < L::NSCW;
+    const int tt = isW ? t : t - L::NSCW;
+    const int bx = isW ? BN : BM;                         // rows of the operand's tile
+    const int cpt = 256 / bx;                             // chunks per transfer (4 or 2)
+    const int chunk = tt * cpt + lane / (bx / 4), grp = lane % (bx / 4);
+    const int64_t rows_p = isW ? a.Np : a.Mp, first = isW ? n0 : m0;
+    int64_t row = first + 4 * grp;
+    row = row + 4 <= rows_p ? row : rows_p - 4;           // groups past the padded rows read the last group
+    offS = (uint32_t)((chunk * rows_p + row) * 4);
+    strideS = 4 * rows_p * 4;                             // bytes per stage: four chunk planes
+    srcS = uniform_ptr(reinterpret_cast<const uint8_t *>(isW ? a.B_sf : a.A_sf) + s0 * strideS);
+    ldsS = (uint32_t)__builtin_amdgcn_readfirstlane((isW ? L::OFF_SFW : L::OFF_SFA) + tt * 1024);
+  }
+  // Transfer q of this wave's NPIECES for stage `st` into the ring slot at `base`.  Past the end of the range
+  // (`real` false) the loop keeps issuing, so that it stays free of branches and its wait counts stay fixed:
+  // those transfers read the last stage again (cache hits) and all land on one spare kilobyte behind the ring.
+  auto issue_piece = [&](uint32_t base, int st, int q, bool real) {
+    const uint32_t dst = real ? base : lds_base + (uint32_t)L::LDS_BYTES;
+    if (q < L::NROW)
+      dma16(uniform_ptr(srcR[q] + (int64_t)st * KW_ROW), offR[q], dst, real ? ldsR[q] : 0u);
+    else
+      dma16(uniform_ptr(srcS + st * strideS), offS, dst, real ? ldsS : 0u);
+  };
+  // the transfers of a stage are issued in four parts, one per 16-k sub-step, so that each one goes out
+  // in the shadow of an MFMA instead of holding the wave at the memory pipeline's door
+  auto issue_part = [&](uint32_t base, int st, int part, bool real) {
+#pragma unroll
+    for (int q = 0; q < NP; ++q)
+      if (q * 4 / NP == part) issue_piece(base, st, q, real);
+  };
+
+  // --- this wave's fragments of a stage: chunk swave; lane (r32, half) holds elements [32 half, 32 half + 32)
+  // of the chunk of one row per fragment (16 packed bytes) and the two block scales that go with them
+  struct Frags {
+    uint4 x[MI], w[NJ];
+    uint32_t xs[MI], ws[NJ];
+  };
+  const int piece = swave * 2 + half;
+  const int f_off = r32 * KW_ROW + ((piece ^ (r32 & 7)) * 16);  // rows 32 apart share the swizzle term
+  const int ws_off = L::OFF_SFW + (swave * BN + r32) * 4 + half * 2;
+  const int xs_off = L::OFF_SFA + (swave * BM + r32) * 4 + half * 2;
+  auto load_frags = [&](int slot) {
+    const char *st = kwlds + slot * L::STAGE_BYTES;
+    Frags f;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      f.w[j] = *reinterpret_cast<const uint4 *>(st + L::OFF_W + f_off + j * 32 * KW_ROW);
+      f.ws[j] = *reinterpret_cast<const uint16_t *>(st + ws_off + j * 128);
+    }
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      f.x[i] = *reinterpret_cast<const uint4 *>(st + L::OFF_A + f_off + i * 32 * KW_ROW);
+      f.xs[i] = *reinterpret_cast<const uint16_t *>(st + xs_off + i * 128);
+    }
+    return f;
+  };
+
+  f32x16 acc[MI][NJ];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  DecFrags<MI, NJ> D[2];
+  auto decode = [&](DecFrags<MI, NJ> &d, const Frags &f, auto S) {
+    constexpr int s = decltype(S)::value;
+#pragma unroll
+#ifdef KW_EXP_NO_DECODE
+    for (int j = 0; j < NJ; ++j) d.b[j] = __builtin_bit_cast(f16x8, f.w[j]);
+    for (int i = 0; i < MI; ++i) d.a[i] = __builtin_bit_cast(f16x8, f.x[i]);
+    return;
+#endif
+    for (int j = 0; j < NJ; ++j)
+      d.b[j] = decode_dword<(s >= 2)>(dword_of<s>(f.w[j]), __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.ws[j], 1.0f, false));
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+      d.a[i] = decode_dword<(s >= 2)>(dword_of<s>(f.x[i]), __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.xs[i], 1.0f, false));
+  };
+  auto mfma_all = [&](const DecFrags<MI, NJ> &d) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int jj = 0; jj < NJ; ++jj) {
+        const int j = (i & 1) ? NJ - 1 - jj : jj;  // neighbours share an operand
+#ifdef KW_EXP_NO_MFMA
+        asm volatile("" :: "v"(d.b[j]), "v"(d.a[i]));
+#else
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(d.b[j], d.a[i], acc[i][j], 0, 0, 0);  // D^T block
+#endif
+      }
+  };
+  auto interleave = [&]() {  // the decode of the next sub-step rides in the shadow of the MFMAs
+    constexpr int NMFMA = MI * NJ, NVALU = 8 * (MI + NJ) + (MI + NJ);
+    constexpr int PER = (NVALU + NMFMA - 1) / NMFMA;
+#pragma unroll
+    for (int g = 0; g < NMFMA; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, PER, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+
+  // prologue: the first PS stages in flight, stage 0 landed and its fragments in registers (every wave's,
+  // before slot 0 is refilled), then stage 1 landed
+#pragma unroll
+  for (int d = 0; d < PS; ++d) {
+#pragma unroll
+    for (int q = 0; q < NP; ++q) issue_piece(lds_base + d * L::STAGE_BYTES, stage_of(d), q, d <= last);
+  }
+  wait_vmcnt<(PS - 1) * NP>();
+  __syncthreads();
+  Frags F0 = load_frags(0), F1;
+  decode(D[0], F0, I0{});
+  wait_vmcnt<(PS - 2) * NP>();
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  int slot_cur = 0, slot_next = 1;
+#ifdef AC4K_LINEAR_TIMELINE
+  const uint64_t tl_c0 = __builtin_readcyclecounter();
+#endif
+  AC4K_LTL(1, wall_clock64());
+  // one stage: `cur` holds its fragments, `nxt` receives those of the next one (two named sets that swap
+  // roles, so that no register is copied between stages)
+  auto stage_step = [&](const Frags &cur, Frags &nxt, int s) {
+    // The slot of this stage is free (every wave had its fragments in registers before the previous
+    // barrier): stage s + PS goes there, if the range has one.
+    const bool more = s + PS <= last;
+    const int st_new = stage_of(s + PS);
+    const uint32_t base_new = lds_base + slot_cur * L::STAGE_BYTES;
+    // fragments of the next stage (it landed before the previous barrier) travel from LDS while this
+    // one is decoded and multiplied (past the range: a stage nobody uses)
+    nxt = load_frags(slot_next);
+    decode(D[1], cur, I1{});
+#ifndef KW_EXP_NO_DMA
+    issue_part(base_new, st_new, 0, more);
+#endif
+    mfma_all(D[0]);
+    interleave();
+    decode(D[0], cur, I2{});
+#ifndef KW_EXP_NO_DMA
+    issue_part(base_new, st_new, 1, more);
+#endif
+    mfma_all(D[1]);
+    interleave();
+    decode(D[1], cur, I3{});
+#ifndef KW_EXP_NO_DMA
+    issue_part(base_new, st_new, 2, more);
+#endif
+    mfma_all(D[0]);
+    interleave();
+    decode(D[0], nxt, I0{});
+#ifndef KW_EXP_NO_DMA
+    issue_part(base_new, st_new, 3, more);
+#endif
+    mfma_all(D[1]);
+    interleave();
+    wait_vmcnt<(PS - 2) * NP>();                        // own transfers of stage s + 2 have landed
+#ifndef KW_EXP_NO_LGKM
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // and the fragments of stage s + 1 are in registers
+#endif
+#ifndef KW_EXP_NO_BARRIER
+    __syncthreads();
+#endif
+    slot_cur = slot_next;
+    slot_next = slot_next + 1 == PS ? 0 : slot_next + 1;
+  };
+  for (int s = 0; s < nst; s += 2) {
+    stage_step(F0, F1, s);
+    if (s + 1 < nst) stage_step(F1, F0, s + 1);
+  }
+  AC4K_LTL(2, wall_clock64());
+#ifdef AC4K_LINEAR_TIMELINE
+  AC4K_LTL(4, __builtin_readcyclecounter() - tl_c0);
+#endif
+  // Every real transfer has landed (the last wait covered "stage last + 2") and every wave has passed the
+  // last barrier; what is still in flight lands on the spare kilobyte, so the ring can be reused.
+
+  // --- the four k parts meet: wave d finishes blocks p = d * PPW + q (i = p / NJ, j = p % NJ).
+  // acc[i][j]: lane l, element e <-> m = 32 i + (l & 31), n = 32 j + (e >> 2) * 8 + (l >> 5) * 4 + (e & 3)
+  constexpr int PPW = L::PPW;
+  float4 *xch = reinterpret_cast<float4 *>(kwlds);
+  auto xch_at = [&](int d, int src, int q, int g) { return xch + ((((d * 4 + src) * PPW + q) * 4 + g) * 64 + lane); };
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    if (d == swave) continue;
+#pragma unroll
+    for (int q = 0; q < PPW; ++q) {
+      const int p = d * PPW + q, i = p / NJ, j = p % NJ;
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        *xch_at(d, swave, q, g) = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+    }
+  }
+  __syncthreads();
+  const float scale = sk.partial ? 1.0f : (*a.A_gs) * (*a.B_gs);
+  using DE = Elem<D_DT>;
+  const bool vec_ok = (a.N & 3) == 0 && (((uintptr_t)a.D | (uintptr_t)sk.partial) & 15) == 0;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    if (d != swave) continue;
+#pragma unroll
+    for (int q = 0; q < PPW; ++q) {
+      const int p = d * PPW + q, i = p / NJ, j = p % NJ;
+      const int64_t m = m0 + 32 * i + r32;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+        for (int src = 0; src < 4; ++src) {  // always in wave order
+          const float4 t = src == d ? make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3])
+                                    : *xch_at(d, src, q, g);
+          if (src == 0) sum = t;
+          else { sum.x += t.x; sum.y += t.y; sum.z += t.z; sum.w += t.w; }
+        }
+        const int64_t n = n0 + 32 * j + g * 8 + half * 4;
+        if (m >= a.M || n >= a.N) continue;
+        if (sk.partial) {  // raw fp32 sums of this K range; the reduce kernel scales and converts
+          float *pp = sk.partial + ((int64_t)blockIdx.y * a.M + m) * a.N + n;
+          if (vec_ok && n + 3 < a.N) *reinterpret_cast<float4 *>(pp) = sum;
+          else {
+            const float v[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+              if (n + c < a.N) pp[c] = v[c];
+          }
+          continue;
+        }
+        float v[4] = {sum.x * scale, sum.y * scale, sum.z * scale, sum.w * scale};
+        if constexpr (BIAS_DT != BIAS_NONE) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) v[c] += n + c < a.N ? Elem<BIAS_DT>::load(a.bias, n + c) : 0.0f;
+        }
+        typename DE::T *dst = static_cast<typename DE::T *>(a.D) + m * a.N + n;
+        if (vec_ok && n + 3 < a.N) {
+          if constexpr (sizeof(typename DE::T) == 2)
+            *reinterpret_cast<uint2 *>(dst) = make_uint2(DE::cvt2(v[0], v[1]), DE::cvt2(v[2], v[3]));
+          else
+            *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+            if (n + c < a.N) dst[c] = DE::cvt(v[c]);
+        }
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may land in LDS after the workgroup has gone
+  AC4K_LTL(3, wall_clock64());
+}
+
+template <int D_DT, int BIAS_DT, int MI, int NJ>
+static int launch_ksplit_t(const LinearArgs &a, const SplitK &sk, hipStream_t st) {
+  using L = KWLayout<MI, NJ>;
+  auto *kern = linear_nvfp4_ksplit_kernel<D_DT, BIAS_DT, MI, NJ>;
+  static std::atomic<uint32_t> lds_ok{0};
+  if (int rc = allow_dynamic_lds(kern, lds_ok, L::LDS_ALLOC)) return rc;
+  const int64_t ntiles = ceil_div(a.M, L::BM) * ceil_div(a.N, L::BN);
+  hipLaunchKernelGGL(kern, dim3((unsigned)ntiles, (unsigned)sk.splits), dim3(256), L::LDS_ALLOC, st, a, sk);
+  return 0;
+}
+
+// Tile and K split of the K-split-waves kernel.
+struct KsplitPlan {
+  int mi, nj;
+  int splits;              // K ranges per tile; > 1 needs `partial_bytes` of fp32 scratch
+  int64_t partial_bytes;
+};
+
+// shapes the K-split-waves kernel takes (its pointer conditions are in ksplit_aligned)
+static bool ksplit_shape(int64_t M, int64_t N, int64_t K) {
+  return M > 32 && M <= 128 && N >= 64 && K >= KW_BK && K % KW_BK == 0 && (K >> 1) * 128 < (1ll << 31) && N < (1ll << 27) &&
+         g_forced_tile_plan.load(std::memory_order_relaxed) == 0;
+}
+static bool ksplit_aligned(const LinearArgs &a) {
+  return (((uintptr_t)a.A | (uintptr_t)a.B | (uintptr_t)a.A_sf | (uintptr_t)a.B_sf) & 15) == 0;
+}
+
+// All of M in one tile: 128 x 64 above 64 rows, 64 x 64 below (64 x 128 when even those fill the GPU).
+// Fewer than 192 tiles: as many K ranges as make about 256 workgroups, each at least two stages long.
+static KsplitPlan ksplit_plan(int64_t M, int64_t N, int64_t K, bool allow_split) {
+  KsplitPlan p{M <= 64 ? 2 : 4, 2, 1, 0};
+  if (M <= 64 && ceil_div(N, 128) >= 192) p.nj = 4;
+  const int64_t tiles = ceil_div(M, 32 * p.mi) * ceil_div(N, 32 * p.nj), stages = K / KW_BK;
+  int64_t splits = 1;
+  if (allow_split) {
+    if (const int f = g_forced_skinny_ks.load(std::memory_order_relaxed)) {  // forced length of a K range
+      splits = K / f;
+    } else if (tiles < 192) {
+      splits = 256 / tiles;
+      if (splits > stages / 2) splits = stages / 2;
+      if (splits > 32) splits = 32;
+    }
+    if (splits < 1) splits = 1;
+    if (splits > stages) splits = stages;
+  }
+  p.splits = (int)splits;
+  p.partial_bytes = splits > 1 ? splits * M * N * 4 : 0;
+  return p;
+}
+
+template <int D_DT, int BIAS_DT>
+static int launch_ksplit(const LinearArgs &a, const KsplitPlan &p, const SplitK &sk, hipStream_t st) {
+  if (p.mi == 4) return launch_ksplit_t<D_DT, BIAS_DT, 4, 2>(a, sk, st);
+  return p.nj == 4 ? launch_ksplit_t<D_DT, BIAS_DT, 2, 4>(a, sk, st) : launch_ksplit_t<D_DT, BIAS_DT, 2, 2>(a, sk, st);
 }
 
 // ===========================================================================
@@ -1758,6 +2160,8 @@ static bool packed_kernel_ok(const LinearArgs &a) {
 // 128x128 kernel, which has no condition beyond K % 64 == 0, takes everything else.
 template <int D_DT, int BIAS_DT>
 static int launch_linear(const LinearArgs &a, hipStream_t st) {
+  if (ksplit_shape(a.M, a.N, a.K) && ksplit_aligned(a))  // all of M in one tile, one K range (no scratch here)
+    return launch_ksplit<D_DT, BIAS_DT>(a, ksplit_plan(a.M, a.N, a.K, false), SplitK{nullptr, 1}, st);
   if (a.M > 32 && a.N >= 128 && packed_kernel_ok(a)) return launch_tile256p<D_DT, BIAS_DT>(a, st);
   const int64_t ntiles = ceil_div(a.M, T_BM) * ceil_div(a.N, T_BN);
   hipLaunchKernelGGL((linear_nvfp4_tile128_kernel<D_DT, BIAS_DT>), dim3((unsigned)ntiles), dim3(256), 0, st, a);
@@ -1817,28 +2221,44 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4(void *D,
 
 namespace ac4k {
 
-// Split-K for problems with too few output tiles to fill the GPU (32 < M, few tiles, long K):
-// the packed-LDS kernel runs `splits` K ranges per tile into fp32 partial buffers in the
-// workspace and skinny_reduce_kernel adds them.
-// shapes the workspace entry point splits along K: the packed-LDS kernel's shapes for which the
-// plan wants more than one K range
-static bool mid_plan(int64_t M, int64_t N, int64_t K, TilePlan &p) {
+// Split-K for problems with too few output tiles to fill the GPU (32 < M, few tiles, long K): the
+// K-split-waves kernel (M <= 128) or the packed-LDS tile kernel runs `splits` K ranges per tile into
+// fp32 partial buffers in the workspace and skinny_reduce_kernel adds them.
+struct MidPlan {
+  bool has_ksplit;   // the shape suits the K-split-waves kernel (taken when the pointers are aligned for it)
+  KsplitPlan kp;
+  TilePlan tp;       // what the tile kernel does with the shape otherwise
+  int64_t bytes;     // scratch that covers either choice
+};
+// shapes for which the workspace entry point has a use for scratch
+static bool mid_plan(int64_t M, int64_t N, int64_t K, MidPlan &p) {
   if (M <= 32 || N < 128 || K % P_BK != 0 || (K >> 1) * 256 >= (1ll << 31) || N >= (1ll << 27)) return false;
-  p = tile_plan(M, N, K, true);
-  return p.splits > 1;
+  p.tp = tile_plan(M, N, K, true);
+  p.has_ksplit = ksplit_shape(M, N, K);
+  p.kp = p.has_ksplit ? ksplit_plan(M, N, K, true) : KsplitPlan{0, 0, 1, 0};
+  p.bytes = p.tp.partial_bytes > p.kp.partial_bytes ? p.tp.partial_bytes : p.kp.partial_bytes;
+  return p.bytes > 0;
 }
 
 template <int D_DT, int BIAS_DT>
-static int launch_mid(const LinearArgs &a, const TilePlan &p, float *partial, hipStream_t st) {
-  const SplitK sk{partial, p.splits};
-  if (int rc = launch_tile_plan<D_DT, BIAS_DT>(a, p, sk, st)) return rc;
-  SkinnyArgs r{a.D, nullptr, nullptr, 0, nullptr, nullptr, a.A_gs, a.B_gs, a.bias, partial, a.M, a.N, a.K, a.Np, 0, p.splits};
-  launch_reduce<D_DT, BIAS_DT>(r, st);
+static int launch_mid(const LinearArgs &a, const MidPlan &p, float *partial, hipStream_t st) {
+  int splits;
+  if (p.has_ksplit && ksplit_aligned(a)) {
+    splits = p.kp.splits;
+    if (int rc = launch_ksplit<D_DT, BIAS_DT>(a, p.kp, SplitK{splits > 1 ? partial : nullptr, splits}, st)) return rc;
+  } else {
+    splits = p.tp.splits;
+    if (int rc = launch_tile_plan<D_DT, BIAS_DT>(a, p.tp, SplitK{splits > 1 ? partial : nullptr, splits}, st)) return rc;
+  }
+  if (splits > 1) {
+    SkinnyArgs r{a.D, nullptr, nullptr, 0, nullptr, nullptr, a.A_gs, a.B_gs, a.bias, partial, a.M, a.N, a.K, a.Np, 0, splits};
+    launch_reduce<D_DT, BIAS_DT>(r, st);
+  }
   return 0;
 }
 
 template <int D_DT>
-static int dispatch_mid_bias(const LinearArgs &a, const TilePlan &p, float *partial, int bias_dtype, hipStream_t st) {
+static int dispatch_mid_bias(const LinearArgs &a, const MidPlan &p, float *partial, int bias_dtype, hipStream_t st) {
   if (!a.bias) return launch_mid<D_DT, BIAS_NONE>(a, p, partial, st);
   switch (bias_dtype) {
     case AC4K_DTYPE_BF16: return launch_mid<D_DT, AC4K_DTYPE_BF16>(a, p, partial, st);
@@ -1848,7 +2268,7 @@ static int dispatch_mid_bias(const LinearArgs &a, const TilePlan &p, float *part
   return set_error("bias must be bfloat16, half or float (dtype tag %d)", bias_dtype);
 }
 
-static int dispatch_mid(const LinearArgs &a, const TilePlan &p, float *partial, int d_dtype, int bias_dtype,
+static int dispatch_mid(const LinearArgs &a, const MidPlan &p, float *partial, int d_dtype, int bias_dtype,
                         hipStream_t st) {
   switch (d_dtype) {
     case AC4K_DTYPE_BF16: return dispatch_mid_bias<AC4K_DTYPE_BF16>(a, p, partial, bias_dtype, st);
@@ -1907,8 +2327,8 @@ static int check_skinny(const SkinnyPlan &p, bool ok, const void *B, void *works
 extern "C" __attribute__((visibility("default"))) int64_t ac4k_linear_nvfp4_skinny_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   SkinnyPlan p;
   if (skinny_plan(M, N, K, p)) return p.partial_bytes > 0 ? p.partial_bytes : 256;  // non-zero selects this path
-  TilePlan mp;
-  if (mid_plan(M, N, K, mp)) return mp.partial_bytes;
+  MidPlan mp;
+  if (mid_plan(M, N, K, mp)) return mp.bytes;
   return 0;
 }
 
@@ -1920,12 +2340,12 @@ static int linear_skinny_impl(void *D, int d_dtype, const void *A, const void *A
                               int64_t N, int64_t K, void *workspace, int64_t workspace_bytes, hipStream_t st,
                               const char *what) {
   AC4K_REQUIRE(D && A && A_sf && A_gs && B && B_sf && B_gs, "null pointer argument");
-  TilePlan mp;
-  if (M > 32 && mid_plan(M, N, K, mp)) {  // few tiles, long K: split-K over the tile kernel
-    AC4K_REQUIRE((((uintptr_t)A | (uintptr_t)B) & 15) == 0, "A and B must be 16-byte aligned");
+  MidPlan mp;
+  if (M > 32 && mid_plan(M, N, K, mp)) {  // few tiles, long K: split-K
+    AC4K_REQUIRE((((uintptr_t)A | (uintptr_t)B) & 15) == 0 && (((uintptr_t)A_sf | (uintptr_t)B_sf) & 3) == 0,
+                 "A and B must be 16-byte aligned and the scale tensors 4-byte aligned");
     AC4K_REQUIRE(workspace && ((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
-    AC4K_REQUIRE(workspace_bytes >= mp.partial_bytes, "workspace too small: %lld bytes needed",
-                 (long long)mp.partial_bytes);
+    AC4K_REQUIRE(workspace_bytes >= mp.bytes, "workspace too small: %lld bytes needed", (long long)mp.bytes);
     LinearArgs la{D, static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B),
                   static_cast<const uint32_t *>(A_sf), static_cast<const uint32_t *>(B_sf), A_gs, B_gs, bias,
                   M, N, K, align_up(M, 16), align_up(N, 16)};
@@ -2099,7 +2519,8 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_prepacke
                 M, N, K, align_up(M, 16), align_up(N, 16), 1};
   int rc;
   if (p.tp.splits > 1) {
-    rc = dispatch_mid(la, p.tp, static_cast<float *>(workspace), d_dtype, bias_dtype, st);
+    rc = dispatch_mid(la, MidPlan{false, KsplitPlan{0, 0, 1, 0}, p.tp, p.tp.partial_bytes}, static_cast<float *>(workspace), d_dtype,
+                      bias_dtype, st);
   } else {
     switch (d_dtype) {
       case AC4K_DTYPE_BF16: rc = dispatch_prepacked_bias<AC4K_DTYPE_BF16>(la, p.tp, bias_dtype, st); break;
@@ -2149,3 +2570,14 @@ extern "C" __attribute__((visibility("default"))) int ac4k_set_linear_tuning(int
   ac4k::g_forced_skinny_ks.store(skinny_ks);
   return 0;
 }
+
+#ifdef AC4K_LINEAR_TIMELINE
+// Timeline build only: copies the per-workgroup stamps of the last tile / K-split-waves launch to host
+// memory ([8192][6]: 100 MHz ticks at kernel entry, loop entry, loop exit, kernel exit; shader cycles in
+// the loop; XCC and hardware id for the tile kernel).  Synchronises the device.
+extern "C" __attribute__((visibility("default"))) int ac4k_debug_linear_timeline(uint64_t *host_out) {
+  hipError_t e = hipDeviceSynchronize();
+  if (e == hipSuccess) e = hipMemcpyFromSymbol(host_out, HIP_SYMBOL(ac4k::g_linear_timeline), sizeof(uint64_t) * 8192 * 6);
+  return e == hipSuccess ? 0 : ac4k::set_error("ac4k_debug_linear_timeline: %s", hipGetErrorString(e));
+}
+#endif

@@ -255,6 +255,32 @@ def test_mid_m_shapes(m, n, k):
         run_case(m, n, k, bias_dtype=torch.bfloat16, o_dtype=torch.float32, seed=m + k + 2, wstd=0.02)
 
 
+# the K-split-waves kernel (32 < M <= 128, K % 256 == 0: all of M in one tile, the four waves split every
+# 256-k stage): its three tiles (128 x 64 above 64 rows, 64 x 64 below, 64 x 128 for very wide weights), ragged
+# M and N, K shorter and longer than the stage ring, one K range and forced ranges of one and two stages
+# (partial sums through the workspace), every output / bias type
+KSPLIT_SHAPES = [(33, 64, 256), (64, 200, 512), (65, 64, 1280), (100, 333, 2048), (128, 130, 3072), (127, 1000, 768),
+                 (40, 24600, 256), (128, 2048, 2560)]
+
+
+@pytest.mark.parametrize("m,n,k", KSPLIT_SHAPES)
+@pytest.mark.parametrize("ks", [0, 256, 512])
+def test_ksplit_kernel(m, n, k, ks, linear_tuning):
+    linear_tuning(skinny_ks=ks)
+    run_case(m, n, k, seed=m + k + ks, wstd=0.02)
+    run_case(m, n, k, bias_dtype=torch.float32, o_dtype=torch.float16, seed=m + k + 1, wstd=0.02)
+    run_case(m, n, k, bias_dtype=torch.bfloat16, o_dtype=torch.float32, seed=m + k + 2, wstd=0.02)
+
+
+def test_ksplit_kernel_against_c_oracle():
+    """fp32 output of the K-split-waves kernel against the C oracle's double sum: 1e-5, far inside the
+    1e-2 contract, so a dropped chunk, a swapped scale or a wrong k part would show."""
+    for (m, n, k) in [(128, 192, 1024), (50, 70, 512)]:
+        aq, bq = gpu_quant(make_input((m, k), seed=21)), gpu_quant(make_input((n, k), seed=22, std=0.02))
+        d = ops().linear(*aq, *bq, out=torch.empty((m, n), dtype=torch.float32, device="cuda")).cpu()
+        torch.testing.assert_close(d, C.linear_nvfp4(*cpu(aq), *cpu(bq)), atol=1e-5, rtol=1e-4)
+
+
 # every tile shape of the packed-LDS kernel (64*mi rows x 64*nj columns, its own LDS stage depth),
 # alone and split along K, forced through ac4k_set_linear_tuning; ragged M and N included
 TILE_PLANS = [(2, 1, 1), (2, 2, 1), (2, 4, 1), (4, 2, 1), (4, 4, 1), (2, 1, 3), (2, 2, 2), (2, 4, 5), (4, 2, 2), (4, 4, 4)]
