@@ -304,10 +304,17 @@ __device__ __forceinline__ const uint8_t *uniform_ptr(const void *p) {
 // s_waitcnt vmcnt(0) in front of every later LDS read, which serialises the prefetch.  The
 // kernel waits with explicit s_waitcnt vmcnt(..) before the barrier that publishes a stage.
 __device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t lds_stage, uint32_t lds_piece) {
+  // (wave-uniform by construction; the read keeps them in scalar registers when the compiler cannot tell)
+  lds_stage = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_stage);
+  lds_piece = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_piece);
+  sbase = uniform_ptr(sbase);
   asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
                :: "s"(lds_stage), "s"(lds_piece), "v"(voff), "s"(sbase) : "memory", "scc");
 }
 __device__ __forceinline__ void dma4(const void *sbase, uint32_t voff, uint32_t lds_stage, uint32_t lds_piece) {
+  lds_stage = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_stage);
+  lds_piece = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_piece);
+  sbase = uniform_ptr(sbase);
   asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3"
                :: "s"(lds_stage), "s"(lds_piece), "v"(voff), "s"(sbase) : "memory", "scc");
 }
@@ -341,7 +348,8 @@ __device__ __forceinline__ uint32_t dword_of(const uint4 &v) {
 __device__ uint64_t g_linear_timeline[8192][6];
 #define AC4K_LTL(i, v)                                                     \
   do {                                                                     \
-    if (threadIdx.x == 0 && blockIdx.x < 8192) g_linear_timeline[blockIdx.x][i] = (v); \
+    if (threadIdx.x == 0 && blockIdx.x + gridDim.x * blockIdx.y < 8192)      \
+      g_linear_timeline[blockIdx.x + gridDim.x * blockIdx.y][i] = (v);        \
   } while (0)
 #else
 #define AC4K_LTL(i, v)
@@ -917,9 +925,8 @@ struct KWLayout {
   static constexpr int OFF_SFW = OFF_A + BM * KW_ROW;     // scale dwords [4 chunks][BN rows]
   static constexpr int OFF_SFA = OFF_SFW + 4 * BN * 4;    // [4 chunks][BM rows]
   static constexpr int STAGE_BYTES = OFF_SFA + 4 * BM * 4;
-  static constexpr int PS = (159 * 1024) / STAGE_BYTES < 8 ? (159 * 1024) / STAGE_BYTES : 8;  // ring slots
-  static constexpr int LDS_BYTES = PS * STAGE_BYTES;      // the ring; one spare kilobyte follows it
-  static constexpr int LDS_ALLOC = LDS_BYTES + 1024;
+  static constexpr int PS = (160 * 1024) / STAGE_BYTES < 8 ? (160 * 1024) / STAGE_BYTES : 8;  // ring slots
+  static constexpr int LDS_BYTES = PS * STAGE_BYTES;
   static constexpr int NROW = (BM + BN) / 8 / 4;          // 8-row transfers per wave per stage
   static constexpr int NSCW = BN / 64, NSCA = BM / 64;    // scale transfers per stage (1 KB each)
   static constexpr int NPIECES = NROW + 1;                // every wave issues the same count
@@ -992,21 +999,19 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_ksplit_kernel(LinearArgs 
     ldsS = (uint32_t)__builtin_amdgcn_readfirstlane((isW ? L::OFF_SFW : L::OFF_SFA) + tt * 1024);
   }
   // Transfer q of this wave's NPIECES for stage `st` into the ring slot at `base`.  Past the end of the range
-  // (`real` false) the loop keeps issuing, so that it stays free of branches and its wait counts stay fixed:
-  // those transfers read the last stage again (cache hits) and all land on one spare kilobyte behind the ring.
-  auto issue_piece = [&](uint32_t base, int st, int q, bool real) {
-    const uint32_t dst = real ? base : lds_base + (uint32_t)L::LDS_BYTES;
+  // the loop keeps issuing, so that it stays free of branches and its wait counts stay fixed: those transfers
+  // read the last stage again (cache hits) into slots nobody reads any more.
+  auto issue_piece = [&](uint32_t base, int st, int q) {
     if (q < L::NROW)
-      dma16(uniform_ptr(srcR[q] + (int64_t)st * KW_ROW), offR[q], dst, real ? ldsR[q] : 0u);
+      dma16(srcR[q] + (int64_t)st * KW_ROW, offR[q], base, ldsR[q]);
     else
-      dma16(uniform_ptr(srcS + st * strideS), offS, dst, real ? ldsS : 0u);
+      dma16(srcS + st * strideS, offS, base, ldsS);
   };
-  // the transfers of a stage are issued in four parts, one per 16-k sub-step, so that each one goes out
-  // in the shadow of an MFMA instead of holding the wave at the memory pipeline's door
-  auto issue_part = [&](uint32_t base, int st, int part, bool real) {
+  // the transfers of a stage are issued in four parts, one per 16-k sub-step
+  auto issue_part = [&](uint32_t base, int st, int part) {
 #pragma unroll
     for (int q = 0; q < NP; ++q)
-      if (q * 4 / NP == part) issue_piece(base, st, q, real);
+      if (q * 4 / NP == part) issue_piece(base, st, q);
   };
 
   // --- this wave's fragments of a stage: chunk swave; lane (r32, half) holds elements [32 half, 32 half + 32)
@@ -1047,11 +1052,6 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_ksplit_kernel(LinearArgs 
   auto decode = [&](DecFrags<MI, NJ> &d, const Frags &f, auto S) {
     constexpr int s = decltype(S)::value;
 #pragma unroll
-#ifdef KW_EXP_NO_DECODE
-    for (int j = 0; j < NJ; ++j) d.b[j] = __builtin_bit_cast(f16x8, f.w[j]);
-    for (int i = 0; i < MI; ++i) d.a[i] = __builtin_bit_cast(f16x8, f.x[i]);
-    return;
-#endif
     for (int j = 0; j < NJ; ++j)
       d.b[j] = decode_dword<(s >= 2)>(dword_of<s>(f.w[j]), __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.ws[j], 1.0f, false));
 #pragma unroll
@@ -1064,11 +1064,7 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_ksplit_kernel(LinearArgs 
 #pragma unroll
       for (int jj = 0; jj < NJ; ++jj) {
         const int j = (i & 1) ? NJ - 1 - jj : jj;  // neighbours share an operand
-#ifdef KW_EXP_NO_MFMA
-        asm volatile("" :: "v"(d.b[j]), "v"(d.a[i]));
-#else
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(d.b[j], d.a[i], acc[i][j], 0, 0, 0);  // D^T block
-#endif
       }
   };
   auto interleave = [&]() {  // the decode of the next sub-step rides in the shadow of the MFMAs
@@ -1091,7 +1087,7 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_ksplit_kernel(LinearArgs 
 #pragma unroll
   for (int d = 0; d < PS; ++d) {
 #pragma unroll
-    for (int q = 0; q < NP; ++q) issue_piece(lds_base + d * L::STAGE_BYTES, stage_of(d), q, d <= last);
+    for (int q = 0; q < NP; ++q) issue_piece(lds_base + d * L::STAGE_BYTES, stage_of(d), q);
   }
   wait_vmcnt<(PS - 1) * NP>();
   __syncthreads();
@@ -1110,44 +1106,31 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_ksplit_kernel(LinearArgs 
   // roles, so that no register is copied between stages)
   auto stage_step = [&](const Frags &cur, Frags &nxt, int s) {
     // The slot of this stage is free (every wave had its fragments in registers before the previous
-    // barrier): stage s + PS goes there, if the range has one.
-    const bool more = s + PS <= last;
+    // barrier): stage s + PS goes there.
     const int st_new = stage_of(s + PS);
     const uint32_t base_new = lds_base + slot_cur * L::STAGE_BYTES;
     // fragments of the next stage (it landed before the previous barrier) travel from LDS while this
     // one is decoded and multiplied (past the range: a stage nobody uses)
     nxt = load_frags(slot_next);
     decode(D[1], cur, I1{});
-#ifndef KW_EXP_NO_DMA
-    issue_part(base_new, st_new, 0, more);
-#endif
+    issue_part(base_new, st_new, 0);
     mfma_all(D[0]);
     interleave();
     decode(D[0], cur, I2{});
-#ifndef KW_EXP_NO_DMA
-    issue_part(base_new, st_new, 1, more);
-#endif
+    issue_part(base_new, st_new, 1);
     mfma_all(D[1]);
     interleave();
     decode(D[1], cur, I3{});
-#ifndef KW_EXP_NO_DMA
-    issue_part(base_new, st_new, 2, more);
-#endif
+    issue_part(base_new, st_new, 2);
     mfma_all(D[0]);
     interleave();
     decode(D[0], nxt, I0{});
-#ifndef KW_EXP_NO_DMA
-    issue_part(base_new, st_new, 3, more);
-#endif
+    issue_part(base_new, st_new, 3);
     mfma_all(D[1]);
     interleave();
     wait_vmcnt<(PS - 2) * NP>();                        // own transfers of stage s + 2 have landed
-#ifndef KW_EXP_NO_LGKM
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // and the fragments of stage s + 1 are in registers
-#endif
-#ifndef KW_EXP_NO_BARRIER
     __syncthreads();
-#endif
     slot_cur = slot_next;
     slot_next = slot_next + 1 == PS ? 0 : slot_next + 1;
   };
@@ -1159,8 +1142,8 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_ksplit_kernel(LinearArgs 
 #ifdef AC4K_LINEAR_TIMELINE
   AC4K_LTL(4, __builtin_readcyclecounter() - tl_c0);
 #endif
-  // Every real transfer has landed (the last wait covered "stage last + 2") and every wave has passed the
-  // last barrier; what is still in flight lands on the spare kilobyte, so the ring can be reused.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-DMA may land after this point: the ring is reused
+  __syncthreads();
 
   // --- the four k parts meet: wave d finishes blocks p = d * PPW + q (i = p / NJ, j = p % NJ).
   // acc[i][j]: lane l, element e <-> m = 32 i + (l & 31), n = 32 j + (e >> 2) * 8 + (l >> 5) * 4 + (e & 3)
@@ -1231,7 +1214,6 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_ksplit_kernel(LinearArgs 
       }
     }
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may land in LDS after the workgroup has gone
   AC4K_LTL(3, wall_clock64());
 }
 
@@ -1240,9 +1222,9 @@ static int launch_ksplit_t(const LinearArgs &a, const SplitK &sk, hipStream_t st
   using L = KWLayout<MI, NJ>;
   auto *kern = linear_nvfp4_ksplit_kernel<D_DT, BIAS_DT, MI, NJ>;
   static std::atomic<uint32_t> lds_ok{0};
-  if (int rc = allow_dynamic_lds(kern, lds_ok, L::LDS_ALLOC)) return rc;
+  if (int rc = allow_dynamic_lds(kern, lds_ok, L::LDS_BYTES)) return rc;
   const int64_t ntiles = ceil_div(a.M, L::BM) * ceil_div(a.N, L::BN);
-  hipLaunchKernelGGL(kern, dim3((unsigned)ntiles, (unsigned)sk.splits), dim3(256), L::LDS_ALLOC, st, a, sk);
+  hipLaunchKernelGGL(kern, dim3((unsigned)ntiles, (unsigned)sk.splits), dim3(256), L::LDS_BYTES, st, a, sk);
   return 0;
 }
 
