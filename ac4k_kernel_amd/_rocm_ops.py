@@ -145,7 +145,7 @@ def _check_linear_operand(x, x_sf, x_gs, rows, name):
 
 
 def _skinny_scratch(device, M, N, K):
-    """Workspace tensor for the decode-sized linear, or None when the shape does not take that path."""
+    """Workspace tensor for the shapes that split K, or None when the shape needs no scratch."""
     nbytes = _L.ac4k_linear_nvfp4_skinny_workspace_bytes(M, N, K)
     if nbytes <= 0:
         return None
@@ -164,9 +164,9 @@ def _bias_args(bias, N):
 
 
 def linear_nvfp4(D, A, A_sf, A_global_scale, B, B_sf, B_global_scale, bias=None) -> None:
-    """Checks of linear_nvfp4.cu:759-805.  Shapes for which the library asks for scratch (decode-sized
-    M <= 32, or few output tiles with a long K) get a workspace tensor and the split-K kernels,
-    everything else the tile kernels."""
+    """Checks of linear_nvfp4.cu:759-805.  Shapes for which the library asks for scratch (too few output
+    tiles for the GPU, long K) get a workspace tensor and the split-K kernels; everything else goes to
+    the reference-shaped entry point, which allocates nothing and picks its kernel by shape."""
     _check(isinstance(D, torch.Tensor) and D.dim() == 2, "d must be a 2d matrix")
     _check(D.dtype in _DTYPE_TAG, "d must be bfloat16, half or float")
     _check(D.is_cuda and D.is_contiguous(), "d must be contiguous")
@@ -251,13 +251,13 @@ def linear_nvfp4_fused(D, X, X_q, X_sf, X_global_scale, B, B_sf, B_global_scale,
     _check(B.dim() == 2 and B.size(0) == N and B.size(1) == K // 2, "weight must be [N, K/2]")
     _check_linear_operand(B, B_sf, B_global_scale, N, "b")
     bias_ptr, bias_tag = _bias_args(bias, N)
-    scratch = _skinny_scratch(D.device, M, N, K)
-    if scratch is None:  # K % 256 != 0: the composition itself
+    if K % 256 != 0:  # no weight-streaming kernel: the composition itself
         quantize_nvfp4_with_global_scale(X_q, X_sf, X_global_scale, X, 0, 1, False, 2688.0)
         linear_nvfp4(D, X_q, X_sf, X_global_scale, B, B_sf, B_global_scale, bias)
         return
-    ws = scratch
+    ws = _skinny_scratch(D.device, M, N, K)  # None: one K range per tile, no scratch
     _lib.check(_L.ac4k_linear_nvfp4_fused_bf16(D.data_ptr(), _DTYPE_TAG[D.dtype], X.data_ptr(), X_q.data_ptr(),
                                                X_sf.data_ptr(), X_global_scale.data_ptr(), B.data_ptr(),
                                                B_sf.data_ptr(), B_global_scale.data_ptr(), bias_ptr, bias_tag,
-                                               M, N, K, ws.data_ptr(), ws.numel(), _stream()))
+                                               M, N, K, None if ws is None else ws.data_ptr(),
+                                               0 if ws is None else ws.numel(), _stream()))

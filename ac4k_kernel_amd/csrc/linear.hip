@@ -2050,7 +2050,7 @@ static void plan_lds_ring(int64_t M, int64_t N, int64_t K, SkinnyPlan &p, int ro
 // Hence: with 192 tiles of 128 rows and more, 128-row tiles from M = 8 on; otherwise 64-row tiles when
 // there are 192 of those, or from M = 8 on; the register kernel in the remaining cases.
 static bool skinny_plan(int64_t M, int64_t N, int64_t K, SkinnyPlan &p) {
-  if (M < 1 || M > 32 || K % SK_STEP != 0 || N < 1) return false;
+  if (M < 1 || M > 32 || K < SK_STEP || K % SK_STEP != 0 || N < 1) return false;
   const bool ring_ok = (K >> 1) * ST_BN < (1ll << 31) && N < (1ll << 27);  // 32-bit lane offsets
   int kind = g_forced_decode_kernel.load(std::memory_order_relaxed);
   if (kind == 0) {
@@ -2138,10 +2138,33 @@ static bool packed_kernel_ok(const LinearArgs &a) {
          a.N < (1ll << 27);
 }
 
-// M > 32 goes to the packed-operand tile kernel whenever its layout conditions hold; the
-// 128x128 kernel, which has no condition beyond K % 64 == 0, takes everything else.
+// Decode-sized shapes through the entry point that has no scratch: the plan of the workspace entry point
+// when it needs none (one K range), otherwise the LDS-ring kernel with one K range per tile - fewer
+// workgroups than the split plan, still the weights streamed once instead of the 128x128 tile kernel.
+static bool noscratch_skinny_plan(const LinearArgs &a, SkinnyPlan &p) {
+  if (!skinny_plan(a.M, a.N, a.K, p) || (((uintptr_t)a.A | (uintptr_t)a.B) & 15) != 0) return false;
+  if (p.partial_bytes == 0) return true;
+  if (!((a.K >> 1) * ST_BN < (1ll << 31) && a.N < (1ll << 27))) return false;  // the ring kernels' 32-bit lane offsets
+  p.kind = ceil_div(a.N, ST_BN) >= 192 ? DECODE_LDS_RING : DECODE_LDS_RING64;
+  p.groups = ceil_div(a.N, p.kind == DECODE_LDS_RING ? ST_BN : S6_BN);
+  p.ks_len = 0;
+  p.split_k = 1;
+  p.partial_bytes = 0;
+  p.lds_bytes = p.kind == DECODE_LDS_RING ? st_lds_bytes(a.M <= 16 ? 16 : 32) : S6_LDS_BYTES;
+  return true;
+}
+
+// Decode-sized M goes to the weight-streaming kernels, 32 < M <= 128 to the K-split-waves kernel, larger
+// M to the packed-operand tile kernel, each whenever its layout conditions hold; the 128x128 kernel,
+// which has no condition beyond K % 64 == 0, takes everything else.
 template <int D_DT, int BIAS_DT>
 static int launch_linear(const LinearArgs &a, hipStream_t st) {
+  SkinnyPlan sp;
+  if (noscratch_skinny_plan(a, sp)) {
+    const SkinnyArgs sa{a.D, a.A, reinterpret_cast<const uint8_t *>(a.A_sf), a.Mp, a.B, a.B_sf, a.A_gs, a.B_gs, a.bias, nullptr,
+                        a.M, a.N, a.K, a.Np, sp.ks_len, sp.split_k};
+    return launch_skinny<D_DT, BIAS_DT>(sa, sp, st);
+  }
   if (ksplit_shape(a.M, a.N, a.K) && ksplit_aligned(a))  // all of M in one tile, one K range (no scratch here)
     return launch_ksplit<D_DT, BIAS_DT>(a, ksplit_plan(a.M, a.N, a.K, false), SplitK{nullptr, 1}, st);
   if (a.M > 32 && a.N >= 128 && packed_kernel_ok(a)) return launch_tile256p<D_DT, BIAS_DT>(a, st);
@@ -2209,28 +2232,31 @@ namespace ac4k {
 struct MidPlan {
   bool has_ksplit;   // the shape suits the K-split-waves kernel (taken when the pointers are aligned for it)
   KsplitPlan kp;
-  TilePlan tp;       // what the tile kernel does with the shape otherwise
-  int64_t bytes;     // scratch that covers either choice
+  TilePlan tp;       // what the tile kernel does with the shape otherwise (given enough scratch)
+  int64_t bytes;     // scratch of the preferred choice
 };
-// shapes for which the workspace entry point has a use for scratch
+// shapes the workspace entry point takes with 32 < M
 static bool mid_plan(int64_t M, int64_t N, int64_t K, MidPlan &p) {
   if (M <= 32 || N < 128 || K % P_BK != 0 || (K >> 1) * 256 >= (1ll << 31) || N >= (1ll << 27)) return false;
   p.tp = tile_plan(M, N, K, true);
   p.has_ksplit = ksplit_shape(M, N, K);
   p.kp = p.has_ksplit ? ksplit_plan(M, N, K, true) : KsplitPlan{0, 0, 1, 0};
-  p.bytes = p.tp.partial_bytes > p.kp.partial_bytes ? p.tp.partial_bytes : p.kp.partial_bytes;
-  return p.bytes > 0;
+  p.bytes = p.has_ksplit ? p.kp.partial_bytes : p.tp.partial_bytes;
+  return p.has_ksplit || p.tp.splits > 1;
 }
 
+// `partial_bytes` of scratch at `partial` (possibly none): the K-split-waves kernel when the shape and the
+// pointers suit it, else the tile kernel, split along K when the scratch holds its partial sums
 template <int D_DT, int BIAS_DT>
-static int launch_mid(const LinearArgs &a, const MidPlan &p, float *partial, hipStream_t st) {
+static int launch_mid(const LinearArgs &a, const MidPlan &p, float *partial, int64_t partial_bytes, hipStream_t st) {
   int splits;
   if (p.has_ksplit && ksplit_aligned(a)) {
     splits = p.kp.splits;
     if (int rc = launch_ksplit<D_DT, BIAS_DT>(a, p.kp, SplitK{splits > 1 ? partial : nullptr, splits}, st)) return rc;
   } else {
-    splits = p.tp.splits;
-    if (int rc = launch_tile_plan<D_DT, BIAS_DT>(a, p.tp, SplitK{splits > 1 ? partial : nullptr, splits}, st)) return rc;
+    const TilePlan tp = p.tp.partial_bytes <= partial_bytes ? p.tp : tile_plan(a.M, a.N, a.K, false);
+    splits = tp.splits;
+    if (int rc = launch_tile_plan<D_DT, BIAS_DT>(a, tp, SplitK{splits > 1 ? partial : nullptr, splits}, st)) return rc;
   }
   if (splits > 1) {
     SkinnyArgs r{a.D, nullptr, nullptr, 0, nullptr, nullptr, a.A_gs, a.B_gs, a.bias, partial, a.M, a.N, a.K, a.Np, 0, splits};
@@ -2240,22 +2266,23 @@ static int launch_mid(const LinearArgs &a, const MidPlan &p, float *partial, hip
 }
 
 template <int D_DT>
-static int dispatch_mid_bias(const LinearArgs &a, const MidPlan &p, float *partial, int bias_dtype, hipStream_t st) {
-  if (!a.bias) return launch_mid<D_DT, BIAS_NONE>(a, p, partial, st);
+static int dispatch_mid_bias(const LinearArgs &a, const MidPlan &p, float *partial, int64_t partial_bytes, int bias_dtype,
+                             hipStream_t st) {
+  if (!a.bias) return launch_mid<D_DT, BIAS_NONE>(a, p, partial, partial_bytes, st);
   switch (bias_dtype) {
-    case AC4K_DTYPE_BF16: return launch_mid<D_DT, AC4K_DTYPE_BF16>(a, p, partial, st);
-    case AC4K_DTYPE_FP16: return launch_mid<D_DT, AC4K_DTYPE_FP16>(a, p, partial, st);
-    case AC4K_DTYPE_FP32: return launch_mid<D_DT, AC4K_DTYPE_FP32>(a, p, partial, st);
+    case AC4K_DTYPE_BF16: return launch_mid<D_DT, AC4K_DTYPE_BF16>(a, p, partial, partial_bytes, st);
+    case AC4K_DTYPE_FP16: return launch_mid<D_DT, AC4K_DTYPE_FP16>(a, p, partial, partial_bytes, st);
+    case AC4K_DTYPE_FP32: return launch_mid<D_DT, AC4K_DTYPE_FP32>(a, p, partial, partial_bytes, st);
   }
   return set_error("bias must be bfloat16, half or float (dtype tag %d)", bias_dtype);
 }
 
-static int dispatch_mid(const LinearArgs &a, const MidPlan &p, float *partial, int d_dtype, int bias_dtype,
-                        hipStream_t st) {
+static int dispatch_mid(const LinearArgs &a, const MidPlan &p, float *partial, int64_t partial_bytes, int d_dtype,
+                        int bias_dtype, hipStream_t st) {
   switch (d_dtype) {
-    case AC4K_DTYPE_BF16: return dispatch_mid_bias<AC4K_DTYPE_BF16>(a, p, partial, bias_dtype, st);
-    case AC4K_DTYPE_FP16: return dispatch_mid_bias<AC4K_DTYPE_FP16>(a, p, partial, bias_dtype, st);
-    case AC4K_DTYPE_FP32: return dispatch_mid_bias<AC4K_DTYPE_FP32>(a, p, partial, bias_dtype, st);
+    case AC4K_DTYPE_BF16: return dispatch_mid_bias<AC4K_DTYPE_BF16>(a, p, partial, partial_bytes, bias_dtype, st);
+    case AC4K_DTYPE_FP16: return dispatch_mid_bias<AC4K_DTYPE_FP16>(a, p, partial, partial_bytes, bias_dtype, st);
+    case AC4K_DTYPE_FP32: return dispatch_mid_bias<AC4K_DTYPE_FP32>(a, p, partial, partial_bytes, bias_dtype, st);
   }
   return set_error("d must be bfloat16, half or float (dtype tag %d)", d_dtype);
 }
@@ -2297,10 +2324,12 @@ static int run_skinny(void *D, int d_dtype, const void *Aq, const void *A_sf, co
 }
 
 static int check_skinny(const SkinnyPlan &p, bool ok, const void *B, void *workspace, int64_t workspace_bytes) {
-  AC4K_REQUIRE(ok, "no workspace-assisted path for this shape (ac4k_linear_nvfp4_skinny_workspace_bytes returns 0)");
+  AC4K_REQUIRE(ok, "no workspace-assisted path for this shape: decode-sized shapes need 1 <= M <= 32 and K a multiple of 256");
   AC4K_REQUIRE(((uintptr_t)B & 15) == 0, "weights must be 16-byte aligned");
-  AC4K_REQUIRE(workspace && ((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
-  AC4K_REQUIRE(workspace_bytes >= p.partial_bytes, "workspace too small: %lld bytes needed", (long long)p.partial_bytes);
+  if (p.partial_bytes > 0) {  // one K range per tile needs no scratch
+    AC4K_REQUIRE(workspace && ((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
+    AC4K_REQUIRE(workspace_bytes >= p.partial_bytes, "workspace too small: %lld bytes needed", (long long)p.partial_bytes);
+  }
   return 0;
 }
 
@@ -2308,7 +2337,7 @@ static int check_skinny(const SkinnyPlan &p, bool ok, const void *B, void *works
 
 extern "C" __attribute__((visibility("default"))) int64_t ac4k_linear_nvfp4_skinny_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   SkinnyPlan p;
-  if (skinny_plan(M, N, K, p)) return p.partial_bytes > 0 ? p.partial_bytes : 256;  // non-zero selects this path
+  if (skinny_plan(M, N, K, p)) return p.partial_bytes;
   MidPlan mp;
   if (mid_plan(M, N, K, mp)) return mp.bytes;
   return 0;
@@ -2322,16 +2351,21 @@ static int linear_skinny_impl(void *D, int d_dtype, const void *A, const void *A
                               int64_t N, int64_t K, void *workspace, int64_t workspace_bytes, hipStream_t st,
                               const char *what) {
   AC4K_REQUIRE(D && A && A_sf && A_gs && B && B_sf && B_gs, "null pointer argument");
+  AC4K_REQUIRE(M >= 1 && N >= 1 && K >= 1, "M, N, K must be positive (M=%lld N=%lld K=%lld)", (long long)M,
+               (long long)N, (long long)K);
   MidPlan mp;
   if (M > 32 && mid_plan(M, N, K, mp)) {  // few tiles, long K: split-K
     AC4K_REQUIRE((((uintptr_t)A | (uintptr_t)B) & 15) == 0 && (((uintptr_t)A_sf | (uintptr_t)B_sf) & 3) == 0,
                  "A and B must be 16-byte aligned and the scale tensors 4-byte aligned");
-    AC4K_REQUIRE(workspace && ((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
-    AC4K_REQUIRE(workspace_bytes >= mp.bytes, "workspace too small: %lld bytes needed", (long long)mp.bytes);
+    if (mp.bytes > 0) {  // one K range per tile needs no scratch
+      AC4K_REQUIRE(workspace && ((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
+      AC4K_REQUIRE(workspace_bytes >= mp.bytes, "workspace too small: %lld bytes needed", (long long)mp.bytes);
+    }
     LinearArgs la{D, static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B),
                   static_cast<const uint32_t *>(A_sf), static_cast<const uint32_t *>(B_sf), A_gs, B_gs, bias,
                   M, N, K, align_up(M, 16), align_up(N, 16)};
-    if (int rc = dispatch_mid(la, mp, static_cast<float *>(workspace), d_dtype, bias_dtype, st)) return rc;
+    if (int rc = dispatch_mid(la, mp, static_cast<float *>(workspace), workspace ? workspace_bytes : 0, d_dtype, bias_dtype, st))
+      return rc;
     return check_launch(what);
   }
   SkinnyPlan p;
@@ -2384,8 +2418,9 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_skinny_s
                                                const float *A_gs, const void *B, const void *B_sf,
                                                const float *B_gs, const void *bias, int bias_dtype, int64_t M,
                                                int64_t N, int64_t K, ac4k_stream_t stream) {
+  AC4K_REQUIRE(M >= 1 && N >= 1 && K >= 1, "M, N, K must be positive (M=%lld N=%lld K=%lld)", (long long)M,
+               (long long)N, (long long)K);
   const int64_t need = ac4k_linear_nvfp4_skinny_workspace_bytes(M, N, K);
-  AC4K_REQUIRE(need > 0, "no workspace-assisted path for this shape (ac4k_linear_nvfp4_skinny_workspace_bytes returns 0)");
   AC4K_REQUIRE(need <= STATIC_SCRATCH_BYTES,
                "shape needs %lld bytes of scratch, the static scratch holds %lld: use ac4k_linear_nvfp4_skinny with a "
                "workspace of the caller",
@@ -2501,8 +2536,8 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_prepacke
                 M, N, K, align_up(M, 16), align_up(N, 16), 1};
   int rc;
   if (p.tp.splits > 1) {
-    rc = dispatch_mid(la, MidPlan{false, KsplitPlan{0, 0, 1, 0}, p.tp, p.tp.partial_bytes}, static_cast<float *>(workspace), d_dtype,
-                      bias_dtype, st);
+    rc = dispatch_mid(la, MidPlan{false, KsplitPlan{0, 0, 1, 0}, p.tp, p.tp.partial_bytes}, static_cast<float *>(workspace),
+                      workspace_bytes, d_dtype, bias_dtype, st);
   } else {
     switch (d_dtype) {
       case AC4K_DTYPE_BF16: rc = dispatch_prepacked_bias<AC4K_DTYPE_BF16>(la, p.tp, bias_dtype, st); break;
@@ -2521,6 +2556,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_fused_bf
                                             void *workspace, int64_t workspace_bytes, ac4k_stream_t stream) {
   AC4K_REQUIRE(D && X && X_q && X_sf && X_gs && B && B_sf && B_gs, "null pointer argument");
   AC4K_REQUIRE(M >= 1 && M <= 32, "the fused skinny linear takes 1 <= M <= 32 (got %lld)", (long long)M);
+  AC4K_REQUIRE(N >= 1 && K >= 1, "N and K must be positive (N=%lld K=%lld)", (long long)N, (long long)K);
   SkinnyPlan p;
   const bool ok = skinny_plan(M, N, K, p);
   if (int rc = check_skinny(p, ok, B, workspace, workspace_bytes)) return rc;
@@ -2535,20 +2571,18 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_fused_bf
 
 extern "C" __attribute__((visibility("default"))) int ac4k_set_linear_tuning(int mi, int nj, int splits, int skinny_ks,
                                                                           int decode_kernel) {
+  // every argument is checked before any is stored: a rejected call changes nothing
   AC4K_REQUIRE(decode_kernel >= 0 && decode_kernel <= 3,
                "decode_kernel must be 0 (by shape), 1 (register kernel), 2 (LDS-ring kernel) or 3 (LDS-ring kernel with "
                "64-row tiles) (got %d)", decode_kernel);
-  ac4k::g_forced_decode_kernel.store(decode_kernel);
-  if (mi == 0 && nj == 0 && splits == 0) {
-    ac4k::g_forced_tile_plan.store(0);
-  } else {
-    AC4K_REQUIRE((mi == 2 || mi == 4) && (nj == 1 || nj == 2 || nj == 4) && !(mi == 4 && nj == 1) && splits >= 1 &&
-                     splits <= 0xffff,
-                 "tile plan must be mi in {2,4}, nj in {1,2,4} (not 4,1), 1 <= splits (got %d,%d,%d)", mi, nj, splits);
-    ac4k::g_forced_tile_plan.store((uint32_t)mi | ((uint32_t)nj << 8) | ((uint32_t)splits << 16));
-  }
+  const bool no_plan = mi == 0 && nj == 0 && splits == 0;
+  AC4K_REQUIRE(no_plan || ((mi == 2 || mi == 4) && (nj == 1 || nj == 2 || nj == 4) && !(mi == 4 && nj == 1) && splits >= 1 &&
+                           splits <= 0xffff),
+               "tile plan must be mi in {2,4}, nj in {1,2,4} (not 4,1), 1 <= splits (got %d,%d,%d)", mi, nj, splits);
   AC4K_REQUIRE(skinny_ks >= 0 && skinny_ks % 256 == 0, "skinny_ks must be 0 (automatic) or a multiple of 256 (got %d)",
                skinny_ks);
+  ac4k::g_forced_decode_kernel.store(decode_kernel);
+  ac4k::g_forced_tile_plan.store(no_plan ? 0u : (uint32_t)mi | ((uint32_t)nj << 8) | ((uint32_t)splits << 16));
   ac4k::g_forced_skinny_ks.store(skinny_ks);
   return 0;
 }

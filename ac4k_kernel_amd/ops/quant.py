@@ -27,20 +27,29 @@ _SCALE_MAX_CACHE = {}
 
 def _scale_max_tensor(value, dtype, device):
     """0-dim device scalar for scale_max.  The reference builds one with torch.full on every call
-    (quant.py:130-135,177-182); here it is kept per (value, dtype, device) once it exists with its
-    value in place.  While the current stream records into a graph nothing is cached: a tensor made
-    there lives in the graph's memory pool and is only filled when the graph replays."""
+    (quant.py:130-135,177-182); here it is kept per (value, dtype, device).  The fill runs on the stream of
+    the first call; until it has completed, calls order their own stream behind it with an event (no host
+    synchronisation anywhere).  While the current stream records into a graph nothing is cached: a tensor
+    made there lives in the graph's memory pool and is only filled when the graph replays."""
     key = (value, dtype, device)
-    t = _SCALE_MAX_CACHE.get(key)
-    if t is not None:
+    hit = _SCALE_MAX_CACHE.get(key)
+    if hit is not None:
+        t, ev = hit
+        if ev is not None:
+            if ev.query():
+                _SCALE_MAX_CACHE[key] = (t, None)  # filled: nothing to order against any more
+            elif not torch.cuda.is_current_stream_capturing():
+                torch.cuda.current_stream(device).wait_event(ev)
+            else:  # a capture must not depend on work outside it: a scalar of the graph's own
+                return torch.full([], value, dtype=dtype, device=device)
         return t
     t = torch.full([], value, dtype=dtype, device=device)
-    if device.type == "cuda" and torch.cuda.is_current_stream_capturing():
-        return t
-    # the fill ran on the current stream; later calls may come from other streams, so the cached
-    # tensor is handed out only after the fill has completed
-    torch.cuda.current_stream(device).synchronize() if device.type == "cuda" else None
-    _SCALE_MAX_CACHE[key] = t
+    if device.type != "cuda":
+        _SCALE_MAX_CACHE[key] = (t, None)
+    elif not torch.cuda.is_current_stream_capturing():
+        ev = torch.cuda.Event()
+        ev.record(torch.cuda.current_stream(device))
+        _SCALE_MAX_CACHE[key] = (t, ev)
     return t
 
 

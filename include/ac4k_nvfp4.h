@@ -114,19 +114,22 @@ int ac4k_linear_nvfp4(void *D, int d_dtype, const void *A, const void *A_sf, con
                       const void *B, const void *B_sf, const float *B_gs, const void *bias,
                       int bias_dtype, int64_t M, int64_t N, int64_t K, ac4k_stream_t stream);
 
-/* Linear for shapes that need device scratch to run well: same contract as ac4k_linear_nvfp4
+/* Linear for shapes that need device scratch to run at their best: same contract as ac4k_linear_nvfp4
  * (lib/cuda/sm120/linear_nvfp4.cu:753-901; the reference runs every shape through its one
  * 128x128 tile kernel).  Two families:
  *   - decode-sized, 1 <= M <= 32 and K % 256 == 0: kernels that stream the weights once (into
  *     registers for small M, through an LDS ring with 128- or 64-row tiles for larger M and for
- *     weights of 12288 to 24575 rows); the workspace receives the fp32 partial sums
+ *     weights of 12225 to 24448 rows); the workspace receives the fp32 partial sums
  *     of their K ranges when they split K; A and B 16-byte aligned;
- *   - 32 < M with too few output tiles to fill the GPU and K % 128 == 0: split-K over the tile
- *     kernel (tile shape and number of K ranges chosen by a cost model); the workspace receives
- *     the fp32 partial sums; A and B 16-byte aligned.
+ *   - 32 < M with too few output tiles to fill the GPU and K % 128 == 0: split-K (the K-split-waves
+ *     kernel up to M = 128 when K % 256 == 0, the tile kernel otherwise; tile shape and number of K
+ *     ranges chosen by a cost model); the workspace receives the fp32 partial sums; A and B 16-byte
+ *     aligned.
  * `workspace` = ac4k_linear_nvfp4_skinny_workspace_bytes(M,N,K) bytes of device memory, 256-byte
- * aligned, contents irrelevant.  The size function returns 0 for shapes that gain nothing from
- * scratch; those go to ac4k_linear_nvfp4. */
+ * aligned, contents irrelevant.  The size function returns 0 for shapes that need no scratch: those
+ * go to ac4k_linear_nvfp4, which runs the same kernels with one K range (a decode-sized shape with
+ * 0 bytes may also come here, with a NULL workspace).  ac4k_linear_nvfp4 takes every shape; where this
+ * entry point would split K it runs one K range per tile instead: fewer workgroups, same contract. */
 int64_t ac4k_linear_nvfp4_skinny_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int ac4k_linear_nvfp4_skinny(void *D, int d_dtype, const void *A, const void *A_sf, const float *A_gs,
                              const void *B, const void *B_sf, const float *B_gs, const void *bias,

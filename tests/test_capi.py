@@ -66,8 +66,22 @@ def test_argument_rejection_without_gpu():
     assert lib.ac4k_set_linear_tuning(4, 1, 1, 0, 0) != 0 and b"tile plan" in lib.ac4k_last_error()
     assert lib.ac4k_set_linear_tuning(0, 0, 0, 100, 0) != 0 and b"skinny_ks" in lib.ac4k_last_error()
     assert lib.ac4k_set_linear_tuning(0, 0, 0, 0, 4) != 0 and b"decode_kernel" in lib.ac4k_last_error()
+    # a rejected call leaves every earlier field alone: here the decode kernel choice is valid, skinny_ks is not,
+    # and the plan of a decode-sized shape stays what the library picks on its own
+    before = lib.ac4k_linear_nvfp4_skinny_workspace_bytes(4, 4096, 14336)
+    assert lib.ac4k_set_linear_tuning(0, 0, 0, 100, 2) != 0
+    assert lib.ac4k_linear_nvfp4_skinny_workspace_bytes(4, 4096, 14336) == before
     assert lib.ac4k_set_linear_tuning(0, 0, 0, 0, 0) == 0
     assert lib.ac4k_debug_last_quantize_path() in (0, 1, 2, 3)
+    # K <= 0 never selects a weight-streaming plan, and the workspace entry points say what is wrong
+    assert lib.ac4k_linear_nvfp4_skinny_workspace_bytes(8, 1024, 0) == 0
+    assert lib.ac4k_linear_nvfp4_skinny_workspace_bytes(8, 1024, -256) == 0
+    rc = lib.ac4k_linear_nvfp4_skinny(one, 0, one, one, one, one, one, one, None, 0, 8, 1024, 0, one, 256, None)
+    assert rc != 0 and b"positive" in lib.ac4k_last_error()
+    rc = lib.ac4k_linear_nvfp4_skinny_static(one, 0, one, one, one, one, one, one, None, 0, 8, 1024, -256, None)
+    assert rc != 0 and b"positive" in lib.ac4k_last_error()
+    rc = lib.ac4k_linear_nvfp4_fused_bf16(one, 0, one, one, one, one, one, one, one, None, 0, 8, 1024, 0, one, 256, None)
+    assert rc != 0 and b"positive" in lib.ac4k_last_error()
     rc = lib.ac4k_linear_nvfp4_fused_bf16(one, 0, one, one, one, one, one, one, one, None, 0, 64, 4, 64, one, 0, None)
     assert rc != 0 and b"1 <= M <= 32" in lib.ac4k_last_error()
     with pytest.raises(RuntimeError):

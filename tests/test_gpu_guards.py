@@ -131,10 +131,9 @@ def test_workspace_linear_stays_inside_workspace_and_output(m, n, k, kind, linea
     linear_tuning(decode_kernel=kind)
     aq = ops().quantize(make_input((m, k), seed=m).cuda(), 0, 1)
     bq = ops().quantize(make_input((n, k), seed=n, std=0.02).cuda(), 0, 1)
-    nbytes = L.ac4k_linear_nvfp4_skinny_workspace_bytes(m, n, k)
-    assert nbytes > 0
+    nbytes = L.ac4k_linear_nvfp4_skinny_workspace_bytes(m, n, k)  # 0: one K range per tile, nothing to write there
     ref = ops().linear(*aq, *bq)
-    d, ws = Window((m, n), torch.bfloat16), Window((nbytes,), torch.uint8)
+    d, ws = Window((m, n), torch.bfloat16), Window((max(nbytes, 256),), torch.uint8)
     _lib.check(L.ac4k_linear_nvfp4_skinny(d.t.data_ptr(), 0, aq[0].data_ptr(), aq[1].data_ptr(), aq[2].data_ptr(),
                                           bq[0].data_ptr(), bq[1].data_ptr(), bq[2].data_ptr(), None, 0, m, n, k,
                                           ws.t.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream))
@@ -151,7 +150,7 @@ def test_fused_linear_stays_inside_every_buffer(m, n, k):
     bq = ops().quantize(make_input((n, k), seed=n, std=0.02).cuda(), 0, 1)
     ref, (rq, rs, rg) = ops().fused_linear(x, *bq, return_quantized=True)
     nbytes = L.ac4k_linear_nvfp4_skinny_workspace_bytes(m, n, k)
-    d, ws = Window((m, n), torch.bfloat16), Window((nbytes,), torch.uint8)
+    d, ws = Window((m, n), torch.bfloat16), Window((max(nbytes, 256),), torch.uint8)
     xq, xs, xg = Window(rq.shape, torch.uint8), Window(rs.shape, torch.float8_e4m3fn), Window((), torch.float32)
     _lib.check(L.ac4k_linear_nvfp4_fused_bf16(d.t.data_ptr(), 0, x.data_ptr(), xq.t.data_ptr(), xs.t.data_ptr(),
                                               xg.t.data_ptr(), bq[0].data_ptr(), bq[1].data_ptr(), bq[2].data_ptr(),

@@ -320,6 +320,47 @@ def test_mid_m_workspace_entry_matches_plain_entry():
     assert b"workspace too small" in L.ac4k_last_error()
 
 
+@pytest.mark.parametrize("m,n,k", [(8, 28672, 8192), (32, 28672, 8192), (16, 14336, 4096), (1, 256, 256), (40, 14336, 4096)])
+def test_reference_shaped_entry_runs_the_fast_kernels(m, n, k):
+    """ac4k_linear_nvfp4 has the reference's signature (no workspace).  Where the plan of the workspace entry
+    point needs no scratch (one K range per tile) both entry points run the same kernel: equal outputs,
+    bit for bit, through the C ABI."""
+    from ac4k_kernel_amd import _lib
+    L = _lib.load()
+    assert L.ac4k_linear_nvfp4_skinny_workspace_bytes(m, n, k) == 0
+    aq, bq = gpu_quant(make_input((m, k), seed=m)), gpu_quant(make_input((n, k), seed=n, std=0.02))
+    bias = make_input((1, n), seed=9).float().cuda()
+    d1 = torch.full((m, n), 7.0, dtype=torch.bfloat16, device="cuda")
+    d2 = torch.full((m, n), -7.0, dtype=torch.bfloat16, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    args = (aq[0].data_ptr(), aq[1].data_ptr(), aq[2].data_ptr(), bq[0].data_ptr(), bq[1].data_ptr(), bq[2].data_ptr(),
+            bias.data_ptr(), 2, m, n, k)
+    _lib.check(L.ac4k_linear_nvfp4(d1.data_ptr(), 0, *args, st))
+    if m <= 32:
+        _lib.check(L.ac4k_linear_nvfp4_skinny(d2.data_ptr(), 0, *args, None, 0, st))
+        assert torch.equal(d1, d2)
+    full = (gpu_dequant(aq, m) @ gpu_dequant(bq, n).t() + bias).to(torch.bfloat16)
+    torch.testing.assert_close(d1, full, atol=ATOL, rtol=RTOL)
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 4096, 14336), (4, 1024, 4096), (1, 4096, 2048), (32, 384, 3584)])
+def test_reference_shaped_entry_without_scratch_on_split_shapes(m, n, k):
+    """Shapes whose best plan splits K: ac4k_linear_nvfp4 streams the weights with one K range per tile
+    instead (no scratch), within the contract; the workspace entry point gives the split result."""
+    from ac4k_kernel_amd import _lib
+    L = _lib.load()
+    assert L.ac4k_linear_nvfp4_skinny_workspace_bytes(m, n, k) > 0
+    aq, bq = gpu_quant(make_input((m, k), seed=m)), gpu_quant(make_input((n, k), seed=n, std=0.02))
+    d1 = torch.full((m, n), 7.0, dtype=torch.float32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    _lib.check(L.ac4k_linear_nvfp4(d1.data_ptr(), 2, aq[0].data_ptr(), aq[1].data_ptr(), aq[2].data_ptr(),
+                                   bq[0].data_ptr(), bq[1].data_ptr(), bq[2].data_ptr(), None, 0, m, n, k, st))
+    d2 = ops().linear(*aq, *bq, out=torch.empty((m, n), dtype=torch.float32, device="cuda"))
+    torch.testing.assert_close(d1, d2, atol=1e-5, rtol=1e-4)
+    full = gpu_dequant(aq, m) @ gpu_dequant(bq, n).t()
+    torch.testing.assert_close(d1, full, atol=ATOL, rtol=RTOL)
+
+
 def test_graph_replay_of_linear_paths():
     """Captured calls of the tile kernel, the split-K path and the fused decode path replay correctly
     with eager work in between (no host-side state is baked into a launch)."""
