@@ -450,3 +450,60 @@ def test_error_behaviour():
     with pytest.raises(RuntimeError):                    # global scale must be 0-dim
         o.quantize_nvfp4(torch.empty((8, 32), dtype=torch.uint8, device="cuda"),
                          torch.empty((1, 16, 4), dtype=torch.float8_e4m3fn, device="cuda"), x, gs, 0, 1, False)
+
+
+def test_reference_bandwidth_shape_at_full_size():
+    """The reference's own quantize shape (test/test_quantize_bandwidth.py:37-38: (1, 75600, 40, 128), nvfp4 with
+    cross 1 / reduce 3 and with cross 3 / reduce 1 swizzled) and the fp8 call of its attention wrapper
+    (python/ac4k_kernel/ops/attention.py:169-174: cross 3, reduce the token dim, swizzled, max_scale 2.25), at full
+    size: 387 M elements.  The global scale must equal the oracle's formula on the tensor's maximum (taken with
+    a torch reduction), and bands of the outputs - the first, a middle one and the last, which holds the padding -
+    must equal the oracle's bytes; the oracle quantizes the band with the global scale given, which is exact
+    because blocks, chunks and swizzle groups do not reach across a band that starts on a multiple of 64."""
+    shape = (1, 75600, 40, 128)
+    g = torch.Generator(device="cuda").manual_seed(20)
+    x = torch.empty(shape, dtype=torch.float32, device="cuda").normal_(generator=g)
+    x = torch.where(torch.rand(shape, device="cuda", generator=g) < 0.001, x * 20.0, x).to(torch.bfloat16)
+    amax = x.abs().max().reshape(1).cpu()
+    gs_ref = T.global_scale(amax)
+
+    # cross 1 (tokens), reduce 3 (head dim): bands of 64 tokens
+    out, sf, gs = ops().quantize(x, 1, 3)
+    assert gs.item() == gs_ref.item()
+    assert list(out.shape) == [1, 40, 75600, 64] and list(sf.shape) == [1, 40, 2, 75600, 4]
+    for t0 in (0, 37792, 75600 - 64):
+        eo, es, _ = T.quantize_nvfp4(x[:, t0:t0 + 64].cpu(), 1, 3, False, gs=gs_ref)
+        assert torch.equal(out[:, :, t0:t0 + 64].cpu(), eo), f"nvfp4 cross 1: bytes of tokens {t0}.. differ"
+        assert torch.equal(sf[:, :, :, t0:t0 + 64].cpu().view(torch.uint8), es), f"nvfp4 cross 1: scales of tokens {t0}.. differ"
+    del out, sf
+
+    # cross 3 (head dim), reduce 1 (tokens), swizzled: bands of 256 tokens along the reduce dim; the last band
+    # ends in the 48 padding positions (75600 -> 75648)
+    out, sf, gs = ops().quantize(x, 3, 1, swizzle=True)
+    assert gs.item() == gs_ref.item()
+    assert list(out.shape) == [1, 40, 128, 75648 // 2] and list(sf.shape) == [1, 40, 1182, 128, 4]
+    for k0 in (0, 37760, 75648 - 256):
+        eo, es, _ = T.quantize_nvfp4(x[:, k0:k0 + 256].cpu(), 3, 1, True, gs=gs_ref)
+        assert torch.equal(out[..., k0 // 2:(k0 + 256) // 2].cpu(), eo), f"nvfp4 cross 3: bytes of tokens {k0}.. differ"
+        assert torch.equal(sf[:, :, k0 // 64:(k0 + 256) // 64].cpu().view(torch.uint8), es), f"nvfp4 cross 3: scales of tokens {k0}.. differ"
+    del out, sf
+
+    # fp8, cross 3, reduce 1, swizzled, max_scale 2.25: a row is (head, d) over all 75600 tokens, so whole heads are compared
+    out, sf = ops().quantize(x, 3, 1, max_scale=2.25, precision="fp8e4m3", swizzle=True)
+    assert list(out.shape) == [1, 40, 128, 75600] and list(sf.shape) == [1, 40, 128]
+    for h in (0, 17, 39):
+        eo, es = T.quantize_fp8(x[:, :, h:h + 1].cpu(), 3, 1, 2.25, True)
+        assert torch.equal(out[:, h:h + 1].cpu().view(torch.uint8), eo), f"fp8 cross 3: bytes of head {h} differ"
+        assert torch.equal(sf[:, h:h + 1].cpu(), es), f"fp8 cross 3: scales of head {h} differ"
+    del out, sf
+
+    # fp8 and int8, cross 1, reduce 3: rows are tokens, bands of 64 tokens
+    for prec, orc in (("fp8e4m3", T.quantize_fp8), ("int8", T.quantize_int8)):
+        out, sf = ops().quantize(x, 1, 3, precision=prec)
+        for t0 in (0, 37792, 75600 - 64):
+            eo, es = orc(x[:, t0:t0 + 64].cpu(), 1, 3)
+            got = out[:, :, t0:t0 + 64].cpu()
+            assert torch.equal(got.view(torch.uint8) if prec == "fp8e4m3" else got, eo), f"{prec} cross 1: tokens {t0}.. differ"
+            assert torch.equal(sf[:, :, t0:t0 + 64].cpu(), es)
+        del out, sf
+    torch.cuda.empty_cache()
