@@ -22,6 +22,7 @@ SIGNATURES = {
     "ac4k_global_scale_bf16": (_int, [_vp, _vp, _i64, _f32, _vp]),
     "ac4k_set_quantize_sync_timeout_us": (None, [_i64]),
     "ac4k_debug_last_quantize_path": (_int, []),
+    "ac4k_debug_quantize_timeouts_seen": (_i64, []),
     "ac4k_quantize_nvfp4": (_int, [_vp, _vp, _vp, _vp] + [_i64] * 8 + [_int, _vp]),
     "ac4k_quantize_nvfp4_bf16": (_int, [_vp, _vp, _vp, _vp] + [_i64] * 8 + [_int, _f32, _vp]),
     "ac4k_quantize_fp8": (_int, [_vp, _vp, _vp, _vp] + [_i64] * 8 + [_int, _vp]),

@@ -11,6 +11,8 @@
 //
 // All kernels are bandwidth-bound: the row-major paths move 16 bytes per lane per load,
 // reduce amax inside the wavefront with DPP, and store packed words.
+#include <string.h>
+
 #include <atomic>
 #include <mutex>
 #include <type_traits>
@@ -332,7 +334,8 @@ __device__ __forceinline__ uint32_t onepass_share_absmax(const uint4 *__restrict
 template <int NV>
 __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
     uint32_t *__restrict__ out, uint32_t *__restrict__ sf, const uint4 *__restrict__ in, float *__restrict__ gs_out,
-    OnePassGeom g, int slot, uint32_t tag, float max_scale, uint64_t timeout_ticks) {
+    OnePassGeom g, int slot, uint32_t tag, float max_scale, uint64_t timeout_ticks, uint32_t *__restrict__ report,
+    uint32_t seq) {
   constexpr int GS = NV < 8 ? NV : 8;  // segments per group
   constexpr int NG = NV / GS;          // groups per workgroup
   constexpr uint32_t GC = GS * 128;    // chunks per group
@@ -436,6 +439,9 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
   __syncthreads();
   uint32_t gm = gmax_s;
   if (helping_s) {  // workgroup-uniform: the wait ran out
+    // tell the host (a word of mapped host memory per slot, read without synchronising before a later call):
+    // launch number `seq` did not find its peers resident
+    if (tid == 0 && report && timeout_ticks) __hip_atomic_store(report + slot, seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     const uint8_t *miss = reinterpret_cast<const uint8_t *>(miss4);
     uint32_t m = 0;
 #pragma unroll 1
@@ -1036,12 +1042,49 @@ struct OnePassSlot {
   hipStream_t st;
   uint64_t last_use;  // 0 = never used
   uint32_t tag;
+  uint32_t seq;       // launches of the single-launch kernel on this slot
+  uint32_t seen;      // highest launch number whose timeout report has been acted on
+  uint32_t backoff;   // calls that still take the three-launch path
 };
 static std::mutex g_slot_mutex;
 static OnePassSlot g_slots[OP_MAX_DEVICES][OP_SLOTS];
 static uint64_t g_slot_clock = 0;
 
-static bool onepass_slot(hipStream_t st, int *slot, uint32_t *tag) {
+// Timeout reports: one word per slot in mapped host memory, written by a workgroup of the single-launch
+// kernel whose grid wait ran out (its peers were not all resident: the GPU is shared with other kernels),
+// read here before a later call on that slot - no synchronisation, no copy.  A stream that has just seen a
+// timeout takes the three-launch path for the next ONEPASS_BACKOFF_CALLS calls, whose cost does not depend
+// on what else runs, and then tries the single launch again.  The page is allocated once per GPU on the
+// first call that needs it (not while any stream of the thread captures); without it nothing is reported
+// and every call keeps the single launch, which stays correct.
+constexpr uint32_t ONEPASS_BACKOFF_CALLS = 64;
+struct TimeoutReports {
+  uint32_t *host = nullptr, *dev = nullptr;
+  bool tried = false;
+};
+static TimeoutReports g_reports[OP_MAX_DEVICES];
+static std::atomic<uint64_t> g_timeouts_seen{0};
+
+static uint32_t *timeout_reports(int dev) {  // called with g_slot_mutex held
+  TimeoutReports &r = g_reports[dev];
+  if (!r.tried) {
+    r.tried = true;
+    void *h = nullptr, *d = nullptr;
+    if (hipHostMalloc(&h, OP_SLOTS * sizeof(uint32_t), hipHostMallocMapped) == hipSuccess && h &&
+        hipHostGetDevicePointer(&d, h, 0) == hipSuccess && d) {
+      memset(h, 0, OP_SLOTS * sizeof(uint32_t));
+      r.host = static_cast<uint32_t *>(h);
+      r.dev = static_cast<uint32_t *>(d);
+    } else {
+      (void)hipGetLastError();
+      if (h) (void)hipHostFree(h);
+    }
+  }
+  return r.dev;
+}
+
+// -> false: take the three-launch path (no slot for this device, or the stream is backing off after a timeout)
+static bool onepass_slot(hipStream_t st, int *slot, uint32_t *tag, uint32_t **report, uint32_t *seq) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= OP_MAX_DEVICES) return false;
   std::lock_guard<std::mutex> lock(g_slot_mutex);
@@ -1057,11 +1100,27 @@ static bool onepass_slot(hipStream_t st, int *slot, uint32_t *tag) {
   if (pick < 0) {
     pick = oldest;
     t[pick].st = st;
+    t[pick].backoff = 0;
   }
   t[pick].last_use = ++g_slot_clock;
+  *report = timeout_reports(dev);
+  if (g_reports[dev].host) {
+    const uint32_t reported = *reinterpret_cast<volatile uint32_t *>(g_reports[dev].host + pick);
+    if ((int32_t)(reported - t[pick].seen) > 0) {  // a launch since the last look ran out of time
+      t[pick].seen = reported;
+      t[pick].backoff = ONEPASS_BACKOFF_CALLS;
+      g_timeouts_seen.fetch_add(1, std::memory_order_relaxed);
+    }
+  }
+  if (t[pick].backoff > 0) {
+    --t[pick].backoff;
+    return false;
+  }
   t[pick].tag = t[pick].tag % 0xffffu + 1;  // 1 .. 65535
+  t[pick].seq += 1;
   *slot = pick;
   *tag = t[pick].tag;
+  *seq = t[pick].seq;
   return true;
 }
 
@@ -1113,11 +1172,16 @@ static int device_cu_count() {
   return n;
 }
 
+struct OnePassLaunch {
+  int slot;
+  uint32_t tag, seq;
+  uint32_t *report;
+};
 template <int NV>
 static void launch_onepass(uint32_t *out, uint32_t *sf, const uint4 *in, float *gs, const OnePassGeom &g, int nwg,
-                           int slot, uint32_t tag, float max_scale, uint64_t ticks, hipStream_t st) {
-  hipLaunchKernelGGL((quantize_nvfp4_onepass_kernel<NV>), dim3(nwg), dim3(OP_THREADS), 0, st, out, sf, in, gs, g, slot,
-                     tag, max_scale, ticks);
+                           const OnePassLaunch &l, float max_scale, uint64_t ticks, hipStream_t st) {
+  hipLaunchKernelGGL((quantize_nvfp4_onepass_kernel<NV>), dim3(nwg), dim3(OP_THREADS), 0, st, out, sf, in, gs, g, l.slot,
+                     l.tag, max_scale, ticks, l.report, l.seq);
 }
 
 // Up to 16 segments (256 KB) every workgroup can afford to read the whole tensor for its maximum:
@@ -1159,22 +1223,21 @@ static int try_quantize_nvfp4_onepass(void *out, void *sf, float *gs, const void
     return QPATH_SMALL;
   }
   if (stream_is_capturing(st)) return QPATH_NONE;
-  int slot = -1;
-  uint32_t tag = 0;
-  if (!onepass_slot(st, &slot, &tag)) return QPATH_NONE;
+  OnePassLaunch l{-1, 0, 0, nullptr};
+  if (!onepass_slot(st, &l.slot, &l.tag, &l.report, &l.seq)) return QPATH_NONE;
   const int64_t per_wg = ceil_div(chunks, (int64_t)nwg * 128);  // 16 KB segments per workgroup
   uint32_t *o = static_cast<uint32_t *>(out), *s = static_cast<uint32_t *>(sf);
   const uint4 *x = static_cast<const uint4 *>(in);
   if (per_wg <= 1)
-    launch_onepass<1>(o, s, x, gs, g, nwg, slot, tag, max_scale, (uint64_t)ticks, st);
+    launch_onepass<1>(o, s, x, gs, g, nwg, l, max_scale, (uint64_t)ticks, st);
   else if (per_wg <= 2)
-    launch_onepass<2>(o, s, x, gs, g, nwg, slot, tag, max_scale, (uint64_t)ticks, st);
+    launch_onepass<2>(o, s, x, gs, g, nwg, l, max_scale, (uint64_t)ticks, st);
   else if (per_wg <= 4)
-    launch_onepass<4>(o, s, x, gs, g, nwg, slot, tag, max_scale, (uint64_t)ticks, st);
+    launch_onepass<4>(o, s, x, gs, g, nwg, l, max_scale, (uint64_t)ticks, st);
   else if (per_wg <= 8)
-    launch_onepass<8>(o, s, x, gs, g, nwg, slot, tag, max_scale, (uint64_t)ticks, st);
+    launch_onepass<8>(o, s, x, gs, g, nwg, l, max_scale, (uint64_t)ticks, st);
   else
-    launch_onepass<16>(o, s, x, gs, g, nwg, slot, tag, max_scale, (uint64_t)ticks, st);
+    launch_onepass<16>(o, s, x, gs, g, nwg, l, max_scale, (uint64_t)ticks, st);
   return QPATH_ONEPASS;
 }
 
@@ -1258,6 +1321,10 @@ extern "C" __attribute__((visibility("default"))) int ac4k_quantize_nvfp4_bf16(v
 }
 
 extern "C" __attribute__((visibility("default"))) int ac4k_debug_last_quantize_path(void) { return ac4k::g_last_quantize_path; }
+
+extern "C" __attribute__((visibility("default"))) int64_t ac4k_debug_quantize_timeouts_seen(void) {
+  return (int64_t)ac4k::g_timeouts_seen.load(std::memory_order_relaxed);
+}
 
 namespace ac4k {
 
@@ -1357,6 +1424,10 @@ extern "C" __attribute__((visibility("default"))) int ac4k_quantize_int8(void *o
 
 extern "C" __attribute__((visibility("default"))) void ac4k_set_quantize_sync_timeout_us(int64_t us) {
   ac4k::g_sync_timeout_ticks.store(us < 0 ? -1 : us * 100);
+  // a new bound starts with a clean slate: no stream keeps backing off because of waits under the old one
+  std::lock_guard<std::mutex> lock(ac4k::g_slot_mutex);
+  for (auto &dev : ac4k::g_slots)
+    for (auto &slot : dev) slot.backoff = 0;
 }
 
 #ifdef AC4K_ONEPASS_TIMELINE

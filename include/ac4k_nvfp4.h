@@ -83,14 +83,24 @@ int ac4k_quantize_nvfp4_bf16(void *out, void *sf, float *global_scale, const voi
  * single-launch kernel wait for each other's maxima for at most this many microseconds (default
  * 200).  A workgroup whose wait runs out - its peers were not all resident because other kernels
  * hold the GPU - recomputes the missing maxima from memory itself and finishes: slower, same bits.
- * 0 = look once, then recompute (used by the tests); a negative value switches the single-launch
- * kernel off (three launches, as under graph capture). */
+ * 0 = look once, then recompute (used by the tests; not reported as a timeout); a negative value
+ * switches the single-launch kernel off (three launches, as under graph capture).  A wait that runs
+ * out costs the bound plus a second read of the missing workgroups' shares, so a stream on which it
+ * happened takes the three-launch path for its next 64 calls (see ac4k_debug_quantize_timeouts_seen);
+ * setting the bound also ends every such back-off. */
 void ac4k_set_quantize_sync_timeout_us(int64_t us);
 
 /* Introspection for tests (no counterpart in the reference): which path the last
  * ac4k_quantize_nvfp4_bf16 call of the calling host thread took: 0 none yet, 1 small one-launch
  * kernel, 2 single-launch kernel with the grid wait, 3 fill + maxima + quantize. */
 int ac4k_debug_last_quantize_path(void);
+
+/* Introspection (no counterpart in the reference): how many times this process has noticed that a launch of
+ * the single-launch kernel ran out of waiting time.  The kernel reports it through a word of mapped host
+ * memory; the next ac4k_quantize_nvfp4_bf16 call on that stream reads the word (no synchronisation) and
+ * sends that stream's next 64 calls down the three-launch path, whose cost does not depend on what else
+ * runs on the GPU; then the single launch is tried again. */
+int64_t ac4k_debug_quantize_timeouts_seen(void);
 
 /* Replaces ac4k::quantize_fp8 (lib/cuda/sm120/quantize_fp8.cu:192-290).
  * out: e4m3 [d0,d1,R,align_up(K,16)];  sf: fp32 [d0,d1,align_up(R,16)] = amax/scale_max.

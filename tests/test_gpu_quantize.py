@@ -507,3 +507,66 @@ def test_reference_bandwidth_shape_at_full_size():
             assert torch.equal(sf[:, :, t0:t0 + 64].cpu(), es)
         del out, sf
     torch.cuda.empty_cache()
+
+
+def test_single_launch_timeout_is_reported_and_backs_off():
+    """A grid wait that runs out is reported to the host through mapped memory; the next calls on that stream
+    take the three-launch path (64 of them), then the single launch is tried again.  The condition is forced
+    from the host with a bound of 1 us, which the launch stagger alone exceeds: every kernel still exits
+    normally, and every output equals the oracle's."""
+    from ac4k_kernel_amd import _lib
+    L = _lib.load()
+    x = make_input((4096, 2048), seed=77, outliers=True)
+    exp = T.quantize_nvfp4(x, 0, 1, False)
+    xg = x.cuda()
+
+    def run():
+        out, sf, gs = ops().quantize(xg, 0, 1)
+        path = L.ac4k_debug_last_quantize_path()
+        torch.cuda.synchronize()  # the report of this launch has reached host memory before the next call looks
+        assert torch.equal(out.cpu(), exp[0]) and torch.equal(sf.cpu().view(torch.uint8), exp[1]) and gs.item() == exp[2].item()
+        return path
+
+    try:
+        L.ac4k_set_quantize_sync_timeout_us(1)
+        seen0 = L.ac4k_debug_quantize_timeouts_seen()
+        assert run() == PATH_ONEPASS          # the wait runs out inside this launch: same bits, slower
+        paths = [run() for _ in range(64)]    # the report is read before the first of these
+        assert L.ac4k_debug_quantize_timeouts_seen() == seen0 + 1
+        assert paths == [PATH_TWO_KERNEL] * 64
+        assert run() == PATH_ONEPASS          # back-off over: the single launch is tried again
+        L.ac4k_set_quantize_sync_timeout_us(200)  # ends the back-off that the last launch caused
+        assert run() == PATH_ONEPASS
+        assert run() == PATH_ONEPASS          # an idle GPU: nothing to report
+    finally:
+        L.ac4k_set_quantize_sync_timeout_us(200)
+
+
+def test_quantize_next_to_a_long_gemm_on_another_stream():
+    """The GPU shared with the 8192^3 linear running back to back on a second stream: the quantizer's workgroups
+    are not all resident at once, waits may run out, calls may back off to the three-launch path - whatever
+    happens, every call returns the oracle's bytes."""
+    from ac4k_kernel_amd import _lib
+    L = _lib.load()
+    L.ac4k_set_quantize_sync_timeout_us(200)
+    aq = ops().quantize(make_input((8192, 8192), seed=1).cuda(), 0, 1)
+    bq = ops().quantize(make_input((8192, 8192), seed=2).cuda(), 0, 1)
+    d = torch.empty((8192, 8192), dtype=torch.bfloat16, device="cuda")
+    x = make_input((8192, 4096), seed=78, outliers=True)
+    exp = T.quantize_nvfp4(x, 0, 1, False)
+    xg = x.cuda()
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    results, paths = [], []
+    with torch.cuda.stream(s1):
+        for _ in range(12):
+            ops().linear(*aq, *bq, out=d)
+    with torch.cuda.stream(s2):
+        for _ in range(12):
+            results.append(ops().quantize(xg, 0, 1))
+            paths.append(L.ac4k_debug_last_quantize_path())
+    torch.cuda.synchronize()
+    for out, sf, gs in results:
+        assert torch.equal(out.cpu(), exp[0]) and torch.equal(sf.cpu().view(torch.uint8), exp[1]) and gs.item() == exp[2].item()
+    assert set(paths) <= {PATH_ONEPASS, PATH_TWO_KERNEL}
+    L.ac4k_set_quantize_sync_timeout_us(200)
