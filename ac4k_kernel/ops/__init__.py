@@ -1,13 +1,15 @@
 """`ac4k_kernel.ops`: the NVFP4-path operators under the reference's module path
-(python/ac4k_kernel/ops/__init__.py:5-26), re-exported from `ac4k_kernel_amd.ops`."""
+(python/ac4k_kernel/ops/__init__.py:5-26), re-exported from `ac4k_kernel_amd.ops`; `attention` takes
+precision="nvfp4" only."""
 import sys as _sys
 
-from ac4k_kernel_amd.ops import (fused_linear, linear, linear_nvfp4, quantize, quantize_fp8, quantize_int8,
-                                 quantize_nvfp4)
+from ac4k_kernel_amd.ops import (attention, fused_linear, linear, linear_nvfp4, mha_nvfp4_fwd, quantize, quantize_fp8,
+                                 quantize_int8, quantize_nvfp4)
 
 # submodule paths of the reference: ac4k_kernel.ops.quant / ac4k_kernel.ops.linear (taken from
 # sys.modules: as attributes of the package, `linear` is the function, not the module)
-for _name in ("quant", "linear", "utils"):
+for _name in ("quant", "linear", "utils", "attention"):
     _sys.modules[__name__ + "." + _name] = _sys.modules["ac4k_kernel_amd.ops." + _name]
 
-__all__ = ["quantize", "linear", "fused_linear", "quantize_nvfp4", "quantize_fp8", "quantize_int8", "linear_nvfp4"]
+__all__ = ["quantize", "linear", "fused_linear", "quantize_nvfp4", "quantize_fp8", "quantize_int8", "linear_nvfp4",
+           "attention", "mha_nvfp4_fwd"]

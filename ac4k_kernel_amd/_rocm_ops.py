@@ -261,3 +261,46 @@ def linear_nvfp4_fused(D, X, X_q, X_sf, X_global_scale, B, B_sf, B_global_scale,
                                                B_sf.data_ptr(), B_global_scale.data_ptr(), bias_ptr, bias_tag,
                                                M, N, K, None if ws is None else ws.data_ptr(),
                                                0 if ws is None else ws.numel(), _stream()))
+
+
+def _check_attention_operand(x, x_sf, x_gs, B, H, rows, width, name):
+    """One packed operand of mha_nvfp4_fwd: x [B,H,rows,width/2], x_sf [B,H,ceil(width/64),align_up(rows,16),4]
+    (mha_nvfp4.cu:917-1003)."""
+    _check_tensor(x, torch.uint8, name)
+    _check(x.dim() == 4 and list(x.shape) == [B, H, rows, width // 2], "{} must be [{}, {}, {}, {}]", name, B, H, rows, width // 2)
+    _check_tensor(x_sf, torch.float8_e4m3fn, name + "_sf")
+    _check(x_sf.dim() == 5, "{}_sf must be a 5D tensor", name)
+    _check(list(x_sf.shape) == [B, H, (width + 63) // 64, _align_up(rows, 16), 4], "Meet invalid {}_sf size", name)
+    _check_tensor(x_gs, torch.float32, name + "_global_scale")
+    _check(x_gs.dim() == 0, "{}_global_scale must be a float tensor", name)
+
+
+def mha_nvfp4_fwd(o, q, q_sf, q_global_scale, k, k_sf, k_global_scale, v, v_sf, v_global_scale, sm_scale: float) -> None:
+    """Checks of mha_nvfp4.cu:917-1012.  o may be a permuted view (the reference's caller passes one): only its
+    shape [B,H,Nq,Dv], dtype and device are checked."""
+    _check(isinstance(q, torch.Tensor) and q.dim() == 4, "Q must be a 4D tensor")
+    B, H, Nq = q.size(0), q.size(1), q.size(2)
+    Dqk = q.size(3) * 2
+    _check(Dqk % 16 == 0, "Dqk must be multiple of 16")
+    _check(Dqk <= 128, "Dqk must be less than 128")
+    _check(isinstance(k, torch.Tensor) and k.dim() == 4, "K must be a 4D tensor")
+    _check(k.size(0) == B, "K must have the same batch size as Q")
+    _check(k.size(1) == H, "K must have the same head number as Q")
+    _check(k.size(3) == q.size(3), "K must have the same dim as Q")
+    Nkv = k.size(2)
+    _check(isinstance(v, torch.Tensor) and v.dim() == 4, "V must be a 4D tensor")
+    Dv = v.size(2)
+    _check(Dv <= 128, "Dv must be less than 128")
+    _check(v.size(3) * 2 == _align_up(Nkv, 64), "V must have the same sequence length as K")
+    _check_attention_operand(q, q_sf, q_global_scale, B, H, Nq, Dqk, "q")
+    _check_attention_operand(k, k_sf, k_global_scale, B, H, Nkv, Dqk, "k")
+    _check_attention_operand(v, v_sf, v_global_scale, B, H, Dv, _align_up(Nkv, 64), "v")
+    _check(isinstance(o, torch.Tensor) and o.is_cuda, "O must be a CUDA tensor")
+    _check(o.dtype == torch.bfloat16, "O must be a bfloat16 tensor")
+    _check(o.dim() == 4 and list(o.shape) == [B, H, Nq, Dv], "O must be [{}, {}, {}, {}]", B, H, Nq, Dv)
+    if B == 0 or H == 0 or Nq == 0:
+        return
+    _check(Nkv > 0, "K must not be empty")
+    _lib.check(_L.ac4k_mha_nvfp4_fwd(o.data_ptr(), *o.stride(), q.data_ptr(), q_sf.data_ptr(), q_global_scale.data_ptr(),
+                                     k.data_ptr(), k_sf.data_ptr(), k_global_scale.data_ptr(), v.data_ptr(), v_sf.data_ptr(),
+                                     v_global_scale.data_ptr(), B, H, Nq, Nkv, Dqk, Dv, float(sm_scale), _stream()))

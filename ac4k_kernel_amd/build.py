@@ -16,7 +16,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libac4k_nvfp4.so")
-SOURCES = ["capi.hip", "quantize.hip", "linear.hip"]
+SOURCES = ["capi.hip", "quantize.hip", "linear.hip", "attention.hip"]
 HEADERS = [os.path.join(CSRC, "ac4k_common.h"), os.path.join(ROOT, "include", "ac4k_nvfp4.h")]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

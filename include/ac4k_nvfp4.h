@@ -210,6 +210,21 @@ int ac4k_linear_nvfp4_fused_bf16(void *D, int d_dtype, const void *X, void *X_q,
                                  const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K,
                                  void *workspace, int64_t workspace_bytes, ac4k_stream_t stream);
 
+/* Replaces ac4k::mha_nvfp4_fwd (include/ac4k_kernel/ops.h:12-16, lib/cuda/sm120/mha_nvfp4.cu:911-1077):
+ * O = softmax(Q K^T * sm_scale) V on NVFP4 operands, the consumer of the quantizer's swizzled layout.
+ * q [B,H,Nq,Dqk/2], k [B,H,Nkv,Dqk/2] packed e2m1 with scales [B,H,Dqk/64,align_up(rows,16),4];
+ * v [B,H,Dv,align_up(Nkv,64)/2] quantized along the kv dim with swizzle (quantize(v, 3, N_dim, swizzle=True)),
+ * v_sf [B,H,align_up(Nkv,64)/64,align_up(Dv,16),4]; the three global scales are device scalars;
+ * O bf16 [B,H,Nq,Dv] addressed through its four element strides (the reference passes a permuted view).
+ * The attention probabilities are re-quantized to NVFP4 per 16-block with the global scale 1/2688, as in
+ * mha_nvfp4.cu:248-319.  First slice of this operator: head dim 128 only (Dqk == Dv == 128; the reference
+ * takes any multiple of 16 up to 128), correctness first, not tuned. */
+int ac4k_mha_nvfp4_fwd(void *O, int64_t o_b_stride, int64_t o_h_stride, int64_t o_n_stride,
+                       int64_t o_d_stride, const void *q, const void *q_sf, const float *q_gs,
+                       const void *k, const void *k_sf, const float *k_gs, const void *v,
+                       const void *v_sf, const float *v_gs, int64_t B, int64_t H, int64_t Nq,
+                       int64_t Nkv, int64_t Dqk, int64_t Dv, float sm_scale, ac4k_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
