@@ -127,9 +127,7 @@ __device__ __forceinline__ TileCoord tile_of_workgroup(int64_t pid, int64_t tile
 // LDS_SWZ(row) so that both the decode stores and the MFMA fragment loads are conflict-free.
 // ===========================================================================
 constexpr int T_BM = 128, T_BN = 128, T_BK = 64;
-#ifndef LDS_SWZ
 #define LDS_SWZ(row) ((row) & 7)
-#endif
 
 struct PackedRegs {
   uint2 d[2];    // two 16-blocks (8 bytes each) of this thread's row

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the NVFP4 path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|linear|quantize|traffic|quantize-timeline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|linear|quantize|traffic|quantize-timeline|linear-timeline]
                     [--no-cpu-baseline] [--no-check]
 
 Prints ONE JSON line.  The headline `value` is the NVFP4 linear at M=N=K=8192 (the
@@ -402,6 +402,37 @@ def bench_quantize_layouts(ops, steps, warmup):
     return res
 
 
+def bench_attention(ops, B, N, H, D, steps, warmup, check=True):
+    """NVFP4 attention forward (first slice of the operator: head dim 128, untuned kernel): flops = 4 B H N^2 D as in
+    the reference's test/test_attention_tflops.py:31-33; the kernel alone on pre-quantized operands and the whole
+    attention() call (three quantizes + kernel).  Check: cosine similarity and elementwise distance to torch's
+    scaled_dot_product_attention on the GPU, at the tolerance of test/test_attention_bench.py:19-66."""
+    import math
+    g = torch.Generator(device="cuda").manual_seed(7)
+    q, k, v = (torch.empty((B, N, H, D), dtype=torch.float32, device="cuda").normal_(generator=g).to(torch.bfloat16)
+               for _ in range(3))
+    out = torch.empty((B, N, H, D), dtype=torch.bfloat16, device="cuda")
+    ops.attention(q, k, v, layout="BNHD", precision="nvfp4", out=out)
+    ok = cos = None
+    if check:
+        ref = torch.nn.functional.scaled_dot_product_attention(q.transpose(1, 2).float(), k.transpose(1, 2).float(),
+                                                               v.transpose(1, 2).float()).transpose(1, 2)
+        cos = torch.nn.functional.cosine_similarity(out.float().flatten(), ref.flatten(), dim=0).item()
+        inside = ((out.float() - ref).abs() <= 2e-1 + 1e-1 * ref.abs()).float().mean().item()
+        ok = bool(cos > 0.98 and inside > 0.999)
+        del ref
+    qq, kq, vq = ops.quantize(q, 1, 3), ops.quantize(k, 1, 3), ops.quantize(v, 3, 1, swizzle=True)
+    o_bhnd = out.permute(0, 2, 1, 3)
+    _, ms_k = time_gpu(lambda: ops.mha_nvfp4_fwd(o_bhnd, *qq, *kq, *vq, 1.0 / math.sqrt(D)), steps, warmup)
+    _, ms_a = time_gpu(lambda: ops.attention(q, k, v, layout="BNHD", precision="nvfp4", out=out), steps, warmup)
+    flops = 4.0 * B * H * N * N * D
+    return {"workload": f"NVFP4 attention forward B={B} N={N} H={H} D={D}, bf16 in / out", "kernel_ms": ms_k,
+            "kernel_TFLOP/s": flops / (ms_k * 1e-3) / 1e12, "with_quantize_ms": ms_a,
+            "with_quantize_TFLOP/s": flops / (ms_a * 1e-3) / 1e12, "cosine_vs_fp32_attention": cos,
+            "within_reference_tolerance_of_fp32_attention": ok,
+            "roofline": roofline("mfma", flops / (ms_k * 1e-3) / 1e12)}
+
+
 def bench_linear_epilogues(ops, steps, warmup, n=8192):
     """Output dtype x bias matrix of the linear (test/test_linear_bench.py:178-205) at n^3."""
     a, b = make_input((n, n), seed=0).cuda(), make_input((n, n), seed=1).cuda()
@@ -519,13 +550,49 @@ def run_quantize_timeline(ops, reps=20):
     print(json.dumps({"quantize_timeline_us": res}))
 
 
+def run_linear_timeline(ops, reps=12):
+    """Per-workgroup phase boundaries of the linear kernels that carry clock stamps (the packed-operand tile
+    kernel and the K-split-waves kernel; needs the library built by `python ac4k_kernel_amd/build.py --timeline`,
+    loaded through AC4K_NVFP4_LIB): microseconds after the first workgroup's entry at loop entry, loop exit and
+    kernel exit (min / mean / max over the workgroups of the last of `reps` launches), shader cycles in the loop."""
+    import ctypes
+    from ac4k_kernel_amd import _lib
+    L = _lib.load()
+    fn = getattr(L, "ac4k_debug_linear_timeline", None)
+    if fn is None:
+        sys.exit("bench.py: this library has no clock stamps; build with `python ac4k_kernel_amd/build.py --timeline` "
+                 "and set AC4K_NVFP4_LIB to the library it prints")
+    fn.restype, fn.argtypes = ctypes.c_int, [ctypes.c_void_p]
+    res = {}
+    for (m, n, k, nwg) in ((8192, 8192, 8192, 1024), (128, 14336, 4096, 224), (128, 4096, 14336, 256)):
+        aq = ops.quantize(make_input((m, k), seed=0).cuda(), 0, 1)
+        bqs = [ops.quantize(make_input((n, k), seed=1 + i, std=0.02).cuda(), 0, 1) for i in range(4)]
+        out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+        buf = (ctypes.c_uint64 * (8192 * 6))()
+        for r in range(reps):
+            ops.linear(*aq, *bqs[r % 4], out=out)
+        _lib.check(fn(buf))
+        rows = [[buf[w * 6 + i] for i in range(6)] for w in range(nwg)]
+        t0 = min(x[0] for x in rows)
+        tag = f"M{m}_N{n}_K{k}"
+        res[tag] = {}
+        for name, i in (("entry", 0), ("loop_entry", 1), ("loop_exit", 2), ("exit", 3)):
+            col = [(x[i] - t0) * 0.01 for x in rows]
+            res[tag][name] = {"min": round(min(col), 2), "mean": round(sum(col) / len(col), 2), "max": round(max(col), 2)}
+        loop_us = sum((x[2] - x[1]) * 0.01 for x in rows) / len(rows)
+        cyc = sum(x[4] for x in rows) / len(rows)
+        res[tag]["loop"] = {"us": round(loop_us, 2), "cycles": round(cyc), "GHz": round(cyc / loop_us / 1e3, 3)}
+        log(f"[timeline] {tag}: " + "  ".join(f"{k_} {v}" for k_, v in res[tag].items()))
+    print(json.dumps({"linear_timeline_us": res}))
+
+
 def main():
     global SETTLE_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", choices=["all", "linear", "quantize", "traffic", "quantize-timeline"])
+    ap.add_argument("--workload", default="all", choices=["all", "linear", "quantize", "traffic", "quantize-timeline", "linear-timeline"])
     ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
                     help="keep the untimed warm-up going for this long (clock ramp); 0 = exactly --warmup calls")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -552,6 +619,8 @@ def main():
         return run_traffic(ops)
     if args.workload == "quantize-timeline":
         return run_quantize_timeline(ops)
+    if args.workload == "linear-timeline":
+        return run_linear_timeline(ops)
     check = not args.no_check  # the GEMM checks: fp32 dequantize-matmul with torch ops on the GPU
     # The CPU leg (the only user of oracle/): the oracle timed on the host cores as `cpu_baseline`, and the
     # same oracle as the checker of the quantizers' GPU output.  --no-cpu-baseline skips all of it.
@@ -640,6 +709,11 @@ def main():
             for k_, v in lay.items():
                 log(f"[bench] quantize layout {k_}: {v['ms'] * 1e3:.1f} us  {v['GB/s']:.0f} GB/s")
             line["quantize_layouts"] = lay
+            att = bench_attention(ops, 1, 16384, 40, 128, max(3, S // 10), 2, check=check)
+            log(f"[bench] {att['workload']}: kernel {att['kernel_ms']:.2f} ms  {att['kernel_TFLOP/s']:.0f} TFLOP/s "
+                f"({100 * att['roofline']['frac']:.1f}% of MFMA peak; first, untuned slice), with the three quantizes "
+                f"{att['with_quantize_ms']:.2f} ms  ok={att['within_reference_tolerance_of_fp32_attention']}")
+            line["attention"] = att
             epi = bench_linear_epilogues(ops, S, W)
             log("[bench] linear 8192^3 by output/bias dtype, TFLOP/s: "
                 + ", ".join(f"{k_} {v['TFLOP/s']:.0f}" for k_, v in epi.items()))

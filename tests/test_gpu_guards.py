@@ -188,3 +188,19 @@ def test_prepacked_linear_stays_inside_image_workspace_and_output(m, n, k):
         torch.cuda.synchronize()
         assert d.intact() and ws.intact() and img.intact(), (m, n, k, shift)
         assert same_bytes(d.t, ref), (m, n, k, shift)
+
+
+def test_attention_stays_inside_its_output():
+    """The attention kernel writes O through its strides: a BNHD output that is a window inside a pattern-filled
+    allocation keeps its surroundings, for query lengths that leave a ragged last tile."""
+    import math
+    for (B, Nq, Nkv, H) in ((1, 33, 70, 2), (2, 130, 130, 1)):
+        q = make_input((B, Nq, H, 128), seed=3).cuda()
+        k, v = make_input((B, Nkv, H, 128), seed=4).cuda(), make_input((B, Nkv, H, 128), seed=5).cuda()
+        qq, kq, vq = ops().quantize(q, 1, 3), ops().quantize(k, 1, 3), ops().quantize(v, 3, 1, swizzle=True)
+        ref = torch.empty((B, Nq, H, 128), dtype=torch.bfloat16, device="cuda")
+        ops().mha_nvfp4_fwd(ref.permute(0, 2, 1, 3), *qq, *kq, *vq, 1 / math.sqrt(128))
+        w = Window((B, Nq, H, 128), torch.bfloat16)
+        ops().mha_nvfp4_fwd(w.t.permute(0, 2, 1, 3), *qq, *kq, *vq, 1 / math.sqrt(128))
+        torch.cuda.synchronize()
+        assert w.intact() and same_bytes(w.t, ref)
