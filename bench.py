@@ -499,6 +499,24 @@ def run_traffic(ops):
             for _ in range(3):
                 ops.linear_prepacked(*xq, wimg, wq[2], out=o)
         del wq, wimg
+    # configuration 4 at M = 128: the K-split-waves kernel (one launch at N = 14336, K ranges + reduce at N = 4096)
+    for (n, k) in ((14336, 4096), (4096, 14336)):
+        wq = ops.quantize(make_input((n, k), seed=3, std=0.02).cuda(), 0, 1)
+        xq = ops.quantize(make_input((128, k), seed=2).cuda(), 0, 1)
+        o = torch.empty((128, n), dtype=torch.bfloat16, device="cuda")
+        for _ in range(3):
+            ops.linear(*xq, *wq, out=o)
+        del wq, xq, o
+    # attention kernel on pre-quantized operands, B = 1, N = 8192, H = 40, D = 128
+    import math
+    g = torch.Generator(device="cuda").manual_seed(7)
+    q, k_, v = (torch.empty((1, 8192, 40, 128), dtype=torch.float32, device="cuda").normal_(generator=g).to(torch.bfloat16)
+                for _ in range(3))
+    qq, kq, vq = ops.quantize(q, 1, 3), ops.quantize(k_, 1, 3), ops.quantize(v, 3, 1, swizzle=True)
+    o = torch.empty((1, 40, 8192, 128), dtype=torch.bfloat16, device="cuda")
+    for _ in range(3):
+        ops.mha_nvfp4_fwd(o, *qq, *kq, *vq, 1.0 / math.sqrt(128))
+    del q, k_, v, qq, kq, vq, o
     x = make_input((8192, 4096), seed=0, outliers=True).cuda()
     for prec in ("nvfp4", "fp8e4m3", "int8"):
         for _ in range(3):
@@ -686,7 +704,7 @@ def main():
                 for m in (16, 128, 2048, 8192):
                     shapes[f"cfg4_M{m}_N{n}_K{k}"] = bench_linear(ops, m, n, k, S, W, wstd=0.02, check=check,
                                                                   with_quantize=True, with_image=True,
-                                                                  key=f"decode_linear_M{m}_N{n}_K{k}" if m <= 32 else None)
+                                                                  key=f"decode_linear_M{m}_N{n}_K{k}" if m <= 128 else None)
             for m in (1, 8, 32):  # configuration 5 with the activation already quantized (linear alone)
                 shapes[f"cfg5_M{m}_linear_alone"] = bench_linear(ops, m, 28672, 8192, S, W, wstd=0.02, check=check,
                                                                  with_image=True, key=f"decode_linear_M{m}")
