@@ -9,8 +9,11 @@
 //   positions {8g + 4h + j} (g, j = 0..3) of a 32-group, h = 0, 1 - the sets that the swizzle of
 //   quantize(v, 3, N_dim, swizzle=True) makes contiguous in V                                    :248-319
 //   O = (sum over tiles of Phat . Vhat^T, rescaled) * ((1/l) * (1/2688) * v_gs) -> bf16          :705-830
-// A first, untuned kernel: every wave owns 32 query rows and reads its operands straight from global
-// memory (the four waves of a workgroup share the K and V tiles through the caches).
+// A workgroup (four waves) owns 128 query rows, a wave 32 of them.  Per kv tile of 128 the packed K rows and
+// the packed V rows (V is stored [d][kv]) are fetched once per workgroup - every thread two 16-byte pieces of
+// each plus one scale dword, issued a whole tile ahead -, decoded once to exact fp16 and written to LDS, from
+// where all four waves read their MFMA operands.  Two LDS buffers alternate, one barrier per tile.  Decoded rows
+// are 256 bytes at a pitch of 272, so that the 16-byte fragment reads of 16 lanes fall on 64 different banks.
 //
 // The MFMAs are issued so that a lane owns ONE query row: S^T = Khat . Qhat^T and O^T = Vhat . Phat^T
 // (v_mfma_f32_32x32x16_f16, exact fp16 decode as in the linear).  Lane (r, h) of a wave then holds, per
@@ -19,6 +22,8 @@
 // halves of the wave.  The k slots of the second product are paired through the stored (swizzled) order
 // of V: slot s of step t holds kv position 8 (2t + (s>>1 & 1)) + 4h + 2 (s>>2) + (s & 1).
 #include "ac4k_common.h"
+
+#include <atomic>
 
 namespace ac4k {
 
@@ -29,6 +34,7 @@ struct MhaArgs {
   const float *q_gs, *k_gs, *v_gs;
   int64_t H, Nq, Nkv, Nqp, Nkvp, Nkv64;  // padded: rows of the Q / K scale planes (16), stored kv length of V (64)
   float sm_scale;
+  int o_vec;  // O rows are contiguous along d and 8-byte aligned: four head dims per store
 };
 
 constexpr int MHA_D = 128;
@@ -44,16 +50,12 @@ __device__ __forceinline__ f16x8 mha_decode8(uint32_t w, f16x2 sc) {
   return (f16x8){d0.x, d0.y, d1.x, d1.y, d2.x, d2.y, d3.x, d3.y};
 }
 
-// A row-major packed row (Q or K): the lane's 32 elements [32 h, 32 h + 32) of 64-chunk c, and the two block
-// scales that go with them, decoded into the four 16-k operands of that chunk.  `valid` false: zeros.
+// A row-major packed row of Q: the lane's 32 elements [32 h, 32 h + 32) of 64-chunk c, and the two block
+// scales that go with them, decoded into the four 16-k operands of that chunk.
 __device__ __forceinline__ void mha_load_row_chunk(const uint8_t *row, const uint8_t *sf_chunk_row, int c, int h,
-                                                   bool valid, f16x8 (&out)[4]) {
-  uint4 w = make_uint4(0, 0, 0, 0);
-  uint32_t sc = 0;
-  if (valid) {
-    w = *reinterpret_cast<const uint4 *>(row + c * 32 + h * 16);
-    sc = *reinterpret_cast<const uint16_t *>(sf_chunk_row + 2 * h);
-  }
+                                                   f16x8 (&out)[4]) {
+  const uint4 w = *reinterpret_cast<const uint4 *>(row + c * 32 + h * 16);
+  const uint32_t sc = *reinterpret_cast<const uint16_t *>(sf_chunk_row + 2 * h);
   const f16x2 s2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(sc, 1.0f, false);
   const f16x2 lo = {s2.x, s2.x}, hi = {s2.y, s2.y};
   out[0] = mha_decode8(w.x, lo);
@@ -66,70 +68,146 @@ __device__ __forceinline__ float mha_xor32(float x) {  // value of the lane 32 a
   return __shfl_xor(x, 32, 64);
 }
 
+constexpr int MHA_PITCH = 272;                   // bytes per decoded row in LDS: 128 fp16 + 16 (bank spread)
+constexpr int MHA_TILE_LDS = 128 * MHA_PITCH;    // one decoded operand tile: K 128 kv rows, V 128 d rows
+constexpr int MHA_LDS_BYTES = 4 * MHA_TILE_LDS;  // two buffers of (K tile, V tile)
+
+// what one thread fetches for a kv tile: half a packed K row (one 64-chunk), half a packed V row of the tile
+// (one 64-chunk of kv positions), and the scale dword of each
+struct MhaFetch {
+  uint4 k0, k1, v0, v1;
+  uint32_t ksc, vsc;
+};
+
 __global__ __launch_bounds__(256) void mha_nvfp4_fwd_d128_kernel(MhaArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t mha_lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
+  const int srow = threadIdx.x >> 1, sc = threadIdx.x & 1;         // staging role: row of the tile, 64-chunk
   const int64_t b = blockIdx.z, head = blockIdx.y, bh = b * a.H + head;
   const int64_t m = (int64_t)blockIdx.x * 128 + wave * 32 + r;   // this lane's query row
   const int64_t mq = m < a.Nq ? m : a.Nq - 1;                    // rows past Nq read the last row; never stored
+  const int64_t v_row_bytes = a.Nkv64 / 2, v_chunks = a.Nkv64 / 64;
+
+  const uint8_t *k_src = a.k + bh * a.Nkv * (MHA_D / 2) + sc * 32;
+  const uint8_t *ksf_src = a.k_sf + (bh * 2 + sc) * a.Nkvp * 4;
+  const uint8_t *v_src = a.v + (bh * MHA_D + srow) * v_row_bytes + sc * 32;
+  const uint8_t *vsf_src = a.v_sf + ((bh * v_chunks + sc) * MHA_D + srow) * 4;
+  auto fetch = [&](int64_t n0, MhaFetch &f) {  // rows past Nkv and chunks past the stored length of V are zeros
+    const int64_t n = n0 + srow;
+    f.k0 = f.k1 = f.v0 = f.v1 = make_uint4(0, 0, 0, 0);
+    f.ksc = f.vsc = 0;
+    if (n < a.Nkv) {
+      const uint4 *p = reinterpret_cast<const uint4 *>(k_src + n * (MHA_D / 2));
+      f.k0 = p[0];
+      f.k1 = p[1];
+      f.ksc = *reinterpret_cast<const uint32_t *>(ksf_src + n * 4);
+    }
+    if (n0 + 64 * sc < a.Nkv64) {
+      const uint4 *p = reinterpret_cast<const uint4 *>(v_src + n0 / 2);
+      f.v0 = p[0];
+      f.v1 = p[1];
+      f.vsc = *reinterpret_cast<const uint32_t *>(vsf_src + (n0 / 64) * (MHA_D * 4));
+    }
+  };
+  auto put = [](uint8_t *dst, f16x8 v) { *reinterpret_cast<f16x8 *>(dst) = v; };
+  auto stage = [&](int buf, const MhaFetch &f) {  // decode once per workgroup, into LDS
+    uint8_t *kd = mha_lds + buf * 2 * MHA_TILE_LDS + srow * MHA_PITCH + sc * 128;
+    const f16x2 k01 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.ksc, 1.0f, false);
+    const f16x2 k23 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.ksc, 1.0f, true);
+    const f16x2 kb0 = {k01.x, k01.x}, kb1 = {k01.y, k01.y}, kb2 = {k23.x, k23.x}, kb3 = {k23.y, k23.y};
+    put(kd + 0, mha_decode8(f.k0.x, kb0));
+    put(kd + 16, mha_decode8(f.k0.y, kb0));
+    put(kd + 32, mha_decode8(f.k0.z, kb1));
+    put(kd + 48, mha_decode8(f.k0.w, kb1));
+    put(kd + 64, mha_decode8(f.k1.x, kb2));
+    put(kd + 80, mha_decode8(f.k1.y, kb2));
+    put(kd + 96, mha_decode8(f.k1.z, kb3));
+    put(kd + 112, mha_decode8(f.k1.w, kb3));
+    // V: the chunk holds two 32-groups of 16 stored bytes; operand piece (t, h) of a group takes the t-th 16-bit
+    // halves of its dwords 2h and 2h + 1, and the scale of stored block h of the group
+    uint8_t *vd = mha_lds + (buf * 2 + 1) * MHA_TILE_LDS + srow * MHA_PITCH + sc * 128;
+    const f16x2 v01 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.vsc, 1.0f, false);
+    const f16x2 v23 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.vsc, 1.0f, true);
+    const f16x2 vs[2][2] = {{{v01.x, v01.x}, {v01.y, v01.y}}, {{v23.x, v23.x}, {v23.y, v23.y}}};
+    const uint32_t g[2][4] = {{f.v0.x, f.v0.y, f.v0.z, f.v0.w}, {f.v1.x, f.v1.y, f.v1.z, f.v1.w}};
+#pragma unroll
+    for (int gi = 0; gi < 2; ++gi)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const uint32_t d0 = g[gi][2 * hh], d1 = g[gi][2 * hh + 1];
+        put(vd + gi * 64 + 0 + hh * 16, mha_decode8((d0 & 0xffffu) | (d1 << 16), vs[gi][hh]));
+        put(vd + gi * 64 + 32 + hh * 16, mha_decode8((d0 >> 16) | (d1 & 0xffff0000u), vs[gi][hh]));
+      }
+  };
 
   // Qhat of the lane's row: 8 operands of 16 k (chunk c, sub-step s), kept for the whole kernel
   f16x8 QF[2][4];
 #pragma unroll
   for (int c = 0; c < 2; ++c)
-    mha_load_row_chunk(a.q + (bh * a.Nq + mq) * (MHA_D / 2), a.q_sf + ((bh * 2 + c) * a.Nqp + mq) * 4, c, h, true, QF[c]);
+    mha_load_row_chunk(a.q + (bh * a.Nq + mq) * (MHA_D / 2), a.q_sf + ((bh * 2 + c) * a.Nqp + mq) * 4, c, h, QF[c]);
 
-  const float qk_scale = (*a.q_gs) * (*a.k_gs) * a.sm_scale;
-  float m_run = -__builtin_inff(), l_run = 0.0f;
+  // exp2 argument = S * cs - (row maximum of S) * cs with cs = q_gs * k_gs * sm_scale * log2(e); a negative cs is
+  // moved into Q so that the row maximum can be taken over the raw dot products
+  float cs = (*a.q_gs) * (*a.k_gs) * a.sm_scale * MHA_LOG2E;
+  if (cs < 0.0f) {
+    cs = -cs;
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int s = 0; s < 4; ++s) QF[c][s] = -QF[c][s];
+  }
+  float ml_run = -__builtin_inff(), l_run = 0.0f;  // running row maximum (in log2 units) and row sum
   f32x16 OT[4];  // O^T: d = 32 fd + 8 (e >> 2) + 4 h + (e & 3), for the lane's query row
 #pragma unroll
   for (int fd = 0; fd < 4; ++fd)
 #pragma unroll
     for (int e = 0; e < 16; ++e) OT[fd][e] = 0.0f;
 
-  const int64_t v_row_bytes = a.Nkv64 / 2, v_chunks = a.Nkv64 / 64;
-  for (int64_t n0 = 0; n0 < a.Nkv; n0 += 128) {
+  MhaFetch nxt;
+  fetch(0, nxt);
+  stage(0, nxt);
+  __syncthreads();
+  int buf = 0;
+  for (int64_t n0 = 0; n0 < a.Nkv; n0 += 128, buf ^= 1) {
+    fetch(n0 + 128, nxt);  // the next tile's packed bytes travel while this one is multiplied (zeros past the end)
+    const uint8_t *kb = mha_lds + buf * 2 * MHA_TILE_LDS + r * MHA_PITCH + h * 64;
+    const uint8_t *vb = mha_lds + (buf * 2 + 1) * MHA_TILE_LDS + r * MHA_PITCH + h * 16;
     // ---- S^T = Khat . Qhat^T for the 128 kv positions of the tile (four 32-row fragments)
     f32x16 ST[4];
 #pragma unroll
     for (int f = 0; f < 4; ++f) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) ST[f][e] = 0.0f;
-      const int64_t n = n0 + f * 32 + r;
-      const bool valid = n < a.Nkv;  // rows past Nkv are zero: S = 0 there
-      const int64_t nn = valid ? n : 0;
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        f16x8 KF[4];
-        mha_load_row_chunk(a.k + (bh * a.Nkv + nn) * (MHA_D / 2), a.k_sf + ((bh * 2 + c) * a.Nkvp + nn) * 4, c, h, valid, KF);
+      for (int c = 0; c < 2; ++c)
 #pragma unroll
-        for (int s = 0; s < 4; ++s) ST[f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(KF[s], QF[c][s], ST[f], 0, 0, 0);
-      }
+        for (int s = 0; s < 4; ++s) {
+          const f16x8 KF = *reinterpret_cast<const f16x8 *>(kb + f * 32 * MHA_PITCH + c * 128 + s * 16);
+          ST[f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(KF, QF[c][s], ST[f], 0, 0, 0);
+        }
     }
     // ---- online softmax of the lane's row: its 64 values here, the other 64 in the lane 32 away
-    float mx = m_run;
+    float mx = -__builtin_inff();
 #pragma unroll
     for (int f = 0; f < 4; ++f)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        ST[f][e] *= qk_scale;
-        mx = __builtin_fmaxf(mx, ST[f][e]);
-      }
-    const float m_new = __builtin_fmaxf(mx, mha_xor32(mx));
-    const float ml = m_new * MHA_LOG2E;
+      for (int e = 0; e < 16; ++e) mx = __builtin_fmaxf(mx, ST[f][e]);
+    mx = __builtin_fmaxf(mx, mha_xor32(mx));
+    const float ml = __builtin_fmaxf(ml_run, mx * cs);
     float lsum = 0.0f;
 #pragma unroll
     for (int f = 0; f < 4; ++f)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        ST[f][e] = __builtin_amdgcn_exp2f(ST[f][e] * MHA_LOG2E - ml);  // p
+        ST[f][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(ST[f][e], cs, -ml));  // p
         lsum += ST[f][e];
       }
     float l_new = lsum + mha_xor32(lsum);
     if (n0 + 128 > a.Nkv)  // the zero-filled positions of the last tile each added exp(0 - m)
       l_new -= (float)(n0 + 128 - a.Nkv) / __builtin_amdgcn_exp2f(ml);
-    const float alpha = __builtin_amdgcn_exp2f(m_run * MHA_LOG2E - ml);
+    const float alpha = __builtin_amdgcn_exp2f(ml_run - ml);
     l_run = alpha * l_run + l_new;
-    m_run = m_new;
+    ml_run = ml;
 #pragma unroll
     for (int fd = 0; fd < 4; ++fd)
 #pragma unroll
@@ -146,9 +224,6 @@ __global__ __launch_bounds__(256) void mha_nvfp4_fwd_d128_kernel(MhaArgs a) {
       const float o = s != 0.0f ? MHA_P_ALPHA * (1.0f / s) : 0.0f;
       const _Float16 sh = (_Float16)s;  // an e4m3 value: exact in fp16
       const f16x2 psc = {sh, sh};
-      // the 32-group of V that holds these kv positions: 16 stored bytes per d row
-      const int64_t g32 = (n0 + f * 32) / 32;
-      const bool v_valid = (n0 + f * 32) < a.Nkv64;
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         // k slots of this step in the order the stored nibbles of V come in (see the header)
@@ -157,32 +232,33 @@ __global__ __launch_bounds__(256) void mha_nvfp4_fwd_d128_kernel(MhaArgs a) {
         const f16x8 PF = mha_decode8(f32x8_to_e2m1x8(pv), psc);
 #pragma unroll
         for (int fd = 0; fd < 4; ++fd) {
-          const int64_t d = fd * 32 + r;
-          uint32_t w = 0, vs = 0;
-          if (v_valid) {
-            const uint32_t *grp = reinterpret_cast<const uint32_t *>(a.v + (bh * MHA_D + d) * v_row_bytes + g32 * 16);
-            const uint32_t lo = (grp[2 * h] >> (16 * t)) & 0xffffu, hi = (grp[2 * h + 1] >> (16 * t)) & 0xffffu;
-            w = lo | (hi << 16);
-            vs = a.v_sf[((bh * v_chunks + g32 / 2) * MHA_D + d) * 4 + 2 * (g32 & 1) + h];
-          }
-          const f16x2 v2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(vs, 1.0f, false);
-          const f16x2 vsc = {v2.x, v2.x};
-          OT[fd] = __builtin_amdgcn_mfma_f32_32x32x16_f16(mha_decode8(w, vsc), PF, OT[fd], 0, 0, 0);
+          const f16x8 VF = *reinterpret_cast<const f16x8 *>(vb + fd * 32 * MHA_PITCH + f * 64 + t * 32);
+          OT[fd] = __builtin_amdgcn_mfma_f32_32x32x16_f16(VF, PF, OT[fd], 0, 0, 0);
         }
       }
     }
+    stage(buf ^ 1, nxt);
+    __syncthreads();
   }
 
   // ---- O = O * ((1/l) * (1/2688) * v_gs) -> bf16
   if (m >= a.Nq) return;
   const float scale = (1.0f / l_run) * (1.0f / MHA_P_ALPHA) * (*a.v_gs);
   uint16_t *orow = a.O + b * a.o_b + head * a.o_h + m * a.o_n;
+  auto bf = [&](float x) { return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)(x * scale)); };
 #pragma unroll
   for (int fd = 0; fd < 4; ++fd)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int d = fd * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
-      orow[d * a.o_d] = __builtin_bit_cast(uint16_t, (__bf16)(OT[fd][e] * scale));
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const int d = fd * 32 + q4 * 8 + h * 4;  // four consecutive head dims
+      if (a.o_vec) {
+        const uint2 w = make_uint2(bf(OT[fd][4 * q4]) | (bf(OT[fd][4 * q4 + 1]) << 16),
+                                   bf(OT[fd][4 * q4 + 2]) | (bf(OT[fd][4 * q4 + 3]) << 16));
+        *reinterpret_cast<uint2 *>(orow + d) = w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) orow[(d + e) * a.o_d] = (uint16_t)bf(OT[fd][4 * q4 + e]);
+      }
     }
 }
 
@@ -208,8 +284,21 @@ extern "C" __attribute__((visibility("default"))) int ac4k_mha_nvfp4_fwd(
   MhaArgs a{static_cast<uint16_t *>(O), o_b_stride, o_h_stride, o_n_stride, o_d_stride,
             static_cast<const uint8_t *>(q), static_cast<const uint8_t *>(k), static_cast<const uint8_t *>(v),
             static_cast<const uint8_t *>(q_sf), static_cast<const uint8_t *>(k_sf), static_cast<const uint8_t *>(v_sf),
-            q_gs, k_gs, v_gs, H, Nq, Nkv, align_up(Nq, 16), align_up(Nkv, 16), align_up(Nkv, 64), sm_scale};
-  hipLaunchKernelGGL(mha_nvfp4_fwd_d128_kernel, dim3((unsigned)ceil_div(Nq, 128), (unsigned)H, (unsigned)B), dim3(256), 0,
-                     (hipStream_t)stream, a);
+            q_gs, k_gs, v_gs, H, Nq, Nkv, align_up(Nq, 16), align_up(Nkv, 16), align_up(Nkv, 64), sm_scale,
+            (o_d_stride == 1 && ((uintptr_t)O & 7) == 0 && o_b_stride % 4 == 0 && o_h_stride % 4 == 0 && o_n_stride % 4 == 0) ? 1 : 0};
+  {  // more than 64 KB of dynamic LDS has to be allowed once per device
+    static std::atomic<uint32_t> lds_done{0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    const uint32_t bit = 1u << (dev & 31);
+    if (!(lds_done.load(std::memory_order_relaxed) & bit)) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(mha_nvfp4_fwd_d128_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, MHA_LDS_BYTES);
+      if (e != hipSuccess) return set_error("hipFuncSetAttribute(LDS=%d): %s", MHA_LDS_BYTES, hipGetErrorString(e));
+      lds_done.fetch_or(bit, std::memory_order_relaxed);
+    }
+  }
+  hipLaunchKernelGGL(mha_nvfp4_fwd_d128_kernel, dim3((unsigned)ceil_div(Nq, 128), (unsigned)H, (unsigned)B), dim3(256),
+                     MHA_LDS_BYTES, (hipStream_t)stream, a);
   return check_launch("ac4k_mha_nvfp4_fwd");
 }
