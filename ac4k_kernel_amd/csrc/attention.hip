@@ -64,80 +64,84 @@ __device__ __forceinline__ void mha_load_row_chunk(const uint8_t *row, const uin
   out[3] = mha_decode8(w.w, hi);
 }
 
-__device__ __forceinline__ float mha_xor32(float x) {  // value of the lane 32 away
-  return __shfl_xor(x, 32, 64);
+// dword i (0..7) of two 16-byte pieces; i is a constant after unrolling
+__device__ __forceinline__ uint32_t mha_dword(const uint4 &a, const uint4 &b, int i) {
+  switch (i) {
+    case 0: return a.x;
+    case 1: return a.y;
+    case 2: return a.z;
+    case 3: return a.w;
+    case 4: return b.x;
+    case 5: return b.y;
+    case 6: return b.z;
+    default: return b.w;
+  }
 }
+
+// both halves of the wave (lanes 0-31 and 32-63) receive op(x of the lower half, x of the upper half)
+__device__ __forceinline__ float mha_halves_max(float x) { return __builtin_fmaxf(x, __shfl_xor(x, 32, 64)); }
+__device__ __forceinline__ float mha_halves_sum(float x) { return x + __shfl_xor(x, 32, 64); }
 
 constexpr int MHA_PITCH = 272;                   // bytes per decoded row in LDS: 128 fp16 + 16 (bank spread)
 constexpr int MHA_TILE_LDS = 128 * MHA_PITCH;    // one decoded operand tile: K 128 kv rows, V 128 d rows
-constexpr int MHA_LDS_BYTES = 4 * MHA_TILE_LDS;  // two buffers of (K tile, V tile)
+constexpr int MHA_LDS_BYTES = 4 * MHA_TILE_LDS;  // K tiles j & 1 at 0 and MHA_TILE_LDS, V tiles j & 1 behind them
+constexpr int MHA_WAVES = 8;                     // waves per workgroup, 32 query rows each
+constexpr int MHA_ROWS = 32 * MHA_WAVES;         // query rows per workgroup
 
-// what one thread fetches for a kv tile: half a packed K row (one 64-chunk), half a packed V row of the tile
-// (one 64-chunk of kv positions), and the scale dword of each
+// what one thread fetches per kv tile: a quarter of a packed K row (two 16-blocks), a quarter of a packed V row of
+// the tile (one 32-group of kv positions), and the two scale bytes of each
 struct MhaFetch {
-  uint4 k0, k1, v0, v1;
+  uint4 k, v;
   uint32_t ksc, vsc;
 };
 
-__global__ __launch_bounds__(256) void mha_nvfp4_fwd_d128_kernel(MhaArgs a) {
+__global__ __launch_bounds__(64 * MHA_WAVES) void mha_nvfp4_fwd_d128_kernel(MhaArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t mha_lds[];
+  __shared__ float lut[128];  // exact reciprocals of the e4m3 values, as in the quantizer
+  load_rcp_table(lut);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
-  const int srow = threadIdx.x >> 1, sc = threadIdx.x & 1;         // staging role: row of the tile, 64-chunk
+  // staging role: row of the tile, 64-chunk sc, half sh of the chunk (K: elements 32 sh.., V: 32-group 2 sc + sh)
+  const int srow = threadIdx.x >> 2, sc = (threadIdx.x >> 1) & 1, sh = threadIdx.x & 1;
   const int64_t b = blockIdx.z, head = blockIdx.y, bh = b * a.H + head;
-  const int64_t m = (int64_t)blockIdx.x * 128 + wave * 32 + r;   // this lane's query row
-  const int64_t mq = m < a.Nq ? m : a.Nq - 1;                    // rows past Nq read the last row; never stored
+  const int64_t m = (int64_t)blockIdx.x * MHA_ROWS + wave * 32 + r;   // this lane's query row
+  const int64_t mq = m < a.Nq ? m : a.Nq - 1;                         // rows past Nq read the last row; never stored
   const int64_t v_row_bytes = a.Nkv64 / 2, v_chunks = a.Nkv64 / 64;
 
-  const uint8_t *k_src = a.k + bh * a.Nkv * (MHA_D / 2) + sc * 32;
-  const uint8_t *ksf_src = a.k_sf + (bh * 2 + sc) * a.Nkvp * 4;
-  const uint8_t *v_src = a.v + (bh * MHA_D + srow) * v_row_bytes + sc * 32;
-  const uint8_t *vsf_src = a.v_sf + ((bh * v_chunks + sc) * MHA_D + srow) * 4;
-  auto fetch = [&](int64_t n0, MhaFetch &f) {  // rows past Nkv and chunks past the stored length of V are zeros
+  const uint8_t *k_src = a.k + bh * a.Nkv * (MHA_D / 2) + sc * 32 + sh * 16;
+  const uint8_t *ksf_src = a.k_sf + (bh * 2 + sc) * a.Nkvp * 4 + sh * 2;
+  const uint8_t *v_src = a.v + (bh * MHA_D + srow) * v_row_bytes + sc * 32 + sh * 16;
+  const uint8_t *vsf_src = a.v_sf + ((bh * v_chunks + sc) * MHA_D + srow) * 4 + sh * 2;
+  // rows past Nkv and chunks past the stored length of V are zeros
+  auto fetch = [&](int64_t n0, MhaFetch &f) {
     const int64_t n = n0 + srow;
-    f.k0 = f.k1 = f.v0 = f.v1 = make_uint4(0, 0, 0, 0);
+    f.k = f.v = make_uint4(0, 0, 0, 0);
     f.ksc = f.vsc = 0;
     if (n < a.Nkv) {
-      const uint4 *p = reinterpret_cast<const uint4 *>(k_src + n * (MHA_D / 2));
-      f.k0 = p[0];
-      f.k1 = p[1];
-      f.ksc = *reinterpret_cast<const uint32_t *>(ksf_src + n * 4);
+      f.k = *reinterpret_cast<const uint4 *>(k_src + n * (MHA_D / 2));
+      f.ksc = *reinterpret_cast<const uint16_t *>(ksf_src + n * 4);
     }
     if (n0 + 64 * sc < a.Nkv64) {
-      const uint4 *p = reinterpret_cast<const uint4 *>(v_src + n0 / 2);
-      f.v0 = p[0];
-      f.v1 = p[1];
-      f.vsc = *reinterpret_cast<const uint32_t *>(vsf_src + (n0 / 64) * (MHA_D * 4));
+      f.v = *reinterpret_cast<const uint4 *>(v_src + n0 / 2);
+      f.vsc = *reinterpret_cast<const uint16_t *>(vsf_src + (n0 / 64) * (MHA_D * 4));
     }
   };
-  auto put = [](uint8_t *dst, f16x8 v) { *reinterpret_cast<f16x8 *>(dst) = v; };
-  auto stage = [&](int buf, const MhaFetch &f) {  // decode once per workgroup, into LDS
-    uint8_t *kd = mha_lds + buf * 2 * MHA_TILE_LDS + srow * MHA_PITCH + sc * 128;
-    const f16x2 k01 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.ksc, 1.0f, false);
-    const f16x2 k23 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.ksc, 1.0f, true);
-    const f16x2 kb0 = {k01.x, k01.x}, kb1 = {k01.y, k01.y}, kb2 = {k23.x, k23.x}, kb3 = {k23.y, k23.y};
-    put(kd + 0, mha_decode8(f.k0.x, kb0));
-    put(kd + 16, mha_decode8(f.k0.y, kb0));
-    put(kd + 32, mha_decode8(f.k0.z, kb1));
-    put(kd + 48, mha_decode8(f.k0.w, kb1));
-    put(kd + 64, mha_decode8(f.k1.x, kb2));
-    put(kd + 80, mha_decode8(f.k1.y, kb2));
-    put(kd + 96, mha_decode8(f.k1.z, kb3));
-    put(kd + 112, mha_decode8(f.k1.w, kb3));
-    // V: the chunk holds two 32-groups of 16 stored bytes; operand piece (t, h) of a group takes the t-th 16-bit
-    // halves of its dwords 2h and 2h + 1, and the scale of stored block h of the group
-    uint8_t *vd = mha_lds + (buf * 2 + 1) * MHA_TILE_LDS + srow * MHA_PITCH + sc * 128;
-    const f16x2 v01 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.vsc, 1.0f, false);
-    const f16x2 v23 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.vsc, 1.0f, true);
-    const f16x2 vs[2][2] = {{{v01.x, v01.x}, {v01.y, v01.y}}, {{v23.x, v23.x}, {v23.y, v23.y}}};
-    const uint32_t g[2][4] = {{f.v0.x, f.v0.y, f.v0.z, f.v0.w}, {f.v1.x, f.v1.y, f.v1.z, f.v1.w}};
-#pragma unroll
-    for (int gi = 0; gi < 2; ++gi)
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
-        const uint32_t d0 = g[gi][2 * hh], d1 = g[gi][2 * hh + 1];
-        put(vd + gi * 64 + 0 + hh * 16, mha_decode8((d0 & 0xffffu) | (d1 << 16), vs[gi][hh]));
-        put(vd + gi * 64 + 32 + hh * 16, mha_decode8((d0 >> 16) | (d1 & 0xffff0000u), vs[gi][hh]));
-      }
+  // decode once per workgroup, into LDS tile buffers `buf`.  V: the thread's 32-group holds 16 stored bytes; operand
+  // piece (t, hh) takes the t-th 16-bit halves of its dwords 2 hh and 2 hh + 1, and the scale of stored block hh.
+  auto stage = [&](int buf, const MhaFetch &f) {
+    uint8_t *kd = mha_lds + buf * MHA_TILE_LDS + srow * MHA_PITCH + sc * 128 + sh * 64;
+    const f16x2 ks = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.ksc, 1.0f, false);
+    const f16x2 kb0 = {ks.x, ks.x}, kb1 = {ks.y, ks.y};
+    *reinterpret_cast<f16x8 *>(kd + 0) = mha_decode8(f.k.x, kb0);
+    *reinterpret_cast<f16x8 *>(kd + 16) = mha_decode8(f.k.y, kb0);
+    *reinterpret_cast<f16x8 *>(kd + 32) = mha_decode8(f.k.z, kb1);
+    *reinterpret_cast<f16x8 *>(kd + 48) = mha_decode8(f.k.w, kb1);
+    uint8_t *vd = mha_lds + (2 + buf) * MHA_TILE_LDS + srow * MHA_PITCH + sc * 128 + sh * 64;
+    const f16x2 vs = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.vsc, 1.0f, false);
+    const f16x2 vb0 = {vs.x, vs.x}, vb1 = {vs.y, vs.y};
+    *reinterpret_cast<f16x8 *>(vd + 0) = mha_decode8((f.v.x & 0xffffu) | (f.v.y << 16), vb0);           // t 0, hh 0
+    *reinterpret_cast<f16x8 *>(vd + 16) = mha_decode8((f.v.z & 0xffffu) | (f.v.w << 16), vb1);          // t 0, hh 1
+    *reinterpret_cast<f16x8 *>(vd + 32) = mha_decode8((f.v.x >> 16) | (f.v.y & 0xffff0000u), vb0);      // t 1, hh 0
+    *reinterpret_cast<f16x8 *>(vd + 48) = mha_decode8((f.v.z >> 16) | (f.v.w & 0xffff0000u), vb1);      // t 1, hh 1
   };
 
   // Qhat of the lane's row: 8 operands of 16 k (chunk c, sub-step s), kept for the whole kernel
@@ -170,30 +174,29 @@ __global__ __launch_bounds__(256) void mha_nvfp4_fwd_d128_kernel(MhaArgs a) {
   int buf = 0;
   for (int64_t n0 = 0; n0 < a.Nkv; n0 += 128, buf ^= 1) {
     fetch(n0 + 128, nxt);  // the next tile's packed bytes travel while this one is multiplied (zeros past the end)
-    const uint8_t *kb = mha_lds + buf * 2 * MHA_TILE_LDS + r * MHA_PITCH + h * 64;
-    const uint8_t *vb = mha_lds + (buf * 2 + 1) * MHA_TILE_LDS + r * MHA_PITCH + h * 16;
+    const uint8_t *kb = mha_lds + buf * MHA_TILE_LDS + r * MHA_PITCH + h * 64;
+    const uint8_t *vb = mha_lds + (2 + buf) * MHA_TILE_LDS + r * MHA_PITCH + h * 16;
     // ---- S^T = Khat . Qhat^T for the 128 kv positions of the tile (four 32-row fragments)
     f32x16 ST[4];
 #pragma unroll
-    for (int f = 0; f < 4; ++f) {
+    for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) ST[f][e] = 0.0f;
+      for (int s = 0; s < 4; ++s)
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
+        for (int f = 0; f < 4; ++f) {  // consecutive MFMAs go to different accumulators
           const f16x8 KF = *reinterpret_cast<const f16x8 *>(kb + f * 32 * MHA_PITCH + c * 128 + s * 16);
-          ST[f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(KF, QF[c][s], ST[f], 0, 0, 0);
+          if (c == 0 && s == 0)
+            ST[f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(KF, QF[c][s], (f32x16)(0.0f), 0, 0, 0);
+          else
+            ST[f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(KF, QF[c][s], ST[f], 0, 0, 0);
         }
-    }
     // ---- online softmax of the lane's row: its 64 values here, the other 64 in the lane 32 away
     float mx = -__builtin_inff();
 #pragma unroll
     for (int f = 0; f < 4; ++f)
 #pragma unroll
       for (int e = 0; e < 16; ++e) mx = __builtin_fmaxf(mx, ST[f][e]);
-    mx = __builtin_fmaxf(mx, mha_xor32(mx));
-    const float ml = __builtin_fmaxf(ml_run, mx * cs);
+    const float ml = __builtin_fmaxf(ml_run, mha_halves_max(mx) * cs);
     float lsum = 0.0f;
 #pragma unroll
     for (int f = 0; f < 4; ++f)
@@ -202,16 +205,16 @@ __global__ __launch_bounds__(256) void mha_nvfp4_fwd_d128_kernel(MhaArgs a) {
         ST[f][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(ST[f][e], cs, -ml));  // p
         lsum += ST[f][e];
       }
-    float l_new = lsum + mha_xor32(lsum);
-    if (n0 + 128 > a.Nkv)  // the zero-filled positions of the last tile each added exp(0 - m)
-      l_new -= (float)(n0 + 128 - a.Nkv) / __builtin_amdgcn_exp2f(ml);
+    const float l_new = mha_halves_sum(lsum);
     const float alpha = __builtin_amdgcn_exp2f(ml_run - ml);
     l_run = alpha * l_run + l_new;
     ml_run = ml;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {  // else no row of this wave raised its maximum
 #pragma unroll
-    for (int fd = 0; fd < 4; ++fd)
+      for (int fd = 0; fd < 4; ++fd)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) OT[fd][e] *= alpha;
+        for (int e = 0; e < 16; ++e) OT[fd][e] *= alpha;
+    }
 
     // ---- P -> NVFP4 (the lane's 16 values of a fragment are one block), then O^T += Vhat . Phat^T
 #pragma unroll
@@ -219,11 +222,10 @@ __global__ __launch_bounds__(256) void mha_nvfp4_fwd_d128_kernel(MhaArgs a) {
       float bm = ST[f][0];
 #pragma unroll
       for (int e = 1; e < 16; ++e) bm = __builtin_fmaxf(bm, ST[f][e]);
-      const uint32_t code = f32_to_ue4m3_satfinite(MHA_P_ALPHA * (bm * 0.16666666666666666f));
-      const float s = e4m3_to_f32(code);
-      const float o = s != 0.0f ? MHA_P_ALPHA * (1.0f / s) : 0.0f;
-      const _Float16 sh = (_Float16)s;  // an e4m3 value: exact in fp16
-      const f16x2 psc = {sh, sh};
+      uint32_t code;
+      const float o = nvfp4_block_scale(bm, MHA_P_ALPHA, lut, code);  // 2688 / e4m3(2688 * (bm / 6)), 0 for code 0
+      const f16x2 s2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(code, 1.0f, false);
+      const f16x2 psc = {s2.x, s2.x};
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         // k slots of this step in the order the stored nibbles of V come in (see the header)
@@ -241,6 +243,8 @@ __global__ __launch_bounds__(256) void mha_nvfp4_fwd_d128_kernel(MhaArgs a) {
     __syncthreads();
   }
 
+  // the zero-filled kv positions of the last tile each added exp(0 - m) to the row sum
+  if (a.Nkv % 128 != 0) l_run -= (float)(128 - a.Nkv % 128) / __builtin_amdgcn_exp2f(ml_run);
   // ---- O = O * ((1/l) * (1/2688) * v_gs) -> bf16
   if (m >= a.Nq) return;
   const float scale = (1.0f / l_run) * (1.0f / MHA_P_ALPHA) * (*a.v_gs);
@@ -279,7 +283,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_mha_nvfp4_fwd(
                (long long)Dqk, (long long)Dv);
   AC4K_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) == 0 && (((uintptr_t)q_sf | (uintptr_t)k_sf | (uintptr_t)v_sf) & 3) == 0,
                "q, k, v must be 16-byte aligned and the scale tensors 4-byte aligned");
-  AC4K_REQUIRE(H <= 65535 && B <= 65535 && ceil_div(Nq, 128) < (1ll << 31), "problem too large");
+  AC4K_REQUIRE(H <= 65535 && B <= 65535 && ceil_div(Nq, MHA_ROWS) < (1ll << 31), "problem too large");
   AC4K_REQUIRE(o_b_stride >= 0 && o_h_stride >= 0 && o_n_stride >= 1 && o_d_stride >= 1, "strides of O must be positive");
   MhaArgs a{static_cast<uint16_t *>(O), o_b_stride, o_h_stride, o_n_stride, o_d_stride,
             static_cast<const uint8_t *>(q), static_cast<const uint8_t *>(k), static_cast<const uint8_t *>(v),
@@ -298,7 +302,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_mha_nvfp4_fwd(
       lds_done.fetch_or(bit, std::memory_order_relaxed);
     }
   }
-  hipLaunchKernelGGL(mha_nvfp4_fwd_d128_kernel, dim3((unsigned)ceil_div(Nq, 128), (unsigned)H, (unsigned)B), dim3(256),
+  hipLaunchKernelGGL(mha_nvfp4_fwd_d128_kernel, dim3((unsigned)ceil_div(Nq, MHA_ROWS), (unsigned)H, (unsigned)B), dim3(64 * MHA_WAVES),
                      MHA_LDS_BYTES, (hipStream_t)stream, a);
   return check_launch("ac4k_mha_nvfp4_fwd");
 }
