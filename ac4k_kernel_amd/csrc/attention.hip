@@ -85,8 +85,6 @@ __device__ __forceinline__ float mha_halves_sum(float x) { return x + __shfl_xor
 constexpr int MHA_PITCH = 272;                   // bytes per decoded row in LDS: 128 fp16 + 16 (bank spread)
 constexpr int MHA_TILE_LDS = 128 * MHA_PITCH;    // one decoded operand tile: K 128 kv rows, V 128 d rows
 constexpr int MHA_LDS_BYTES = 4 * MHA_TILE_LDS;  // K tiles j & 1 at 0 and MHA_TILE_LDS, V tiles j & 1 behind them
-constexpr int MHA_WAVES = 8;                     // waves per workgroup, 32 query rows each
-constexpr int MHA_ROWS = 32 * MHA_WAVES;         // query rows per workgroup
 
 // what one thread fetches per kv tile: a quarter of a packed K row (two 16-blocks), a quarter of a packed V row of
 // the tile (one 32-group of kv positions), and the two scale bytes of each
@@ -95,15 +93,21 @@ struct MhaFetch {
   uint32_t ksc, vsc;
 };
 
-__global__ __launch_bounds__(64 * MHA_WAVES) void mha_nvfp4_fwd_d128_kernel(MhaArgs a) {
+// WAVES = 8 (256 query rows per workgroup, two waves per SIMD: one wave's MFMAs run under the other's vector work)
+// or 4 (128 query rows, for problems with too few workgroups of 256 rows to fill the GPU)
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void mha_nvfp4_fwd_d128_kernel(MhaArgs a) {
+  constexpr int PARTS = 8 / WAVES;  // staging shares per thread: a tile is 512 quarter rows of K and of V
   extern __shared__ __attribute__((aligned(16))) uint8_t mha_lds[];
   __shared__ float lut[128];  // exact reciprocals of the e4m3 values, as in the quantizer
   load_rcp_table(lut);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
-  // staging role: row of the tile, 64-chunk sc, half sh of the chunk (K: elements 32 sh.., V: 32-group 2 sc + sh)
+  // staging role of share p: row srow + p * (128 / PARTS) of the tile, 64-chunk sc, half sh of the chunk (K:
+  // elements 32 sh.. of the chunk, V: 32-group 2 sc + sh)
   const int srow = threadIdx.x >> 2, sc = (threadIdx.x >> 1) & 1, sh = threadIdx.x & 1;
+  constexpr int PROWS = 128 / PARTS;
   const int64_t b = blockIdx.z, head = blockIdx.y, bh = b * a.H + head;
-  const int64_t m = (int64_t)blockIdx.x * MHA_ROWS + wave * 32 + r;   // this lane's query row
+  const int64_t m = (int64_t)blockIdx.x * (32 * WAVES) + wave * 32 + r;   // this lane's query row
   const int64_t mq = m < a.Nq ? m : a.Nq - 1;                         // rows past Nq read the last row; never stored
   const int64_t v_row_bytes = a.Nkv64 / 2, v_chunks = a.Nkv64 / 64;
 
@@ -112,36 +116,44 @@ __global__ __launch_bounds__(64 * MHA_WAVES) void mha_nvfp4_fwd_d128_kernel(MhaA
   const uint8_t *v_src = a.v + (bh * MHA_D + srow) * v_row_bytes + sc * 32 + sh * 16;
   const uint8_t *vsf_src = a.v_sf + ((bh * v_chunks + sc) * MHA_D + srow) * 4 + sh * 2;
   // rows past Nkv and chunks past the stored length of V are zeros
-  auto fetch = [&](int64_t n0, MhaFetch &f) {
-    const int64_t n = n0 + srow;
-    f.k = f.v = make_uint4(0, 0, 0, 0);
-    f.ksc = f.vsc = 0;
-    if (n < a.Nkv) {
-      f.k = *reinterpret_cast<const uint4 *>(k_src + n * (MHA_D / 2));
-      f.ksc = *reinterpret_cast<const uint16_t *>(ksf_src + n * 4);
-    }
-    if (n0 + 64 * sc < a.Nkv64) {
-      f.v = *reinterpret_cast<const uint4 *>(v_src + n0 / 2);
-      f.vsc = *reinterpret_cast<const uint16_t *>(vsf_src + (n0 / 64) * (MHA_D * 4));
+  auto fetch = [&](int64_t n0, MhaFetch (&fs)[PARTS]) {
+#pragma unroll
+    for (int p = 0; p < PARTS; ++p) {
+      MhaFetch &f = fs[p];
+      const int64_t n = n0 + srow + p * PROWS;
+      f.k = f.v = make_uint4(0, 0, 0, 0);
+      f.ksc = f.vsc = 0;
+      if (n < a.Nkv) {
+        f.k = *reinterpret_cast<const uint4 *>(k_src + n * (MHA_D / 2));
+        f.ksc = *reinterpret_cast<const uint16_t *>(ksf_src + n * 4);
+      }
+      if (n0 + 64 * sc < a.Nkv64) {
+        f.v = *reinterpret_cast<const uint4 *>(v_src + p * PROWS * v_row_bytes + n0 / 2);
+        f.vsc = *reinterpret_cast<const uint16_t *>(vsf_src + p * PROWS * 4 + (n0 / 64) * (MHA_D * 4));
+      }
     }
   };
   // decode once per workgroup, into LDS tile buffers `buf`.  V: the thread's 32-group holds 16 stored bytes; operand
   // piece (t, hh) takes the t-th 16-bit halves of its dwords 2 hh and 2 hh + 1, and the scale of stored block hh.
-  auto stage = [&](int buf, const MhaFetch &f) {
-    uint8_t *kd = mha_lds + buf * MHA_TILE_LDS + srow * MHA_PITCH + sc * 128 + sh * 64;
+  auto stage = [&](int buf, const MhaFetch (&fs)[PARTS]) {
+#pragma unroll
+    for (int p = 0; p < PARTS; ++p) {
+    const MhaFetch &f = fs[p];
+    uint8_t *kd = mha_lds + buf * MHA_TILE_LDS + (srow + p * PROWS) * MHA_PITCH + sc * 128 + sh * 64;
     const f16x2 ks = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.ksc, 1.0f, false);
     const f16x2 kb0 = {ks.x, ks.x}, kb1 = {ks.y, ks.y};
     *reinterpret_cast<f16x8 *>(kd + 0) = mha_decode8(f.k.x, kb0);
     *reinterpret_cast<f16x8 *>(kd + 16) = mha_decode8(f.k.y, kb0);
     *reinterpret_cast<f16x8 *>(kd + 32) = mha_decode8(f.k.z, kb1);
     *reinterpret_cast<f16x8 *>(kd + 48) = mha_decode8(f.k.w, kb1);
-    uint8_t *vd = mha_lds + (2 + buf) * MHA_TILE_LDS + srow * MHA_PITCH + sc * 128 + sh * 64;
+    uint8_t *vd = mha_lds + (2 + buf) * MHA_TILE_LDS + (srow + p * PROWS) * MHA_PITCH + sc * 128 + sh * 64;
     const f16x2 vs = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(f.vsc, 1.0f, false);
     const f16x2 vb0 = {vs.x, vs.x}, vb1 = {vs.y, vs.y};
     *reinterpret_cast<f16x8 *>(vd + 0) = mha_decode8((f.v.x & 0xffffu) | (f.v.y << 16), vb0);           // t 0, hh 0
     *reinterpret_cast<f16x8 *>(vd + 16) = mha_decode8((f.v.z & 0xffffu) | (f.v.w << 16), vb1);          // t 0, hh 1
     *reinterpret_cast<f16x8 *>(vd + 32) = mha_decode8((f.v.x >> 16) | (f.v.y & 0xffff0000u), vb0);      // t 1, hh 0
     *reinterpret_cast<f16x8 *>(vd + 48) = mha_decode8((f.v.z >> 16) | (f.v.w & 0xffff0000u), vb1);      // t 1, hh 1
+    }
   };
 
   // Qhat of the lane's row: 8 operands of 16 k (chunk c, sub-step s), kept for the whole kernel
@@ -167,7 +179,7 @@ __global__ __launch_bounds__(64 * MHA_WAVES) void mha_nvfp4_fwd_d128_kernel(MhaA
 #pragma unroll
     for (int e = 0; e < 16; ++e) OT[fd][e] = 0.0f;
 
-  MhaFetch nxt;
+  MhaFetch nxt[PARTS];
   fetch(0, nxt);
   stage(0, nxt);
   __syncthreads();
@@ -191,12 +203,19 @@ __global__ __launch_bounds__(64 * MHA_WAVES) void mha_nvfp4_fwd_d128_kernel(MhaA
             ST[f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(KF, QF[c][s], ST[f], 0, 0, 0);
         }
     // ---- online softmax of the lane's row: its 64 values here, the other 64 in the lane 32 away
-    float mx = -__builtin_inff();
+    // maxima of the raw values per fragment = per P block: exp2 and the scaling are monotonic, so the largest p of
+    // a block is the p of its largest raw value, bit for bit
+    float bmax[4];
 #pragma unroll
-    for (int f = 0; f < 4; ++f)
+    for (int f = 0; f < 4; ++f) {
+      bmax[f] = ST[f][0];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) mx = __builtin_fmaxf(mx, ST[f][e]);
+      for (int e = 1; e < 16; ++e) bmax[f] = __builtin_fmaxf(bmax[f], ST[f][e]);
+    }
+    const float mx = __builtin_fmaxf(__builtin_fmaxf(bmax[0], bmax[1]), __builtin_fmaxf(bmax[2], bmax[3]));
     const float ml = __builtin_fmaxf(ml_run, mha_halves_max(mx) * cs);
+#pragma unroll
+    for (int f = 0; f < 4; ++f) bmax[f] = __builtin_amdgcn_exp2f(__builtin_fmaf(bmax[f], cs, -ml));
     float lsum = 0.0f;
 #pragma unroll
     for (int f = 0; f < 4; ++f)
@@ -219,11 +238,8 @@ __global__ __launch_bounds__(64 * MHA_WAVES) void mha_nvfp4_fwd_d128_kernel(MhaA
     // ---- P -> NVFP4 (the lane's 16 values of a fragment are one block), then O^T += Vhat . Phat^T
 #pragma unroll
     for (int f = 0; f < 4; ++f) {
-      float bm = ST[f][0];
-#pragma unroll
-      for (int e = 1; e < 16; ++e) bm = __builtin_fmaxf(bm, ST[f][e]);
       uint32_t code;
-      const float o = nvfp4_block_scale(bm, MHA_P_ALPHA, lut, code);  // 2688 / e4m3(2688 * (bm / 6)), 0 for code 0
+      const float o = nvfp4_block_scale(bmax[f], MHA_P_ALPHA, lut, code);  // 2688 / e4m3(2688 * (bm / 6)), 0 for code 0
       const f16x2 s2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(code, 1.0f, false);
       const f16x2 psc = {s2.x, s2.x};
 #pragma unroll
@@ -283,26 +299,30 @@ extern "C" __attribute__((visibility("default"))) int ac4k_mha_nvfp4_fwd(
                (long long)Dqk, (long long)Dv);
   AC4K_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) == 0 && (((uintptr_t)q_sf | (uintptr_t)k_sf | (uintptr_t)v_sf) & 3) == 0,
                "q, k, v must be 16-byte aligned and the scale tensors 4-byte aligned");
-  AC4K_REQUIRE(H <= 65535 && B <= 65535 && ceil_div(Nq, MHA_ROWS) < (1ll << 31), "problem too large");
+  AC4K_REQUIRE(H <= 65535 && B <= 65535 && ceil_div(Nq, 128) < (1ll << 31), "problem too large");
   AC4K_REQUIRE(o_b_stride >= 0 && o_h_stride >= 0 && o_n_stride >= 1 && o_d_stride >= 1, "strides of O must be positive");
   MhaArgs a{static_cast<uint16_t *>(O), o_b_stride, o_h_stride, o_n_stride, o_d_stride,
             static_cast<const uint8_t *>(q), static_cast<const uint8_t *>(k), static_cast<const uint8_t *>(v),
             static_cast<const uint8_t *>(q_sf), static_cast<const uint8_t *>(k_sf), static_cast<const uint8_t *>(v_sf),
             q_gs, k_gs, v_gs, H, Nq, Nkv, align_up(Nq, 16), align_up(Nkv, 16), align_up(Nkv, 64), sm_scale,
             (o_d_stride == 1 && ((uintptr_t)O & 7) == 0 && o_b_stride % 4 == 0 && o_h_stride % 4 == 0 && o_n_stride % 4 == 0) ? 1 : 0};
-  {  // more than 64 KB of dynamic LDS has to be allowed once per device
-    static std::atomic<uint32_t> lds_done{0};
+  // 256 query rows per workgroup unless that leaves most of the GPU's 256 CUs without one
+  const bool wide = ceil_div(Nq, 256) * H * B >= 192 || ceil_div(Nq, 128) * H * B <= ceil_div(Nq, 256) * H * B;
+  auto kern = wide ? mha_nvfp4_fwd_d128_kernel<8> : mha_nvfp4_fwd_d128_kernel<4>;
+  {  // more than 64 KB of dynamic LDS has to be allowed once per device and kernel
+    static std::atomic<uint32_t> lds_done[2] = {{0}, {0}};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) dev = 0;
     const uint32_t bit = 1u << (dev & 31);
-    if (!(lds_done.load(std::memory_order_relaxed) & bit)) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(mha_nvfp4_fwd_d128_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, MHA_LDS_BYTES);
+    if (!(lds_done[wide].load(std::memory_order_relaxed) & bit)) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         MHA_LDS_BYTES);
       if (e != hipSuccess) return set_error("hipFuncSetAttribute(LDS=%d): %s", MHA_LDS_BYTES, hipGetErrorString(e));
-      lds_done.fetch_or(bit, std::memory_order_relaxed);
+      lds_done[wide].fetch_or(bit, std::memory_order_relaxed);
     }
   }
-  hipLaunchKernelGGL(mha_nvfp4_fwd_d128_kernel, dim3((unsigned)ceil_div(Nq, MHA_ROWS), (unsigned)H, (unsigned)B), dim3(64 * MHA_WAVES),
-                     MHA_LDS_BYTES, (hipStream_t)stream, a);
+  const int rows = wide ? 256 : 128;
+  hipLaunchKernelGGL(kern, dim3((unsigned)ceil_div(Nq, rows), (unsigned)H, (unsigned)B), dim3(rows * 2), MHA_LDS_BYTES,
+                     (hipStream_t)stream, a);
   return check_launch("ac4k_mha_nvfp4_fwd");
 }

@@ -33,7 +33,9 @@ def sdpa_fp32(q, k, v, layout):
 
 
 CASES = [(1, 256, 1, 128, "BNHD"), (1, 64, 1, 128, "BNHD"), (2, 100, 3, 128, "BHND"), (1, 33, 2, 128, "BNHD"),
-         (1, 300, 1, 128, "BNHD"), (1, 129, 2, 128, "BHND"), (2, 1, 1, 128, "BNHD"), (1, 1000, 4, 128, "BNHD")]
+         (1, 300, 1, 128, "BNHD"), (1, 129, 2, 128, "BHND"), (2, 1, 1, 128, "BNHD"), (1, 1000, 4, 128, "BNHD"),
+         # enough (query block, head) pairs that the kernel takes 256 query rows per workgroup, ragged last block
+         (1, 300, 200, 128, "BHND"), (2, 513, 100, 128, "BNHD")]
 
 
 @pytest.mark.parametrize("B,N,H,D,layout", CASES)

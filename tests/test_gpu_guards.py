@@ -194,7 +194,7 @@ def test_attention_stays_inside_its_output():
     """The attention kernel writes O through its strides: a BNHD output that is a window inside a pattern-filled
     allocation keeps its surroundings, for query lengths that leave a ragged last tile."""
     import math
-    for (B, Nq, Nkv, H) in ((1, 33, 70, 2), (2, 130, 130, 1)):
+    for (B, Nq, Nkv, H) in ((1, 33, 70, 2), (2, 130, 130, 1), (1, 260, 200, 192)):  # the last: 256-row workgroups
         q = make_input((B, Nq, H, 128), seed=3).cuda()
         k, v = make_input((B, Nkv, H, 128), seed=4).cuda(), make_input((B, Nkv, H, 128), seed=5).cuda()
         qq, kq, vq = ops().quantize(q, 1, 3), ops().quantize(k, 1, 3), ops().quantize(v, 3, 1, swizzle=True)
