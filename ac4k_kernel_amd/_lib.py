@@ -42,6 +42,8 @@ SIGNATURES = {
     "ac4k_linear_nvfp4_fused_bf16": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int,
                                             _i64, _i64, _i64, _vp, _i64, _vp]),
     "ac4k_mha_nvfp4_fwd": (_int, [_vp] + [_i64] * 4 + [_vp] * 9 + [_i64] * 6 + [_f32, _vp]),
+    "ac4k_mha_int8_x_fp8_fwd": (_int, [_vp] + [_i64] * 4 + [_vp, _vp, _int, _vp, _vp, _int, _vp, _vp] + [_i64] * 6 + [_f32, _vp]),
+    "ac4k_quantize_int8_token_block_bf16": (_int, [_vp, _vp, _vp] + [_i64] * 7 + [_int, _vp]),
 }
 
 _lib = None

@@ -304,3 +304,60 @@ def mha_nvfp4_fwd(o, q, q_sf, q_global_scale, k, k_sf, k_global_scale, v, v_sf, 
     _lib.check(_L.ac4k_mha_nvfp4_fwd(o.data_ptr(), *o.stride(), q.data_ptr(), q_sf.data_ptr(), q_global_scale.data_ptr(),
                                      k.data_ptr(), k_sf.data_ptr(), k_global_scale.data_ptr(), v.data_ptr(), v_sf.data_ptr(),
                                      v_global_scale.data_ptr(), B, H, Nq, Nkv, Dqk, Dv, float(sm_scale), _stream()))
+
+
+def mha_int8_x_fp8_fwd(o, q, q_sf, q_quantize_block_size: int, k, k_sf, k_quantize_block_size: int, v, v_sf,
+                       sm_scale: float) -> None:
+    """Checks of mha_int8_x_fp8.cu:982-1044.  o may be a permuted view: only its shape [B,H,Nq,Dv], dtype and
+    device are checked."""
+    _check_tensor(q, torch.int8, "Q")
+    _check(q.dim() == 4, "Q must be a 4D tensor")
+    B, H, Nq, Dqk = q.size(0), q.size(1), q.size(2), q.size(3)
+    _check(Dqk % 16 == 0, "Dqk must be multiple of 16")
+    _check(Dqk <= 128, "Dqk must be less than 128")
+    _check_tensor(q_sf, torch.float32, "Q_SF")
+    _check(q_sf.dim() == 3, "Q_SF must be a 3D tensor")
+    _check(list(q_sf.shape) == [B, H, -(-Nq // q_quantize_block_size)], "Meet invalid Q_SF size")
+    _check_tensor(k, torch.int8, "K")
+    _check(k.dim() == 4, "K must be a 4D tensor")
+    _check(k.size(0) == B, "K must have the same batch size as Q")
+    _check(k.size(1) == H, "K must have the same head number as Q")
+    _check(k.size(3) == Dqk, "K must have the same dim as Q")
+    Nkv = k.size(2)
+    _check_tensor(k_sf, torch.float32, "K_SF")
+    _check(k_sf.dim() == 3, "K_SF must be a 3D tensor")
+    _check(list(k_sf.shape) == [B, H, -(-Nkv // k_quantize_block_size)], "Meet invalid K_SF size")
+    _check_tensor(v, torch.float8_e4m3fn, "V")
+    _check(v.dim() == 4, "V must be a 4D tensor")
+    _check(v.size(0) == B, "V must have the same batch size as Q")
+    _check(v.size(1) == H, "V must have the same head number as Q")
+    Dv = v.size(2)
+    _check(v.size(3) == _align_up(Nkv, 16), "Meet invalid v size(3) with {}=={}", v.size(3), _align_up(Nkv, 16))
+    _check(Dv <= 128, "Dv must be less than 128")
+    _check_tensor(v_sf, torch.float32, "V_SF")
+    _check(v_sf.dim() == 3 and list(v_sf.shape) == [B, H, _align_up(Dv, 16)], "Meet invalid v_sf size")
+    _check(isinstance(o, torch.Tensor) and o.is_cuda, "O must be a CUDA tensor")
+    _check(o.dtype == torch.bfloat16, "O must be a bfloat16 tensor")
+    _check(o.dim() == 4 and list(o.shape) == [B, H, Nq, Dv], "O must be [{}, {}, {}, {}]", B, H, Nq, Dv)
+    if B == 0 or H == 0 or Nq == 0:
+        return
+    _check(Nkv > 0, "K must not be empty")
+    _lib.check(_L.ac4k_mha_int8_x_fp8_fwd(o.data_ptr(), *o.stride(), q.data_ptr(), q_sf.data_ptr(), int(q_quantize_block_size),
+                                          k.data_ptr(), k_sf.data_ptr(), int(k_quantize_block_size), v.data_ptr(),
+                                          v_sf.data_ptr(), B, H, Nq, Nkv, Dqk, Dv, float(sm_scale), _stream()))
+
+
+def quantize_int8_token_block(y, scale, x_bhnd, block: int) -> None:
+    """y int8 [B,H,N,align_up(D,16)], scale fp32 [B,H,ceil(N/block)] <- x bf16 viewed as [B,H,N,D] (any batch, head and
+    token strides, head dim contiguous): the per-token-block quantizer of python/ac4k_kernel/ops/attention.py:18-99."""
+    _check(isinstance(x_bhnd, torch.Tensor) and x_bhnd.is_cuda and x_bhnd.dtype == torch.bfloat16, "x must be a CUDA bfloat16 tensor")
+    _check(x_bhnd.dim() == 4 and x_bhnd.stride(3) == 1, "x must be 4D with a contiguous head dim")
+    B, H, N, D = x_bhnd.shape
+    _check_tensor(y, torch.int8, "y")
+    _check(list(y.shape) == [B, H, N, _align_up(D, 16)], "Meet invalid y size")
+    _check_tensor(scale, torch.float32, "scale")
+    _check(list(scale.shape) == [B, H, -(-N // block)], "Meet invalid scale size")
+    if x_bhnd.numel() == 0:
+        return
+    _lib.check(_L.ac4k_quantize_int8_token_block_bf16(y.data_ptr(), scale.data_ptr(), x_bhnd.data_ptr(), B, H, N, D,
+                                                      x_bhnd.stride(0), x_bhnd.stride(1), x_bhnd.stride(2), int(block), _stream()))

@@ -282,6 +282,260 @@ __global__ __launch_bounds__(64 * WAVES) void mha_nvfp4_fwd_d128_kernel(MhaArgs 
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// INT8 (QK) x FP8 (PV) attention forward, head dim 128 (lib/cuda/sm120/mha_int8_x_fp8.cu:346-975; host :979-1137;
+// interface include/ac4k_kernel/ops.h:18-21):
+//   S = Q . K^T in int32 (exact); s = float(S) * ((sm_scale * log2e) * q_sf[row / q_block] * k_sf[tile])   :476,657-677
+//   kv positions past Nkv are -inf                                                                    :679-700
+//   m = max(rowmax(s) - 7.5, m_old); p = exp2(s - m); l = l * exp2(m_old - m) + sum(p)                 :702-776
+//   P -> e4m3 per element (cvt.rn.satfinite, no scales); O = O * exp2(m_old - m) + Phat . Vhat^T        :323-345,828-880
+//   O * ((1 / l) * v_sf[d]) -> bf16                                                                   :886-905
+// The product Phat . Vhat^T is accumulated in fp32 here (the reference's MMA accumulates each tile in fp16).
+// Same structure as the NVFP4 kernel above: a lane owns one query row (S^T = K . Q^T with v_mfma_i32_32x32x32_i8,
+// O^T = Vhat . Phat^T with v_mfma_f32_32x32x16_fp8_fp8), but nothing has to be decoded: the int8 rows of K and the
+// e4m3 rows of V go from global memory into LDS as they are, and from there into the MFMAs.  V is stored with the
+// 16-group swizzle of quantize(v, 3, N_dim, swizzle=True, precision="fp8e4m3"): stored byte 8 h + 4 (j >> 1) + 2 q
+// + (j & 1) of a 16-group holds kv position 8 q + 4 h + j, so the eight positions that lane half h owns in a
+// 16-group are the contiguous stored bytes [8 h, 8 h + 8): one MFMA operand.
+
+struct Mha8Args {
+  uint16_t *O;
+  int64_t o_b, o_h, o_n, o_d;  // element strides of O [B, H, Nq, 128]
+  const int8_t *q, *k;
+  const uint8_t *v;
+  const float *q_sf, *k_sf, *v_sf;
+  int64_t H, Nq, Nkv, Nkv16, nqb, nkb;  // stored kv length of V (16), scales per head of Q and K
+  int q_block;
+  float sm_scale;
+  int o_vec;
+};
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int MHA8_PITCH = 144;                    // bytes per 128-byte row in LDS (bank spread)
+constexpr int MHA8_TILE_LDS = 128 * MHA8_PITCH;    // K tile: 128 kv rows; V tile: 128 d rows
+constexpr int MHA8_LDS_BYTES = 4 * MHA8_TILE_LDS;  // K tiles j & 1, then V tiles j & 1
+constexpr float MHA8_EXP_OFFSET = 7.5f;
+
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_d128_kernel(Mha8Args a) {
+  constexpr int PARTS = 8 / WAVES, PROWS = 128 / PARTS;
+  extern __shared__ __attribute__((aligned(16))) uint8_t mha_lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
+  const int srow = threadIdx.x >> 2, sq = threadIdx.x & 3;  // staging role: row of the tile, 32-byte quarter of it
+  const int64_t b = blockIdx.z, head = blockIdx.y, bh = b * a.H + head;
+  const int64_t m = (int64_t)blockIdx.x * (32 * WAVES) + wave * 32 + r;  // this lane's query row
+  const int64_t mq = m < a.Nq ? m : a.Nq - 1;                            // rows past Nq read the last row; never stored
+
+  const int8_t *k_src = a.k + bh * a.Nkv * MHA_D + sq * 32;
+  const uint8_t *v_src = a.v + (bh * MHA_D + srow) * a.Nkv16 + sq * 32;
+  struct Fetch {
+    uint4 k0, k1, v0, v1;
+  };
+  // rows of K past Nkv and 16-groups of V past its stored length are zeros
+  auto fetch = [&](int64_t n0, Fetch (&fs)[PARTS]) {
+#pragma unroll
+    for (int p = 0; p < PARTS; ++p) {
+      Fetch &f = fs[p];
+      const int64_t n = n0 + srow + p * PROWS;
+      f.k0 = f.k1 = f.v0 = f.v1 = make_uint4(0, 0, 0, 0);
+      if (n < a.Nkv) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(k_src + n * MHA_D);
+        f.k0 = src[0];
+        f.k1 = src[1];
+      }
+      const uint8_t *vs = v_src + p * PROWS * a.Nkv16 + n0;
+      if (n0 + sq * 32 < a.Nkv16) f.v0 = *reinterpret_cast<const uint4 *>(vs);
+      if (n0 + sq * 32 + 16 < a.Nkv16) f.v1 = *reinterpret_cast<const uint4 *>(vs + 16);
+    }
+  };
+  // K rows as they are; V: the thread's two 16-groups (2 sq, 2 sq + 1) regrouped so that the 8-byte pieces of lane
+  // half hh of both are one 16-byte run at 32 sq + 16 hh
+  auto stage = [&](int buf, const Fetch (&fs)[PARTS]) {
+#pragma unroll
+    for (int p = 0; p < PARTS; ++p) {
+      const Fetch &f = fs[p];
+      uint8_t *kd = mha_lds + buf * MHA8_TILE_LDS + (srow + p * PROWS) * MHA8_PITCH + sq * 32;
+      *reinterpret_cast<uint4 *>(kd) = f.k0;
+      *reinterpret_cast<uint4 *>(kd + 16) = f.k1;
+      uint8_t *vd = mha_lds + (2 + buf) * MHA8_TILE_LDS + (srow + p * PROWS) * MHA8_PITCH + sq * 32;
+      *reinterpret_cast<uint4 *>(vd) = make_uint4(f.v0.x, f.v0.y, f.v1.x, f.v1.y);
+      *reinterpret_cast<uint4 *>(vd + 16) = make_uint4(f.v0.z, f.v0.w, f.v1.z, f.v1.w);
+    }
+  };
+
+  // Q of the lane's row: the 16 bytes [32 s + 16 h, +16) of k-step s, kept for the whole kernel
+  i32x4 QF[4];
+#pragma unroll
+  for (int s4 = 0; s4 < 4; ++s4)
+    QF[s4] = *reinterpret_cast<const i32x4 *>(a.q + (bh * a.Nq + mq) * MHA_D + s4 * 32 + h * 16);
+  const float qs = (a.sm_scale * MHA_LOG2E) * a.q_sf[bh * a.nqb + mq / a.q_block];
+
+  float m_run = -__builtin_inff(), l_run = 0.0f;  // running maximum (held 7.5 below the row maximum) and row sum
+  f32x16 OT[4];  // O^T: d = 32 fd + 8 (e >> 2) + 4 h + (e & 3), for the lane's query row
+#pragma unroll
+  for (int fd = 0; fd < 4; ++fd)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) OT[fd][e] = 0.0f;
+
+  Fetch nxt[PARTS];
+  fetch(0, nxt);
+  stage(0, nxt);
+  __syncthreads();
+  int buf = 0;
+  for (int64_t n0 = 0; n0 < a.Nkv; n0 += 128, buf ^= 1) {
+    fetch(n0 + 128, nxt);  // the next tile travels while this one is multiplied (zeros past the end)
+    const uint8_t *kb = mha_lds + buf * MHA8_TILE_LDS + r * MHA8_PITCH + h * 16;
+    const uint8_t *vb = mha_lds + (2 + buf) * MHA8_TILE_LDS + r * MHA8_PITCH + h * 16;
+    const float qk = qs * a.k_sf[bh * a.nkb + n0 / 128];
+    // ---- S^T = K . Q^T for the 128 kv positions of the tile (four 32-row fragments)
+    i32x16 SI[4];
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+      for (int f = 0; f < 4; ++f) {
+        const i32x4 KF = *reinterpret_cast<const i32x4 *>(kb + f * 32 * MHA8_PITCH + s4 * 32);
+        if (s4 == 0)
+          SI[f] = __builtin_amdgcn_mfma_i32_32x32x32_i8(KF, QF[s4], (i32x16)(0), 0, 0, 0);
+        else
+          SI[f] = __builtin_amdgcn_mfma_i32_32x32x32_i8(KF, QF[s4], SI[f], 0, 0, 0);
+      }
+    // ---- online softmax of the lane's row: its 64 values here, the other 64 in the lane 32 away
+    float ST[4][16];
+#pragma unroll
+    for (int f = 0; f < 4; ++f)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) ST[f][e] = (float)SI[f][e];
+    const bool tail = n0 + 128 > a.Nkv;
+    if (tail) {  // positions past Nkv take no part in the maximum
+#pragma unroll
+      for (int f = 0; f < 4; ++f)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          if (n0 + f * 32 + (e >> 2) * 8 + h * 4 + (e & 3) >= a.Nkv) ST[f][e] = -__builtin_inff();
+    }
+    // the maximum of s = float(S) * qk is taken over float(S): qk >= 0 keeps the order, qk < 0 reverses it
+    float hi = -__builtin_inff(), lo = __builtin_inff();
+#pragma unroll
+    for (int f = 0; f < 4; ++f)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) hi = __builtin_fmaxf(hi, ST[f][e]);
+    if (qk < 0.0f) {
+#pragma unroll
+      for (int f = 0; f < 4; ++f)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          lo = __builtin_fminf(lo, ST[f][e] == -__builtin_inff() ? __builtin_inff() : ST[f][e]);
+    }
+    const float smax = qk < 0.0f ? mha_halves_max(lo * qk) : mha_halves_max(hi * qk);
+    const float m_new = __builtin_fmaxf(smax - MHA8_EXP_OFFSET, m_run);
+    float lsum = 0.0f;
+#pragma unroll
+    for (int f = 0; f < 4; ++f)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        ST[f][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(ST[f][e], qk, -m_new));  // p <= 2^7.5
+        lsum += ST[f][e];
+      }
+    if (tail) {  // p of the masked positions is 0 whatever qk is (-inf * 0 would be NaN)
+      lsum = 0.0f;
+#pragma unroll
+      for (int f = 0; f < 4; ++f)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          if (n0 + f * 32 + (e >> 2) * 8 + h * 4 + (e & 3) >= a.Nkv) ST[f][e] = 0.0f;
+          lsum += ST[f][e];
+        }
+    }
+    const float l_new = mha_halves_sum(lsum);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    l_run = __builtin_fmaf(l_run, alpha, l_new);
+    m_run = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {  // else no row of this wave raised its maximum
+#pragma unroll
+      for (int fd = 0; fd < 4; ++fd)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) OT[fd][e] *= alpha;
+    }
+    // ---- P -> e4m3, O^T += Vhat . Phat^T: one MFMA per 16-group G of kv positions and 32 rows of d
+#pragma unroll
+    for (int pj = 0; pj < 4; ++pj) {  // pairs of 16-groups = 32-row fragments of S^T
+      long PF[2];
+#pragma unroll
+      for (int gh = 0; gh < 2; ++gh) {  // k slots in the stored order of V: e = 8 gh + {0, 1, 4, 5, 2, 3, 6, 7}
+        const float *pe = &ST[pj][8 * gh];
+        int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(pe[0], pe[1], 0, false);
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(pe[4], pe[5], w0, true);
+        int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(pe[2], pe[3], 0, false);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(pe[6], pe[7], w1, true);
+        PF[gh] = (long)(((unsigned long)(uint32_t)w1 << 32) | (uint32_t)w0);
+      }
+#pragma unroll
+      for (int fd = 0; fd < 4; ++fd) {
+        const uint4 vv = *reinterpret_cast<const uint4 *>(vb + fd * 32 * MHA8_PITCH + pj * 32);
+        const long v0 = (long)(((unsigned long)vv.y << 32) | vv.x), v1 = (long)(((unsigned long)vv.w << 32) | vv.z);
+        OT[fd] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(v0, PF[0], OT[fd], 0, 0, 0);
+        OT[fd] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(v1, PF[1], OT[fd], 0, 0, 0);
+      }
+    }
+    stage(buf ^ 1, nxt);
+    __syncthreads();
+  }
+
+  // ---- O = O * ((1 / l) * v_sf[d]) -> bf16
+  if (m >= a.Nq) return;
+  const float rl = 1.0f / l_run;
+  const float *vsf = a.v_sf + bh * MHA_D;
+  uint16_t *orow = a.O + b * a.o_b + head * a.o_h + m * a.o_n;
+#pragma unroll
+  for (int fd = 0; fd < 4; ++fd)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const int d = fd * 32 + q4 * 8 + h * 4;  // four consecutive head dims
+      const float4 sv = *reinterpret_cast<const float4 *>(vsf + d);
+      const float sc[4] = {rl * sv.x, rl * sv.y, rl * sv.z, rl * sv.w};
+      uint32_t o4[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o4[e] = __builtin_bit_cast(uint16_t, (__bf16)(OT[fd][4 * q4 + e] * sc[e]));
+      if (a.o_vec) {
+        *reinterpret_cast<uint2 *>(orow + d) = make_uint2(o4[0] | (o4[1] << 16), o4[2] | (o4[3] << 16));
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) orow[(d + e) * a.o_d] = (uint16_t)o4[e];
+      }
+    }
+}
+
+// Per-token-block int8 quantizer in front of it (python/ac4k_kernel/ops/attention.py:18-99, a Triton kernel in the
+// reference): one scale = max|x| / 127 per block of `block` tokens of a head (all D columns), y = int8(trunc(x /
+// scale)), 0 where the scale is 0; y is [B, H, N, Dp] with pad columns 0, the scales [B, H, ceil(N / block)].
+__global__ __launch_bounds__(256) void quantize_int8_token_block_kernel(int8_t *__restrict__ y, float *__restrict__ scale,
+                                                                        const uint16_t *__restrict__ x, int64_t s_b,
+                                                                        int64_t s_h, int64_t s_n, int64_t H, int64_t N,
+                                                                        int D, int Dp, int block) {
+  __shared__ uint32_t wmax[4];
+  const int64_t nb = gridDim.x, blk = blockIdx.x, head = blockIdx.y, b = blockIdx.z;
+  const int64_t n0 = blk * block;
+  const int rows = (int)((N - n0) < block ? (N - n0) : block);
+  const uint16_t *src = x + b * s_b + head * s_h + n0 * s_n;
+  uint32_t mx = 0;
+  for (int i = threadIdx.x; i < rows * D; i += 256) mx = umax32(mx, src[(int64_t)(i / D) * s_n + i % D] & 0x7fffu);
+  mx = group_umax<64>(mx);
+  if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = umax32(umax32(wmax[0], wmax[1]), umax32(wmax[2], wmax[3]));
+  const float sc = bf16_bits_to_f32(mx) / 127.0f;
+  if (threadIdx.x == 0) scale[(b * H + head) * nb + blk] = sc;
+  int8_t *dst = y + ((b * H + head) * N + n0) * Dp;
+  for (int i = threadIdx.x; i < rows * Dp; i += 256) {
+    const int rr = i / Dp, c = i % Dp;
+    float q = 0.0f;
+    if (c < D && sc != 0.0f) q = bf16_bits_to_f32(src[(int64_t)rr * s_n + c]) / sc;
+    dst[i] = (int8_t)(int)q;  // toward zero; |q| <= 127 up to rounding
+  }
+}
+
 }  // namespace ac4k
 
 using namespace ac4k;
@@ -325,4 +579,65 @@ extern "C" __attribute__((visibility("default"))) int ac4k_mha_nvfp4_fwd(
   hipLaunchKernelGGL(kern, dim3((unsigned)ceil_div(Nq, rows), (unsigned)H, (unsigned)B), dim3(rows * 2), MHA_LDS_BYTES,
                      (hipStream_t)stream, a);
   return check_launch("ac4k_mha_nvfp4_fwd");
+}
+
+// Replaces ac4k::mha_int8_x_fp8_fwd (lib/cuda/sm120/mha_int8_x_fp8.cu:979-1137).
+extern "C" __attribute__((visibility("default"))) int ac4k_mha_int8_x_fp8_fwd(
+    void *O, int64_t o_b_stride, int64_t o_h_stride, int64_t o_n_stride, int64_t o_d_stride, const void *q,
+    const float *q_sf, int q_quantize_block_size, const void *k, const float *k_sf, int k_quantize_block_size, const void *v,
+    const float *v_sf, int64_t B, int64_t H, int64_t Nq, int64_t Nkv, int64_t Dqk, int64_t Dv, float sm_scale,
+    ac4k_stream_t stream) {
+  AC4K_REQUIRE(O && q && q_sf && k && k_sf && v && v_sf, "null pointer argument");
+  AC4K_REQUIRE(B >= 1 && H >= 1 && Nq >= 1 && Nkv >= 1, "B, H, Nq, Nkv must be positive (B=%lld H=%lld Nq=%lld Nkv=%lld)",
+               (long long)B, (long long)H, (long long)Nq, (long long)Nkv);
+  AC4K_REQUIRE(Dqk % 16 == 0, "Dqk must be multiple of 16");
+  AC4K_REQUIRE(Dqk <= 128 && Dv <= 128, "Dqk and Dv must not exceed 128");
+  AC4K_REQUIRE(q_quantize_block_size == 32 || q_quantize_block_size == 64, "q_quantize_block_size must be 32 or 64 (got %d)",
+               q_quantize_block_size);
+  AC4K_REQUIRE(k_quantize_block_size == 128, "k_quantize_block_size must be 128 (got %d)", k_quantize_block_size);
+  AC4K_REQUIRE(Dqk == MHA_D && Dv == MHA_D, "this build of the attention kernel takes head dim 128 only (Dqk=%lld Dv=%lld)",
+               (long long)Dqk, (long long)Dv);
+  AC4K_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)v_sf) & 15) == 0,
+               "q, k, v and v_sf must be 16-byte aligned");
+  AC4K_REQUIRE(H <= 65535 && B <= 65535 && ceil_div(Nq, 128) < (1ll << 31), "problem too large");
+  AC4K_REQUIRE(o_b_stride >= 0 && o_h_stride >= 0 && o_n_stride >= 1 && o_d_stride >= 1, "strides of O must be positive");
+  Mha8Args a{static_cast<uint16_t *>(O), o_b_stride, o_h_stride, o_n_stride, o_d_stride,
+             static_cast<const int8_t *>(q), static_cast<const int8_t *>(k), static_cast<const uint8_t *>(v),
+             q_sf, k_sf, v_sf, H, Nq, Nkv, align_up(Nkv, 16), ceil_div(Nq, q_quantize_block_size), ceil_div(Nkv, 128),
+             q_quantize_block_size, sm_scale,
+             (o_d_stride == 1 && ((uintptr_t)O & 7) == 0 && o_b_stride % 4 == 0 && o_h_stride % 4 == 0 && o_n_stride % 4 == 0) ? 1 : 0};
+  const bool wide = ceil_div(Nq, 256) * H * B >= 192 || ceil_div(Nq, 128) * H * B <= ceil_div(Nq, 256) * H * B;
+  auto kern = wide ? mha_int8_x_fp8_fwd_d128_kernel<8> : mha_int8_x_fp8_fwd_d128_kernel<4>;
+  {  // more than 64 KB of dynamic LDS has to be allowed once per device and kernel
+    static std::atomic<uint32_t> lds_done[2] = {{0}, {0}};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    const uint32_t bit = 1u << (dev & 31);
+    if (!(lds_done[wide].load(std::memory_order_relaxed) & bit)) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         MHA8_LDS_BYTES);
+      if (e != hipSuccess) return set_error("hipFuncSetAttribute(LDS=%d): %s", MHA8_LDS_BYTES, hipGetErrorString(e));
+      lds_done[wide].fetch_or(bit, std::memory_order_relaxed);
+    }
+  }
+  const int rows = wide ? 256 : 128;
+  hipLaunchKernelGGL(kern, dim3((unsigned)ceil_div(Nq, rows), (unsigned)H, (unsigned)B), dim3(rows * 2), MHA8_LDS_BYTES,
+                     (hipStream_t)stream, a);
+  return check_launch("ac4k_mha_int8_x_fp8_fwd");
+}
+
+// Replaces _int8_quantize / _triton_block_token_quantize (python/ac4k_kernel/ops/attention.py:18-99): x bf16 with element
+// strides (s_b, s_h, s_n, 1) over [B, H, N, D] -> y int8 [B, H, N, align_up(D, 16)], scale fp32 [B, H, ceil(N / block)].
+extern "C" __attribute__((visibility("default"))) int ac4k_quantize_int8_token_block_bf16(
+    void *y, float *scale, const void *x, int64_t B, int64_t H, int64_t N, int64_t D, int64_t s_b, int64_t s_h, int64_t s_n,
+    int block, ac4k_stream_t stream) {
+  AC4K_REQUIRE(y && scale && x, "null pointer argument");
+  AC4K_REQUIRE(B >= 1 && H >= 1 && N >= 1 && D >= 1, "B, H, N, D must be positive");
+  AC4K_REQUIRE(block >= 16 && (block & (block - 1)) == 0, "the block size must be a power of two, at least 16 (got %d)", block);
+  AC4K_REQUIRE(D <= 1024 && block <= 1024, "D and the block size must not exceed 1024");
+  AC4K_REQUIRE(H <= 65535 && B <= 65535 && ceil_div(N, (int64_t)block) < (1ll << 31), "problem too large");
+  hipLaunchKernelGGL(quantize_int8_token_block_kernel, dim3((unsigned)ceil_div(N, (int64_t)block), (unsigned)H, (unsigned)B),
+                     dim3(256), 0, (hipStream_t)stream, static_cast<int8_t *>(y), scale, static_cast<const uint16_t *>(x), s_b,
+                     s_h, s_n, H, N, (int)D, (int)align_up(D, 16), block);
+  return check_launch("ac4k_quantize_int8_token_block_bf16");
 }

@@ -217,13 +217,37 @@ int ac4k_linear_nvfp4_fused_bf16(void *D, int d_dtype, const void *X, void *X_q,
  * v_sf [B,H,align_up(Nkv,64)/64,align_up(Dv,16),4]; the three global scales are device scalars;
  * O bf16 [B,H,Nq,Dv] addressed through its four element strides (the reference passes a permuted view).
  * The attention probabilities are re-quantized to NVFP4 per 16-block with the global scale 1/2688, as in
- * mha_nvfp4.cu:248-319.  First slice of this operator: head dim 128 only (Dqk == Dv == 128; the reference
- * takes any multiple of 16 up to 128), correctness first, not tuned. */
+ * mha_nvfp4.cu:248-319.  Head dim 128 only (Dqk == Dv == 128; the reference takes any multiple of 16 up to 128). */
 int ac4k_mha_nvfp4_fwd(void *O, int64_t o_b_stride, int64_t o_h_stride, int64_t o_n_stride,
                        int64_t o_d_stride, const void *q, const void *q_sf, const float *q_gs,
                        const void *k, const void *k_sf, const float *k_gs, const void *v,
                        const void *v_sf, const float *v_gs, int64_t B, int64_t H, int64_t Nq,
                        int64_t Nkv, int64_t Dqk, int64_t Dv, float sm_scale, ac4k_stream_t stream);
+
+/* Replaces ac4k::mha_int8_x_fp8_fwd (include/ac4k_kernel/ops.h:18-21, lib/cuda/sm120/mha_int8_x_fp8.cu:979-1137):
+ * O = softmax(Q K^T * sm_scale) V with Q K^T on int8 and P V on e4m3.
+ * q int8 [B,H,Nq,Dqk], q_sf fp32 [B,H,ceil(Nq/q_quantize_block_size)] (block 32 or 64);
+ * k int8 [B,H,Nkv,Dqk], k_sf fp32 [B,H,ceil(Nkv/128)] (k_quantize_block_size must be 128);
+ * v e4m3 [B,H,Dv,align_up(Nkv,16)] quantized per (head, d) row along kv with the 16-group swizzle
+ * (quantize(v, 3, N_dim, swizzle=True, max_scale=2.25, precision="fp8e4m3")), v_sf fp32 [B,H,align_up(Dv,16)];
+ * O bf16 [B,H,Nq,Dv] addressed through its four element strides.  The probabilities are held up to 2^7.5 and
+ * converted to e4m3 per element (mha_int8_x_fp8.cu:718-736,323-345); P V accumulates in fp32 (the reference's MMA
+ * accumulates each kv tile in fp16).  Head dim 128 only (the reference takes any multiple of 16 up to 128). */
+int ac4k_mha_int8_x_fp8_fwd(void *O, int64_t o_b_stride, int64_t o_h_stride, int64_t o_n_stride,
+                            int64_t o_d_stride, const void *q, const float *q_sf,
+                            int q_quantize_block_size, const void *k, const float *k_sf,
+                            int k_quantize_block_size, const void *v, const float *v_sf, int64_t B,
+                            int64_t H, int64_t Nq, int64_t Nkv, int64_t Dqk, int64_t Dv, float sm_scale,
+                            ac4k_stream_t stream);
+
+/* Replaces _int8_quantize / _triton_block_token_quantize (python/ac4k_kernel/ops/attention.py:18-99), the
+ * quantizer of Q and K in front of ac4k_mha_int8_x_fp8_fwd: x bf16 [B,H,N,D] with element strides
+ * (s_b, s_h, s_n, 1) -> y int8 [B,H,N,align_up(D,16)] (pad columns 0), scale fp32 [B,H,ceil(N/block)];
+ * one scale = max|x| / 127 per block of `block` tokens of a head, y = int8(trunc(x / scale)), 0 where the
+ * scale is 0.  block: a power of two, at least 16. */
+int ac4k_quantize_int8_token_block_bf16(void *y, float *scale, const void *x, int64_t B, int64_t H,
+                                        int64_t N, int64_t D, int64_t s_b, int64_t s_h, int64_t s_n,
+                                        int block, ac4k_stream_t stream);
 
 #ifdef __cplusplus
 }

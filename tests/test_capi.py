@@ -109,7 +109,7 @@ def test_reference_import_lines_resolve():
     import ac4k_kernel
     import ac4k_kernel_amd
     from ac4k_kernel.ops import attention, linear, quantize
-    from ac4k_kernel.ops.attention import mha_nvfp4_fwd
+    from ac4k_kernel.ops.attention import mha_int8_x_fp8_fwd, mha_nvfp4_fwd
     from ac4k_kernel.ops.linear import Ac4kLinearOp
     from ac4k_kernel.ops.quant import Ac4kQuantizeOp
     import ac4k_kernel._rocm_ops as binding
@@ -117,6 +117,7 @@ def test_reference_import_lines_resolve():
     assert ac4k_kernel.get_info() == ac4k_kernel_amd.get_info()
     assert quantize is ac4k_kernel_amd.ops.quantize and linear is ac4k_kernel_amd.ops.linear
     assert attention is ac4k_kernel_amd.ops.attention and mha_nvfp4_fwd is binding.mha_nvfp4_fwd
+    assert mha_int8_x_fp8_fwd is binding.mha_int8_x_fp8_fwd
     assert binding is ac4k_kernel_amd._rocm_ops and binding.__backend__ == "rocm"
     assert issubclass(Ac4kLinearOp, __import__("torch").nn.Module) and Ac4kQuantizeOp is not None
     for name in ("quantize_nvfp4", "quantize_fp8", "quantize_int8", "linear_nvfp4"):

@@ -82,10 +82,11 @@ def test_mha_entry_point_on_given_operands_and_out_argument():
 def test_attention_argument_checks():
     o = ops()
     q = make_input((1, 16, 1, 128), seed=1).cuda()
-    with pytest.raises(NotImplementedError):
-        o.attention(q, q, q, precision="int8+fp8e4m3")
+    with pytest.raises(AssertionError):
+        o.attention(q, q, q, precision="fp16")
     with pytest.raises(AssertionError):
         o.attention(q.float(), q, q)
     q64 = make_input((1, 16, 1, 64), seed=1).cuda()
-    with pytest.raises(RuntimeError):  # head dim 64: refused by this build with a message
-        o.attention(q64, q64, q64)
+    for precision in ("nvfp4", "int8+fp8e4m3"):
+        with pytest.raises(RuntimeError, match="head dim 128"):  # head dim 64: refused by this build with a message
+            o.attention(q64, q64, q64, precision=precision)

@@ -204,3 +204,18 @@ def test_attention_stays_inside_its_output():
         ops().mha_nvfp4_fwd(w.t.permute(0, 2, 1, 3), *qq, *kq, *vq, 1 / math.sqrt(128))
         torch.cuda.synchronize()
         assert w.intact() and same_bytes(w.t, ref)
+        # the int8 x fp8 attention on the same shapes, and its quantizer's outputs
+        import importlib
+        front = importlib.import_module("ac4k_kernel_amd.ops.attention")
+        q8, q_sf = front._int8_quantize(q, "BNHD", 1, BLOCK_SIZE=64)
+        k8, k_sf = front._int8_quantize(k, "BNHD", 1, BLOCK_SIZE=128)
+        v8, v_sf = ops().quantize(v, 3, 1, swizzle=True, max_scale=2.25, precision="fp8e4m3")
+        ops().mha_int8_x_fp8_fwd(ref.permute(0, 2, 1, 3), q8, q_sf, 64, k8, k_sf, 128, v8, v_sf, 1 / math.sqrt(128))
+        w = Window((B, Nq, H, 128), torch.bfloat16)
+        ops().mha_int8_x_fp8_fwd(w.t.permute(0, 2, 1, 3), q8, q_sf, 64, k8, k_sf, 128, v8, v_sf, 1 / math.sqrt(128))
+        wy, ws = Window(tuple(q8.shape), torch.int8), Window(tuple(q_sf.shape), torch.float32)
+        from ac4k_kernel_amd import _rocm_ops
+        _rocm_ops.quantize_int8_token_block(wy.t, ws.t, q.permute(0, 2, 1, 3), 64)
+        torch.cuda.synchronize()
+        assert w.intact() and same_bytes(w.t, ref)
+        assert wy.intact() and ws.intact() and same_bytes(wy.t, q8) and same_bytes(ws.t, q_sf)

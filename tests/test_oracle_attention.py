@@ -100,3 +100,91 @@ def test_output_is_linear_in_v_global_scale_and_invariant_to_row_order():
     ops3[1] = sfq
     o3 = A.mha_nvfp4_fwd(*ops3, 0.1).float()
     assert torch.equal(o3, o1[:, :, perm])
+
+
+# --------------------------------------------------------------------------- INT8 (QK) x FP8 (PV)
+def _sdpa(q, k, v, layout):
+    q, k, v = (t.float() for t in (q, k, v))
+    if layout == "BNHD":
+        q, k, v = (t.transpose(1, 2) for t in (q, k, v))
+    o = torch.softmax(q @ k.transpose(-1, -2) / math.sqrt(q.shape[-1]), dim=-1) @ v
+    return o.transpose(1, 2).contiguous() if layout == "BNHD" else o
+
+
+@pytest.mark.parametrize("B,N,H,layout", [(1, 256, 1, "BNHD"), (1, 100, 1, "BNHD"), (2, 111, 2, "BHND"), (1, 444, 1, "BNHD")])
+def test_int8_x_fp8_oracle_within_the_reference_tolerance_of_fp32_attention(B, N, H, layout):
+    """The end-to-end pin the reference itself uses for this operator (test/test_attention_bench.py:69-177, its
+    D = 128 shapes and ragged lengths): atol 0.2, rtol 1e-2, cosine similarity > 0.99 against fp32 attention."""
+    shape = (B, N, H, 128) if layout == "BNHD" else (B, H, N, 128)
+    g = torch.Generator().manual_seed(N)
+    q, k, v = (torch.randn(shape, generator=g).to(torch.bfloat16) for _ in range(3))
+    o = A.attention_int8_x_fp8(q, k, v, layout)
+    ref = _sdpa(q, k, v, layout)
+    cos = torch.nn.functional.cosine_similarity(o.float().flatten(), ref.flatten(), dim=0).item()
+    assert cos > 0.99, cos
+    torch.testing.assert_close(o.float(), ref, atol=2e-1, rtol=1e-2)
+
+
+def test_token_block_quantizer_closed_forms():
+    """One scale per block of tokens = max|x| / 127 over all columns; values truncated toward zero; a zero block
+    gives scale 0 and zeros; the head dim is padded to 16 with zeros; BNHD and BHND agree."""
+    x = torch.zeros((1, 40, 1, 20), dtype=torch.bfloat16)
+    x[0, 0, 0, 3] = 127.0      # block 0 (tokens 0-15): scale 1
+    x[0, 5, 0, 7] = -2.75      # -> trunc(-2.75) = -2 (rounding to nearest would give -3)
+    x[0, 15, 0, 0] = 0.99      # -> 0
+    x[0, 32, 0, 1] = -63.5     # block 2 (tokens 32-39, ragged): scale 0.5 -> -127
+    x[0, 39, 0, 19] = 0.75     # -> trunc(1.5) = 1
+    y, s = A.int8_block_token_quantize(x, "BNHD", 16)
+    assert list(y.shape) == [1, 1, 40, 32] and list(s.shape) == [1, 1, 3]
+    assert s.tolist() == [[[1.0, 0.0, 0.5]]]
+    assert y[0, 0, 0, 3] == 127 and y[0, 0, 5, 7] == -2 and y[0, 0, 15, 0] == 0
+    assert y[0, 0, 32, 1] == -127 and y[0, 0, 39, 19] == 1
+    assert int(y.abs().sum()) == 127 + 2 + 127 + 1 and (y[..., 20:] == 0).all()
+    y2, s2 = A.int8_block_token_quantize(x.permute(0, 2, 1, 3).contiguous(), "BHND", 16)
+    assert torch.equal(y, y2) and torch.equal(s, s2)
+
+
+def test_fp8_deswizzle_inverts_the_quantizer_swizzle():
+    v = torch.arange(64, dtype=torch.float32).reshape(1, 1, 2, 32).to(torch.bfloat16) / 64
+    plain, _ = T.quantize_fp8(v, 2, 3, 448.0, False)
+    swz, _ = T.quantize_fp8(v, 2, 3, 448.0, True)
+    assert not torch.equal(plain, swz)
+    assert torch.equal(A.deswizzle_fp8(swz), plain)
+
+
+def test_int8_x_fp8_kernel_oracle_closed_forms():
+    """Cases a person can evaluate: (1) one kv position: O is the dequantized V row whatever Q and K are;
+    (2) equal scores: O is the mean of the V rows, through the 7.5 offset, p = 2^7.5 -> e4m3(181.02) = 176 for every
+    position, so numerator and denominator scale alike only up to e4m3(p) / p, which the result must show;
+    (3) kv positions past Nkv are masked: appending garbage rows behind Nkv changes nothing."""
+    g = torch.Generator().manual_seed(3)
+    v = torch.randn((1, 1, 1, 128), generator=g).to(torch.bfloat16)           # [B,H,Nkv=1,D]
+    v8, v_sf = T.quantize_fp8(v, 3, 2, 2.25, True)
+    q = torch.randint(-127, 128, (1, 1, 5, 128), generator=g, dtype=torch.int8)
+    k = torch.randint(-127, 128, (1, 1, 1, 128), generator=g, dtype=torch.int8)
+    one = torch.ones((1, 1, 1))
+    o = A.mha_int8_x_fp8_fwd(q, one, 64, k, one, 128, v8, v_sf, 0.01)
+    # p = 2^7.5 -> e4m3 176; l = 181.02; O = 176 / 181.02 * dequant(V)
+    p = torch.exp2(torch.tensor(7.5))
+    vd = T.e4m3_bits_to_f32(v8)[0, 0, :, 0] * v_sf[0, 0]
+    expect = ((176.0 * T.e4m3_bits_to_f32(v8)[0, 0, :, 0]) * ((1.0 / p) * v_sf[0, 0])).to(torch.bfloat16)
+    assert torch.equal(o[0, 0, 0], expect) and torch.equal(o[0, 0, 4], expect)
+    assert torch.allclose(o[0, 0, 0].float(), vd * (176.0 / p), rtol=1e-2)
+    # (2) all scores equal (K = 0): mean of V over 48 positions, times 176 / 2^7.5
+    v = torch.randn((1, 1, 48, 128), generator=g).to(torch.bfloat16)
+    v8, v_sf = T.quantize_fp8(v, 3, 2, 2.25, True)
+    k0 = torch.zeros((1, 1, 48, 128), dtype=torch.int8)
+    o = A.mha_int8_x_fp8_fwd(q, one, 64, k0, one, 128, v8, v_sf, 0.01)
+    vdq = A.deswizzle_fp8(T.e4m3_bits_to_f32(v8))[0, 0, :, :48] * v_sf[0, 0, :, None]     # [D, 48]
+    assert torch.allclose(o[0, 0, 2].float(), vdq.mean(dim=1) * (176.0 / p), atol=4e-3, rtol=1e-2)
+    # (3) the masked tail: V is stored to a multiple of 16, K rows behind Nkv do not exist; a longer K / V pair that
+    # agrees on the first 40 positions gives another result, the same pair cut to 40 the same one
+    k = torch.randint(-127, 128, (1, 1, 48, 128), generator=g, dtype=torch.int8)
+    sf = torch.full((1, 1, 1), 0.02)
+    o48 = A.mha_int8_x_fp8_fwd(q, sf, 64, k, sf, 128, v8, v_sf, 0.05)
+    v40 = v[:, :, :40]
+    v8c, v_sfc = T.quantize_fp8(v40, 3, 2, 2.25, True)
+    o40 = A.mha_int8_x_fp8_fwd(q, sf, 64, k[:, :, :40], sf, 128, v8c, v_sfc, 0.05)
+    full = torch.softmax((q.float() @ k[:, :, :40].float().transpose(-1, -2)) * (0.02 * 0.02 * 0.05), -1) @ v40.float()
+    assert not torch.allclose(o48.float(), o40.float(), atol=1e-2)
+    assert torch.allclose(o40.float(), full, atol=5e-2, rtol=5e-2)
