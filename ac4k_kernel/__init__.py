@@ -5,7 +5,7 @@ test/test_quantize_bench.py:7; `from ac4k_kernel.ops import linear, quantize`,
 test/test_linear_bench.py:4; `from ac4k_kernel.ops import attention`, test/test_attention_bench.py:4)
 keep their import lines.  Only the NVFP4 path exists here: the meta API of
 python/ac4k_kernel/__init__.py:58-74, the quantize / linear operators of
-python/ac4k_kernel/ops/__init__.py:5-26 and `attention` (both precisions, head dim 128).  The RoPE and
+python/ac4k_kernel/ops/__init__.py:5-26 and `attention` (both precisions, head dims up to 128).  The RoPE and
 sparse-attention names of the reference are absent, and asking for them raises AttributeError / ImportError.
 """
 import sys as _sys

@@ -1,4 +1,4 @@
-// NVFP4 attention forward for gfx950, head dim 128:  O = softmax(Q K^T * sm_scale) V on NVFP4 operands.
+// NVFP4 attention forward for gfx950, head dims up to 128:  O = softmax(Q K^T * sm_scale) V on NVFP4 operands.
 //
 // Math contract of the reference kernel (lib/cuda/sm120/mha_nvfp4.cu:336-905, host checks :911-1077,
 // interface include/ac4k_kernel/ops.h:12-16):
@@ -33,11 +33,11 @@ struct MhaArgs {
   const uint8_t *q, *k, *v, *q_sf, *k_sf, *v_sf;
   const float *q_gs, *k_gs, *v_gs;
   int64_t H, Nq, Nkv, Nqp, Nkvp, Nkv64;  // padded: rows of the Q / K scale planes (16), stored kv length of V (64)
+  int chunks, Dv, Dvp;                   // 64-chunks of a Q / K row (1 or 2), rows of V, rows of a V scale plane (16)
   float sm_scale;
   int o_vec;  // O rows are contiguous along d and 8-byte aligned: four head dims per store
 };
 
-constexpr int MHA_D = 128;
 constexpr float MHA_LOG2E = 1.4426950408889634f;
 constexpr float MHA_P_ALPHA = 2688.0f;  // 1 / (global scale of P)
 
@@ -96,7 +96,7 @@ struct MhaFetch {
 // WAVES = 8 (256 query rows per workgroup, two waves per SIMD: one wave's MFMAs run under the other's vector work)
 // or 4 (128 query rows, for problems with too few workgroups of 256 rows to fill the GPU)
 template <int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void mha_nvfp4_fwd_d128_kernel(MhaArgs a) {
+__global__ __launch_bounds__(64 * WAVES) void mha_nvfp4_fwd_kernel(MhaArgs a) {
   constexpr int PARTS = 8 / WAVES;  // staging shares per thread: a tile is 512 quarter rows of K and of V
   extern __shared__ __attribute__((aligned(16))) uint8_t mha_lds[];
   __shared__ float lut[128];  // exact reciprocals of the e4m3 values, as in the quantizer
@@ -111,10 +111,12 @@ __global__ __launch_bounds__(64 * WAVES) void mha_nvfp4_fwd_d128_kernel(MhaArgs 
   const int64_t mq = m < a.Nq ? m : a.Nq - 1;                         // rows past Nq read the last row; never stored
   const int64_t v_row_bytes = a.Nkv64 / 2, v_chunks = a.Nkv64 / 64;
 
-  const uint8_t *k_src = a.k + bh * a.Nkv * (MHA_D / 2) + sc * 32 + sh * 16;
-  const uint8_t *ksf_src = a.k_sf + (bh * 2 + sc) * a.Nkvp * 4 + sh * 2;
-  const uint8_t *v_src = a.v + (bh * MHA_D + srow) * v_row_bytes + sc * 32 + sh * 16;
-  const uint8_t *vsf_src = a.v_sf + ((bh * v_chunks + sc) * MHA_D + srow) * 4 + sh * 2;
+  // head dims below 128: the missing chunk of Q and K and the missing rows of V are zeros
+  const int64_t qk_row = a.chunks * 32;  // packed bytes of a Q / K row
+  const uint8_t *k_src = a.k + bh * a.Nkv * qk_row + sc * 32 + sh * 16;
+  const uint8_t *ksf_src = a.k_sf + (bh * a.chunks + sc) * a.Nkvp * 4 + sh * 2;
+  const uint8_t *v_src = a.v + (bh * a.Dv + srow) * v_row_bytes + sc * 32 + sh * 16;
+  const uint8_t *vsf_src = a.v_sf + ((bh * v_chunks + sc) * a.Dvp + srow) * 4 + sh * 2;
   // rows past Nkv and chunks past the stored length of V are zeros
   auto fetch = [&](int64_t n0, MhaFetch (&fs)[PARTS]) {
 #pragma unroll
@@ -123,13 +125,13 @@ __global__ __launch_bounds__(64 * WAVES) void mha_nvfp4_fwd_d128_kernel(MhaArgs 
       const int64_t n = n0 + srow + p * PROWS;
       f.k = f.v = make_uint4(0, 0, 0, 0);
       f.ksc = f.vsc = 0;
-      if (n < a.Nkv) {
-        f.k = *reinterpret_cast<const uint4 *>(k_src + n * (MHA_D / 2));
+      if (n < a.Nkv && sc < a.chunks) {
+        f.k = *reinterpret_cast<const uint4 *>(k_src + n * qk_row);
         f.ksc = *reinterpret_cast<const uint16_t *>(ksf_src + n * 4);
       }
-      if (n0 + 64 * sc < a.Nkv64) {
+      if (n0 + 64 * sc < a.Nkv64 && srow + p * PROWS < a.Dv) {
         f.v = *reinterpret_cast<const uint4 *>(v_src + p * PROWS * v_row_bytes + n0 / 2);
-        f.vsc = *reinterpret_cast<const uint16_t *>(vsf_src + p * PROWS * 4 + (n0 / 64) * (MHA_D * 4));
+        f.vsc = *reinterpret_cast<const uint16_t *>(vsf_src + p * PROWS * 4 + (n0 / 64) * (a.Dvp * 4));
       }
     }
   };
@@ -159,8 +161,12 @@ __global__ __launch_bounds__(64 * WAVES) void mha_nvfp4_fwd_d128_kernel(MhaArgs 
   // Qhat of the lane's row: 8 operands of 16 k (chunk c, sub-step s), kept for the whole kernel
   f16x8 QF[2][4];
 #pragma unroll
-  for (int c = 0; c < 2; ++c)
-    mha_load_row_chunk(a.q + (bh * a.Nq + mq) * (MHA_D / 2), a.q_sf + ((bh * 2 + c) * a.Nqp + mq) * 4, c, h, QF[c]);
+  for (int c = 0; c < 2; ++c) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) QF[c][s] = (f16x8)((_Float16)0);
+    if (c < a.chunks)
+      mha_load_row_chunk(a.q + (bh * a.Nq + mq) * qk_row, a.q_sf + ((bh * a.chunks + c) * a.Nqp + mq) * 4, c, h, QF[c]);
+  }
 
   // exp2 argument = S * cs - (row maximum of S) * cs with cs = q_gs * k_gs * sm_scale * log2(e); a negative cs is
   // moved into Q so that the row maximum can be taken over the raw dot products
@@ -271,19 +277,20 @@ __global__ __launch_bounds__(64 * WAVES) void mha_nvfp4_fwd_d128_kernel(MhaArgs 
 #pragma unroll
     for (int q4 = 0; q4 < 4; ++q4) {
       const int d = fd * 32 + q4 * 8 + h * 4;  // four consecutive head dims
-      if (a.o_vec) {
+      if (a.o_vec && d + 3 < a.Dv) {
         const uint2 w = make_uint2(bf(OT[fd][4 * q4]) | (bf(OT[fd][4 * q4 + 1]) << 16),
                                    bf(OT[fd][4 * q4 + 2]) | (bf(OT[fd][4 * q4 + 3]) << 16));
         *reinterpret_cast<uint2 *>(orow + d) = w;
       } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) orow[(d + e) * a.o_d] = (uint16_t)bf(OT[fd][4 * q4 + e]);
+        for (int e = 0; e < 4; ++e)
+          if (d + e < a.Dv) orow[(d + e) * a.o_d] = (uint16_t)bf(OT[fd][4 * q4 + e]);
       }
     }
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// INT8 (QK) x FP8 (PV) attention forward, head dim 128 (lib/cuda/sm120/mha_int8_x_fp8.cu:346-975; host :979-1137;
+// INT8 (QK) x FP8 (PV) attention forward, head dims up to 128 (lib/cuda/sm120/mha_int8_x_fp8.cu:346-975; host :979-1137;
 // interface include/ac4k_kernel/ops.h:18-21):
 //   S = Q . K^T in int32 (exact); s = float(S) * ((sm_scale * log2e) * q_sf[row / q_block] * k_sf[tile])   :476,657-677
 //   kv positions past Nkv are -inf                                                                    :679-700
@@ -305,6 +312,7 @@ struct Mha8Args {
   const uint8_t *v;
   const float *q_sf, *k_sf, *v_sf;
   int64_t H, Nq, Nkv, Nkv16, nqb, nkb;  // stored kv length of V (16), scales per head of Q and K
+  int Dp, Dv, Dvp;                      // bytes of a Q / K row (head dim padded to 16), rows of V, scales of V per head (16)
   int q_block;
   float sm_scale;
   int o_vec;
@@ -319,7 +327,7 @@ constexpr int MHA8_LDS_BYTES = 4 * MHA8_TILE_LDS;  // K tiles j & 1, then V tile
 constexpr float MHA8_EXP_OFFSET = 7.5f;
 
 template <int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_d128_kernel(Mha8Args a) {
+__global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_kernel(Mha8Args a) {
   constexpr int PARTS = 8 / WAVES, PROWS = 128 / PARTS;
   extern __shared__ __attribute__((aligned(16))) uint8_t mha_lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
@@ -328,8 +336,10 @@ __global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_d128_kernel(Mha
   const int64_t m = (int64_t)blockIdx.x * (32 * WAVES) + wave * 32 + r;  // this lane's query row
   const int64_t mq = m < a.Nq ? m : a.Nq - 1;                            // rows past Nq read the last row; never stored
 
-  const int8_t *k_src = a.k + bh * a.Nkv * MHA_D + sq * 32;
-  const uint8_t *v_src = a.v + (bh * MHA_D + srow) * a.Nkv16 + sq * 32;
+  // head dims below 128: the missing columns of Q and K and the missing rows of V are zeros
+  const int8_t *k_src = a.k + bh * a.Nkv * a.Dp + sq * 32;
+  const uint8_t *v_src = a.v + (bh * a.Dv + srow) * a.Nkv16 + sq * 32;
+  const bool kc0 = sq * 32 < a.Dp, kc1 = sq * 32 + 16 < a.Dp;
   struct Fetch {
     uint4 k0, k1, v0, v1;
   };
@@ -341,13 +351,14 @@ __global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_d128_kernel(Mha
       const int64_t n = n0 + srow + p * PROWS;
       f.k0 = f.k1 = f.v0 = f.v1 = make_uint4(0, 0, 0, 0);
       if (n < a.Nkv) {
-        const uint4 *src = reinterpret_cast<const uint4 *>(k_src + n * MHA_D);
-        f.k0 = src[0];
-        f.k1 = src[1];
+        const uint4 *src = reinterpret_cast<const uint4 *>(k_src + n * a.Dp);
+        if (kc0) f.k0 = src[0];
+        if (kc1) f.k1 = src[1];
       }
       const uint8_t *vs = v_src + p * PROWS * a.Nkv16 + n0;
-      if (n0 + sq * 32 < a.Nkv16) f.v0 = *reinterpret_cast<const uint4 *>(vs);
-      if (n0 + sq * 32 + 16 < a.Nkv16) f.v1 = *reinterpret_cast<const uint4 *>(vs + 16);
+      const bool vrow = srow + p * PROWS < a.Dv;
+      if (vrow && n0 + sq * 32 < a.Nkv16) f.v0 = *reinterpret_cast<const uint4 *>(vs);
+      if (vrow && n0 + sq * 32 + 16 < a.Nkv16) f.v1 = *reinterpret_cast<const uint4 *>(vs + 16);
     }
   };
   // K rows as they are; V: the thread's two 16-groups (2 sq, 2 sq + 1) regrouped so that the 8-byte pieces of lane
@@ -368,8 +379,10 @@ __global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_d128_kernel(Mha
   // Q of the lane's row: the 16 bytes [32 s + 16 h, +16) of k-step s, kept for the whole kernel
   i32x4 QF[4];
 #pragma unroll
-  for (int s4 = 0; s4 < 4; ++s4)
-    QF[s4] = *reinterpret_cast<const i32x4 *>(a.q + (bh * a.Nq + mq) * MHA_D + s4 * 32 + h * 16);
+  for (int s4 = 0; s4 < 4; ++s4) {
+    QF[s4] = (i32x4)(0);
+    if (s4 * 32 + h * 16 < a.Dp) QF[s4] = *reinterpret_cast<const i32x4 *>(a.q + (bh * a.Nq + mq) * a.Dp + s4 * 32 + h * 16);
+  }
   const float qs = (a.sm_scale * MHA_LOG2E) * a.q_sf[bh * a.nqb + mq / a.q_block];
 
   float m_run = -__builtin_inff(), l_run = 0.0f;  // running maximum (held 7.5 below the row maximum) and row sum
@@ -486,23 +499,25 @@ __global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_d128_kernel(Mha
   // ---- O = O * ((1 / l) * v_sf[d]) -> bf16
   if (m >= a.Nq) return;
   const float rl = 1.0f / l_run;
-  const float *vsf = a.v_sf + bh * MHA_D;
+  const float *vsf = a.v_sf + bh * a.Dvp;
   uint16_t *orow = a.O + b * a.o_b + head * a.o_h + m * a.o_n;
 #pragma unroll
   for (int fd = 0; fd < 4; ++fd)
 #pragma unroll
     for (int q4 = 0; q4 < 4; ++q4) {
       const int d = fd * 32 + q4 * 8 + h * 4;  // four consecutive head dims
-      const float4 sv = *reinterpret_cast<const float4 *>(vsf + d);
+      if (d >= a.Dv) continue;
+      const float4 sv = *reinterpret_cast<const float4 *>(vsf + d);  // the scale row is padded to 16
       const float sc[4] = {rl * sv.x, rl * sv.y, rl * sv.z, rl * sv.w};
       uint32_t o4[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) o4[e] = __builtin_bit_cast(uint16_t, (__bf16)(OT[fd][4 * q4 + e] * sc[e]));
-      if (a.o_vec) {
+      if (a.o_vec && d + 3 < a.Dv) {
         *reinterpret_cast<uint2 *>(orow + d) = make_uint2(o4[0] | (o4[1] << 16), o4[2] | (o4[3] << 16));
       } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) orow[(d + e) * a.o_d] = (uint16_t)o4[e];
+        for (int e = 0; e < 4; ++e)
+          if (d + e < a.Dv) orow[(d + e) * a.o_d] = (uint16_t)o4[e];
       }
     }
 }
@@ -549,7 +564,8 @@ extern "C" __attribute__((visibility("default"))) int ac4k_mha_nvfp4_fwd(
                (long long)B, (long long)H, (long long)Nq, (long long)Nkv);
   AC4K_REQUIRE(Dqk % 16 == 0, "Dqk must be multiple of 16");
   AC4K_REQUIRE(Dqk <= 128 && Dv <= 128, "Dqk and Dv must not exceed 128");
-  AC4K_REQUIRE(Dqk == MHA_D && Dv == MHA_D, "this build of the attention kernel takes head dim 128 only (Dqk=%lld Dv=%lld)",
+  AC4K_REQUIRE(Dqk % 64 == 0 && Dqk >= 64 && Dv >= 1,
+               "Dqk must be 64 or 128 (packed rows of whole 64-chunks, as the quantizer writes them) and Dv positive (Dqk=%lld Dv=%lld)",
                (long long)Dqk, (long long)Dv);
   AC4K_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) == 0 && (((uintptr_t)q_sf | (uintptr_t)k_sf | (uintptr_t)v_sf) & 3) == 0,
                "q, k, v must be 16-byte aligned and the scale tensors 4-byte aligned");
@@ -558,11 +574,12 @@ extern "C" __attribute__((visibility("default"))) int ac4k_mha_nvfp4_fwd(
   MhaArgs a{static_cast<uint16_t *>(O), o_b_stride, o_h_stride, o_n_stride, o_d_stride,
             static_cast<const uint8_t *>(q), static_cast<const uint8_t *>(k), static_cast<const uint8_t *>(v),
             static_cast<const uint8_t *>(q_sf), static_cast<const uint8_t *>(k_sf), static_cast<const uint8_t *>(v_sf),
-            q_gs, k_gs, v_gs, H, Nq, Nkv, align_up(Nq, 16), align_up(Nkv, 16), align_up(Nkv, 64), sm_scale,
+            q_gs, k_gs, v_gs, H, Nq, Nkv, align_up(Nq, 16), align_up(Nkv, 16), align_up(Nkv, 64), (int)(Dqk / 64), (int)Dv,
+            (int)align_up(Dv, 16), sm_scale,
             (o_d_stride == 1 && ((uintptr_t)O & 7) == 0 && o_b_stride % 4 == 0 && o_h_stride % 4 == 0 && o_n_stride % 4 == 0) ? 1 : 0};
   // 256 query rows per workgroup unless that leaves most of the GPU's 256 CUs without one
   const bool wide = ceil_div(Nq, 256) * H * B >= 192 || ceil_div(Nq, 128) * H * B <= ceil_div(Nq, 256) * H * B;
-  auto kern = wide ? mha_nvfp4_fwd_d128_kernel<8> : mha_nvfp4_fwd_d128_kernel<4>;
+  auto kern = wide ? mha_nvfp4_fwd_kernel<8> : mha_nvfp4_fwd_kernel<4>;
   {  // more than 64 KB of dynamic LDS has to be allowed once per device and kernel
     static std::atomic<uint32_t> lds_done[2] = {{0}, {0}};
     int dev = 0;
@@ -595,8 +612,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_mha_int8_x_fp8_fwd(
   AC4K_REQUIRE(q_quantize_block_size == 32 || q_quantize_block_size == 64, "q_quantize_block_size must be 32 or 64 (got %d)",
                q_quantize_block_size);
   AC4K_REQUIRE(k_quantize_block_size == 128, "k_quantize_block_size must be 128 (got %d)", k_quantize_block_size);
-  AC4K_REQUIRE(Dqk == MHA_D && Dv == MHA_D, "this build of the attention kernel takes head dim 128 only (Dqk=%lld Dv=%lld)",
-               (long long)Dqk, (long long)Dv);
+  AC4K_REQUIRE(Dqk >= 16 && Dv >= 1, "Dqk and Dv must be positive");
   AC4K_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)v_sf) & 15) == 0,
                "q, k, v and v_sf must be 16-byte aligned");
   AC4K_REQUIRE(H <= 65535 && B <= 65535 && ceil_div(Nq, 128) < (1ll << 31), "problem too large");
@@ -604,10 +620,10 @@ extern "C" __attribute__((visibility("default"))) int ac4k_mha_int8_x_fp8_fwd(
   Mha8Args a{static_cast<uint16_t *>(O), o_b_stride, o_h_stride, o_n_stride, o_d_stride,
              static_cast<const int8_t *>(q), static_cast<const int8_t *>(k), static_cast<const uint8_t *>(v),
              q_sf, k_sf, v_sf, H, Nq, Nkv, align_up(Nkv, 16), ceil_div(Nq, q_quantize_block_size), ceil_div(Nkv, 128),
-             q_quantize_block_size, sm_scale,
+             (int)Dqk, (int)Dv, (int)align_up(Dv, 16), q_quantize_block_size, sm_scale,
              (o_d_stride == 1 && ((uintptr_t)O & 7) == 0 && o_b_stride % 4 == 0 && o_h_stride % 4 == 0 && o_n_stride % 4 == 0) ? 1 : 0};
   const bool wide = ceil_div(Nq, 256) * H * B >= 192 || ceil_div(Nq, 128) * H * B <= ceil_div(Nq, 256) * H * B;
-  auto kern = wide ? mha_int8_x_fp8_fwd_d128_kernel<8> : mha_int8_x_fp8_fwd_d128_kernel<4>;
+  auto kern = wide ? mha_int8_x_fp8_fwd_kernel<8> : mha_int8_x_fp8_fwd_kernel<4>;
   {  // more than 64 KB of dynamic LDS has to be allowed once per device and kernel
     static std::atomic<uint32_t> lds_done[2] = {{0}, {0}};
     int dev = 0;

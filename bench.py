@@ -403,7 +403,7 @@ def bench_quantize_layouts(ops, steps, warmup):
 
 
 def bench_attention(ops, B, N, H, D, steps, warmup, check=True, precision="nvfp4"):
-    """Attention forward (head dim 128), precision "nvfp4" or "int8+fp8e4m3": flops = 4 B H N^2 D as in
+    """Attention forward, precision "nvfp4" or "int8+fp8e4m3": flops = 4 B H N^2 D as in
     the reference's test/test_attention_tflops.py:31-33; the kernel alone on pre-quantized operands and the whole
     attention() call (its quantizers + kernel).  Check: cosine similarity and elementwise distance to torch's
     scaled_dot_product_attention on the GPU, at the tolerance of test/test_attention_bench.py:19-66 (nvfp4: cosine

@@ -217,7 +217,8 @@ int ac4k_linear_nvfp4_fused_bf16(void *D, int d_dtype, const void *X, void *X_q,
  * v_sf [B,H,align_up(Nkv,64)/64,align_up(Dv,16),4]; the three global scales are device scalars;
  * O bf16 [B,H,Nq,Dv] addressed through its four element strides (the reference passes a permuted view).
  * The attention probabilities are re-quantized to NVFP4 per 16-block with the global scale 1/2688, as in
- * mha_nvfp4.cu:248-319.  Head dim 128 only (Dqk == Dv == 128; the reference takes any multiple of 16 up to 128). */
+ * mha_nvfp4.cu:248-319.  Dqk = 2 * (packed row bytes) must be 64 or 128 (the quantizer pads packed rows to whole 64-chunks), Dv any
+ * number up to 128. */
 int ac4k_mha_nvfp4_fwd(void *O, int64_t o_b_stride, int64_t o_h_stride, int64_t o_n_stride,
                        int64_t o_d_stride, const void *q, const void *q_sf, const float *q_gs,
                        const void *k, const void *k_sf, const float *k_gs, const void *v,
@@ -232,7 +233,8 @@ int ac4k_mha_nvfp4_fwd(void *O, int64_t o_b_stride, int64_t o_h_stride, int64_t 
  * (quantize(v, 3, N_dim, swizzle=True, max_scale=2.25, precision="fp8e4m3")), v_sf fp32 [B,H,align_up(Dv,16)];
  * O bf16 [B,H,Nq,Dv] addressed through its four element strides.  The probabilities are held up to 2^7.5 and
  * converted to e4m3 per element (mha_int8_x_fp8.cu:718-736,323-345); P V accumulates in fp32 (the reference's MMA
- * accumulates each kv tile in fp16).  Head dim 128 only (the reference takes any multiple of 16 up to 128). */
+ * accumulates each kv tile in fp16).  Dqk: a multiple of 16 up to 128 (the quantizer pads the head dim to 16), Dv any
+ * number up to 128. */
 int ac4k_mha_int8_x_fp8_fwd(void *O, int64_t o_b_stride, int64_t o_h_stride, int64_t o_n_stride,
                             int64_t o_d_stride, const void *q, const float *q_sf,
                             int q_quantize_block_size, const void *k, const float *k_sf,

@@ -1,4 +1,4 @@
-"""GPU parity of the NVFP4 attention forward (head dim 128): the HIP kernel, through the C ABI, against the
+"""GPU parity of the NVFP4 attention forward (head dims up to 128): the HIP kernel, through the C ABI, against the
 CPU oracle on the same packed operands, and the whole `attention()` call against an fp32 attention at the
 tolerance of the reference's test (test/test_attention_bench.py:19-66,178-191)."""
 import math
@@ -35,7 +35,9 @@ def sdpa_fp32(q, k, v, layout):
 CASES = [(1, 256, 1, 128, "BNHD"), (1, 64, 1, 128, "BNHD"), (2, 100, 3, 128, "BHND"), (1, 33, 2, 128, "BNHD"),
          (1, 300, 1, 128, "BNHD"), (1, 129, 2, 128, "BHND"), (2, 1, 1, 128, "BNHD"), (1, 1000, 4, 128, "BNHD"),
          # enough (query block, head) pairs that the kernel takes 256 query rows per workgroup, ragged last block
-         (1, 300, 200, 128, "BHND"), (2, 513, 100, 128, "BNHD")]
+         (1, 300, 200, 128, "BHND"), (2, 513, 100, 128, "BNHD"),
+         # head dims below 128: 64 (one 64-chunk), 100 and 40 (the quantizer pads the packed rows to 128 / 64)
+         (1, 200, 2, 64, "BNHD"), (2, 150, 3, 100, "BHND"), (1, 77, 2, 40, "BNHD")]
 
 
 @pytest.mark.parametrize("B,N,H,D,layout", CASES)
@@ -86,7 +88,7 @@ def test_attention_argument_checks():
         o.attention(q, q, q, precision="fp16")
     with pytest.raises(AssertionError):
         o.attention(q.float(), q, q)
-    q64 = make_input((1, 16, 1, 64), seed=1).cuda()
+    q192 = make_input((1, 16, 1, 192), seed=1).cuda()
     for precision in ("nvfp4", "int8+fp8e4m3"):
-        with pytest.raises(RuntimeError, match="head dim 128"):  # head dim 64: refused by this build with a message
-            o.attention(q64, q64, q64, precision=precision)
+        with pytest.raises(RuntimeError, match="less than 128"):  # the reference's limit (mha_nvfp4.cu:927-929)
+            o.attention(q192, q192, q192, precision=precision)

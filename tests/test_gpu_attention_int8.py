@@ -1,4 +1,4 @@
-"""GPU parity of the INT8 (QK) x FP8 (PV) attention forward (head dim 128) and of the per-token-block int8
+"""GPU parity of the INT8 (QK) x FP8 (PV) attention forward (head dims up to 128) and of the per-token-block int8
 quantizer in front of it: the HIP kernels, through the C ABI, against the CPU oracle on the same operands, and
 the whole `attention(..., precision="int8+fp8e4m3")` call against an fp32 attention at the tolerance of the
 reference's test (test/test_attention_bench.py:69-177: atol 0.2, rtol 1e-2, cosine similarity > 0.99)."""
@@ -53,7 +53,9 @@ def test_token_block_quantizer_bit_exact(shape, layout, block):
     assert torch.equal(s.cpu(), es) and torch.equal(y.cpu(), ey)
 
 
-CASES = [(1, 256, 1, 128, "BNHD"), (1, 100, 1, 128, "BNHD"), (2, 111, 2, 128, "BHND"), (1, 444, 1, 128, "BNHD"),
+# the first rows are the reference's own test shapes (test/test_attention_bench.py:69-177), head dims 12 to 128
+CASES = [(1, 256, 1, 128, "BNHD"), (1, 100, 1, 128, "BNHD"), (2, 111, 2, 100, "BHND"), (1, 444, 1, 88, "BNHD"),
+         (11, 100, 12, 12, "BNHD"), (11, 100, 12, 65, "BNHD"), (2, 330, 3, 100, "BNHD"), (2, 111, 2, 128, "BHND"),
          (1, 129, 2, 128, "BHND"), (2, 1, 1, 128, "BNHD"), (1, 1000, 4, 128, "BNHD"),
          # enough (query block, head) pairs that the kernel takes 256 query rows per workgroup, ragged last block
          (1, 300, 200, 128, "BHND")]
@@ -108,6 +110,6 @@ def test_error_behaviour():
         b.mha_int8_x_fp8_fwd(o, q.float(), sf, 64, q, sf, 128, v, v_sf, 1.0)
     with pytest.raises(RuntimeError, match="k_quantize_block_size"):
         b.mha_int8_x_fp8_fwd(o, q, sf, 64, q, torch.ones((1, 1, 1), device="cuda"), 64, v, v_sf, 1.0)
-    with pytest.raises(RuntimeError, match="head dim 128"):
-        q64 = torch.zeros((1, 1, 16, 64), dtype=torch.int8, device="cuda")
-        b.mha_int8_x_fp8_fwd(o, q64, sf, 64, q64, sf, 128, v, v_sf, 1.0)
+    with pytest.raises(RuntimeError, match="multiple of 16"):
+        q24 = torch.zeros((1, 1, 16, 24), dtype=torch.int8, device="cuda")
+        b.mha_int8_x_fp8_fwd(o, q24, sf, 64, q24, sf, 128, v, v_sf, 1.0)
