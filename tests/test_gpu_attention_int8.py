@@ -113,3 +113,25 @@ def test_error_behaviour():
     with pytest.raises(RuntimeError, match="multiple of 16"):
         q24 = torch.zeros((1, 1, 16, 24), dtype=torch.int8, device="cuda")
         b.mha_int8_x_fp8_fwd(o, q24, sf, 64, q24, sf, 128, v, v_sf, 1.0)
+
+
+@pytest.mark.parametrize("precision", ["int8+fp8e4m3", "nvfp4"])
+def test_reference_long_sequence_shape(precision):
+    """The long shape of the reference's test list, (1, 75600, 1, 128) BNHD (test/test_attention_bench.py:69-77), for
+    both precisions, against an fp32 attention evaluated on the GPU in blocks of query rows, at the reference's
+    tolerance."""
+    B, N, H, D = 1, 75600, 1, 128
+    g = torch.Generator(device="cuda").manual_seed(9567)
+    q, k, v = (torch.empty((B, N, H, D), dtype=torch.float32, device="cuda").normal_(generator=g).to(torch.bfloat16)
+               for _ in range(3))
+    o = ops().attention(q, k, v, layout="BNHD", precision=precision)
+    kf, vf = k[0, :, 0].float(), v[0, :, 0].float()
+    ref = torch.empty((N, D), dtype=torch.float32, device="cuda")
+    for m0 in range(0, N, 4096):
+        s = (q[0, m0:m0 + 4096, 0].float() @ kf.t()) / math.sqrt(D)
+        ref[m0:m0 + 4096] = torch.softmax(s, dim=-1) @ vf
+    got = o[0, :, 0].float()
+    cos = torch.nn.functional.cosine_similarity(got.flatten(), ref.flatten(), dim=0).item()
+    rtol, stol = (1e-2, 0.99) if precision == "int8+fp8e4m3" else (1e-1, 0.98)
+    assert cos > stol, cos
+    torch.testing.assert_close(got, ref, atol=2e-1, rtol=rtol)
