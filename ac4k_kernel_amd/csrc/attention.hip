@@ -24,6 +24,7 @@
 #include "ac4k_common.h"
 
 #include <atomic>
+#include <type_traits>
 
 namespace ac4k {
 
@@ -396,8 +397,10 @@ __global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_kernel(Mha8Args
   fetch(0, nxt);
   stage(0, nxt);
   __syncthreads();
-  int buf = 0;
-  for (int64_t n0 = 0; n0 < a.Nkv; n0 += 128, buf ^= 1) {
+  // one kv tile; TAIL: the last, partial one, whose positions past Nkv are masked (a copy of the code of its own:
+  // as a branch inside one body the masks were turned into selects that every tile paid for)
+  auto tile_step = [&](auto tail_tag, int64_t n0, int buf) {
+    constexpr bool tail = decltype(tail_tag)::value;
     fetch(n0 + 128, nxt);  // the next tile travels while this one is multiplied (zeros past the end)
     const uint8_t *kb = mha_lds + buf * MHA8_TILE_LDS + r * MHA8_PITCH + h * 16;
     const uint8_t *vb = mha_lds + (2 + buf) * MHA8_TILE_LDS + r * MHA8_PITCH + h * 16;
@@ -420,13 +423,13 @@ __global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_kernel(Mha8Args
     for (int f = 0; f < 4; ++f)
 #pragma unroll
       for (int e = 0; e < 16; ++e) ST[f][e] = (float)SI[f][e];
-    const bool tail = n0 + 128 > a.Nkv;
+    const int left = (int)(a.Nkv - n0) - h * 4;  // kv positions of this tile that exist, seen from the lane's first one
     if (tail) {  // positions past Nkv take no part in the maximum
 #pragma unroll
       for (int f = 0; f < 4; ++f)
 #pragma unroll
         for (int e = 0; e < 16; ++e)
-          if (n0 + f * 32 + (e >> 2) * 8 + h * 4 + (e & 3) >= a.Nkv) ST[f][e] = -__builtin_inff();
+          if (f * 32 + (e >> 2) * 8 + (e & 3) >= left) ST[f][e] = -__builtin_inff();
     }
     // the maximum of s = float(S) * qk is taken over float(S): qk >= 0 keeps the order, qk < 0 reverses it
     float hi = -__builtin_inff(), lo = __builtin_inff();
@@ -435,6 +438,7 @@ __global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_kernel(Mha8Args
 #pragma unroll
       for (int e = 0; e < 16; ++e) hi = __builtin_fmaxf(hi, ST[f][e]);
     if (qk < 0.0f) {
+      asm volatile("" ::: "memory");
 #pragma unroll
       for (int f = 0; f < 4; ++f)
 #pragma unroll
@@ -457,7 +461,7 @@ __global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_kernel(Mha8Args
       for (int f = 0; f < 4; ++f)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          if (n0 + f * 32 + (e >> 2) * 8 + h * 4 + (e & 3) >= a.Nkv) ST[f][e] = 0.0f;
+          if (f * 32 + (e >> 2) * 8 + (e & 3) >= left) ST[f][e] = 0.0f;
           lsum += ST[f][e];
         }
     }
@@ -494,7 +498,11 @@ __global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_kernel(Mha8Args
     }
     stage(buf ^ 1, nxt);
     __syncthreads();
-  }
+  };
+  int buf = 0;
+  int64_t n0 = 0;
+  for (; n0 + 128 <= a.Nkv; n0 += 128, buf ^= 1) tile_step(std::false_type{}, n0, buf);
+  if (n0 < a.Nkv) tile_step(std::true_type{}, n0, buf);
 
   // ---- O = O * ((1 / l) * v_sf[d]) -> bf16
   if (m >= a.Nq) return;
@@ -528,13 +536,51 @@ __global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_kernel(Mha8Args
 __global__ __launch_bounds__(256) void quantize_int8_token_block_kernel(int8_t *__restrict__ y, float *__restrict__ scale,
                                                                         const uint16_t *__restrict__ x, int64_t s_b,
                                                                         int64_t s_h, int64_t s_n, int64_t H, int64_t N,
-                                                                        int D, int Dp, int block) {
+                                                                        int D, int Dp, int block, int vec) {
   __shared__ uint32_t wmax[4];
   const int64_t nb = gridDim.x, blk = blockIdx.x, head = blockIdx.y, b = blockIdx.z;
   const int64_t n0 = blk * block;
   const int rows = (int)((N - n0) < block ? (N - n0) : block);
   const uint16_t *src = x + b * s_b + head * s_h + n0 * s_n;
+  int8_t *dst = y + ((b * H + head) * N + n0) * Dp;
   uint32_t mx = 0;
+  // rows of whole 16-byte vectors (D % 8 == 0, aligned), at most eight vectors per thread: the block is read once,
+  // into registers
+  const int vpr = D / 8, nvec = rows * vpr;
+  if (vec && nvec <= 8 * 256) {
+    uint4 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = threadIdx.x + j * 256;
+      v[j] = make_uint4(0, 0, 0, 0);
+      if (i < nvec) v[j] = ld_stream_u4(src + (int64_t)(i / vpr) * s_n + (i % vpr) * 8);
+      mx = umax32(mx, absmax_bf16x8(v[j]));
+    }
+    mx = group_umax<64>(mx);
+    if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = mx;
+    __syncthreads();
+    mx = umax32(umax32(wmax[0], wmax[1]), umax32(wmax[2], wmax[3]));
+    const float sc = bf16_bits_to_f32(mx) / 127.0f;
+    if (threadIdx.x == 0) scale[(b * H + head) * nb + blk] = sc;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = threadIdx.x + j * 256;
+      if (i >= nvec) continue;
+      const uint32_t w[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+      uint32_t o2[2] = {0, 0};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float xe = bf16_bits_to_f32((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+        const int q = sc != 0.0f ? (int)(xe / sc) : 0;  // toward zero; |q| <= 127 up to rounding
+        o2[e >> 2] |= ((uint32_t)q & 0xffu) << (8 * (e & 3));
+      }
+      *reinterpret_cast<uint2 *>(dst + (int64_t)(i / vpr) * Dp + (i % vpr) * 8) = make_uint2(o2[0], o2[1]);
+    }
+    if (Dp != D) {  // D % 16 == 8: eight pad columns per row
+      for (int rr = threadIdx.x; rr < rows; rr += 256) *reinterpret_cast<uint2 *>(dst + (int64_t)rr * Dp + D) = make_uint2(0, 0);
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < rows * D; i += 256) mx = umax32(mx, src[(int64_t)(i / D) * s_n + i % D] & 0x7fffu);
   mx = group_umax<64>(mx);
   if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = mx;
@@ -542,7 +588,6 @@ __global__ __launch_bounds__(256) void quantize_int8_token_block_kernel(int8_t *
   mx = umax32(umax32(wmax[0], wmax[1]), umax32(wmax[2], wmax[3]));
   const float sc = bf16_bits_to_f32(mx) / 127.0f;
   if (threadIdx.x == 0) scale[(b * H + head) * nb + blk] = sc;
-  int8_t *dst = y + ((b * H + head) * N + n0) * Dp;
   for (int i = threadIdx.x; i < rows * Dp; i += 256) {
     const int rr = i / Dp, c = i % Dp;
     float q = 0.0f;
@@ -654,6 +699,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_quantize_int8_token_b
   AC4K_REQUIRE(H <= 65535 && B <= 65535 && ceil_div(N, (int64_t)block) < (1ll << 31), "problem too large");
   hipLaunchKernelGGL(quantize_int8_token_block_kernel, dim3((unsigned)ceil_div(N, (int64_t)block), (unsigned)H, (unsigned)B),
                      dim3(256), 0, (hipStream_t)stream, static_cast<int8_t *>(y), scale, static_cast<const uint16_t *>(x), s_b,
-                     s_h, s_n, H, N, (int)D, (int)align_up(D, 16), block);
+                     s_h, s_n, H, N, (int)D, (int)align_up(D, 16), block,
+                     (D % 8 == 0 && ((uintptr_t)x & 15) == 0 && s_b % 8 == 0 && s_h % 8 == 0 && s_n % 8 == 0) ? 1 : 0);
   return check_launch("ac4k_quantize_int8_token_block_bf16");
 }

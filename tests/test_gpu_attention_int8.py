@@ -37,7 +37,8 @@ def sdpa_fp32(q, k, v, layout):
 
 
 @pytest.mark.parametrize("shape,layout,block", [((1, 100, 1, 128), "BNHD", 64), ((2, 3, 333, 128), "BHND", 128),
-                                                 ((1, 64, 2, 100), "BNHD", 32), ((2, 2, 17, 12), "BHND", 16)])
+                                                 ((1, 64, 2, 100), "BNHD", 32), ((2, 2, 17, 12), "BHND", 16),
+                                                 ((1, 200, 3, 88), "BNHD", 64)])
 def test_token_block_quantizer_bit_exact(shape, layout, block):
     """Scales and int8 values equal the oracle's bit for bit, over ragged last blocks, head dims that are padded
     to 16, both layouts, an all-zero block and an outlier."""
