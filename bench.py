@@ -531,7 +531,15 @@ def run_traffic(ops):
     o = torch.empty((1, 40, 8192, 128), dtype=torch.bfloat16, device="cuda")
     for _ in range(3):
         ops.mha_nvfp4_fwd(o, *qq, *kq, *vq, 1.0 / math.sqrt(128))
-    del q, k_, v, qq, kq, vq, o
+    # the int8 x fp8 attention kernel on the same tensors, with its quantizers in front
+    import importlib
+    front = importlib.import_module("ac4k_kernel_amd.ops.attention")
+    q8, q_sf = front._int8_quantize(q, "BNHD", 1, BLOCK_SIZE=64)
+    k8, k_sf = front._int8_quantize(k_, "BNHD", 1, BLOCK_SIZE=128)
+    v8, v_sf = ops.quantize(v, 3, 1, swizzle=True, max_scale=2.25, precision="fp8e4m3")
+    for _ in range(3):
+        ops.mha_int8_x_fp8_fwd(o, q8, q_sf, 64, k8, k_sf, 128, v8, v_sf, 1.0 / math.sqrt(128))
+    del q, k_, v, qq, kq, vq, o, q8, k8, v8
     x = make_input((8192, 4096), seed=0, outliers=True).cuda()
     for prec in ("nvfp4", "fp8e4m3", "int8"):
         for _ in range(3):
