@@ -36,7 +36,7 @@ struct MhaArgs {
   int64_t H, Nq, Nkv, Nqp, Nkvp, Nkv64;  // padded: rows of the Q / K scale planes (16), stored kv length of V (64)
   int chunks, Dv, Dvp;                   // 64-chunks of a Q / K row (1 or 2), rows of V, rows of a V scale plane (16)
   float sm_scale;
-  int o_vec;  // O rows are contiguous along d and 8-byte aligned: four head dims per store
+  int o_vec;  // O rows are contiguous along d, 16-byte aligned, Dv % 8 == 0: rows leave as 16-byte pieces
 };
 
 constexpr float MHA_LOG2E = 1.4426950408889634f;
@@ -82,6 +82,47 @@ __device__ __forceinline__ uint32_t mha_dword(const uint4 &a, const uint4 &b, in
 // both halves of the wave (lanes 0-31 and 32-63) receive op(x of the lower half, x of the upper half)
 __device__ __forceinline__ float mha_halves_max(float x) { return __builtin_fmaxf(x, __shfl_xor(x, 32, 64)); }
 __device__ __forceinline__ float mha_halves_sum(float x) { return x + __shfl_xor(x, 32, 64); }
+
+// Output of one wave: O^T in the MFMA accumulator layout (lane (r, h) owns query row r of the wave: OT[fd][e] is head
+// dim 32 fd + 8 (e >> 2) + 4 h + (e & 3)), already scaled, as bf16 bits in ob[fd][e].  Vector path (rows of O
+// contiguous along d, 16-byte aligned, Dv % 8 == 0): the wave's 32 x 128 tile goes through LDS (8448 bytes at
+// `stage`, free to use: every wave has passed the last barrier of the loop) and leaves as 16-byte pieces of
+// adjacent lanes, whole 256-byte rows; otherwise element by element.
+constexpr int MHA_OUT_PITCH = 264;  // bytes per row of the staged tile (256 + 8: bank spread)
+constexpr int MHA_OUT_LDS = 32 * MHA_OUT_PITCH;
+__device__ __forceinline__ void mha_store_rows(uint16_t *o_base, int64_t o_n, int64_t o_d, int o_vec, int64_t row0,
+                                               int64_t Nq, int Dv, int lane, uint8_t *stage,
+                                               const uint16_t (&ob)[4][16]) {
+  const int r = lane & 31, h = lane >> 5;
+  if (o_vec) {
+#pragma unroll
+    for (int fd = 0; fd < 4; ++fd)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int d = fd * 32 + q4 * 8 + h * 4;
+        *reinterpret_cast<uint2 *>(stage + r * MHA_OUT_PITCH + d * 2) =
+            make_uint2(ob[fd][4 * q4] | ((uint32_t)ob[fd][4 * q4 + 1] << 16), ob[fd][4 * q4 + 2] | ((uint32_t)ob[fd][4 * q4 + 3] << 16));
+      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      const int row = p * 4 + (lane >> 4), d = (lane & 15) * 8;
+      const uint4 w = *reinterpret_cast<const uint4 *>(stage + row * MHA_OUT_PITCH + d * 2);
+      if (row0 + row < Nq && d < Dv) *reinterpret_cast<uint4 *>(o_base + (row0 + row) * o_n + d) = w;
+    }
+  } else if (row0 + r < Nq) {
+    uint16_t *orow = o_base + (row0 + r) * o_n;
+#pragma unroll
+    for (int fd = 0; fd < 4; ++fd)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int d = fd * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
+        if (d < Dv) orow[d * o_d] = ob[fd][e];
+      }
+  }
+}
 
 constexpr int MHA_PITCH = 272;                   // bytes per decoded row in LDS: 128 fp16 + 16 (bank spread)
 constexpr int MHA_TILE_LDS = 128 * MHA_PITCH;    // one decoded operand tile: K 128 kv rows, V 128 d rows
@@ -269,25 +310,14 @@ __global__ __launch_bounds__(64 * WAVES) void mha_nvfp4_fwd_kernel(MhaArgs a) {
   // the zero-filled kv positions of the last tile each added exp(0 - m) to the row sum
   if (a.Nkv % 128 != 0) l_run -= (float)(128 - a.Nkv % 128) / __builtin_amdgcn_exp2f(ml_run);
   // ---- O = O * ((1/l) * (1/2688) * v_gs) -> bf16
-  if (m >= a.Nq) return;
   const float scale = (1.0f / l_run) * (1.0f / MHA_P_ALPHA) * (*a.v_gs);
-  uint16_t *orow = a.O + b * a.o_b + head * a.o_h + m * a.o_n;
-  auto bf = [&](float x) { return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)(x * scale)); };
+  uint16_t ob[4][16];
 #pragma unroll
   for (int fd = 0; fd < 4; ++fd)
 #pragma unroll
-    for (int q4 = 0; q4 < 4; ++q4) {
-      const int d = fd * 32 + q4 * 8 + h * 4;  // four consecutive head dims
-      if (a.o_vec && d + 3 < a.Dv) {
-        const uint2 w = make_uint2(bf(OT[fd][4 * q4]) | (bf(OT[fd][4 * q4 + 1]) << 16),
-                                   bf(OT[fd][4 * q4 + 2]) | (bf(OT[fd][4 * q4 + 3]) << 16));
-        *reinterpret_cast<uint2 *>(orow + d) = w;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (d + e < a.Dv) orow[(d + e) * a.o_d] = (uint16_t)bf(OT[fd][4 * q4 + e]);
-      }
-    }
+    for (int e = 0; e < 16; ++e) ob[fd][e] = __builtin_bit_cast(uint16_t, (__bf16)(OT[fd][e] * scale));
+  mha_store_rows(a.O + b * a.o_b + head * a.o_h, a.o_n, a.o_d, a.o_vec, (int64_t)blockIdx.x * (32 * WAVES) + wave * 32, a.Nq,
+                 a.Dv, lane, mha_lds + wave * MHA_OUT_LDS, ob);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -505,29 +535,21 @@ __global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_kernel(Mha8Args
   if (n0 < a.Nkv) tile_step(std::true_type{}, n0, buf);
 
   // ---- O = O * ((1 / l) * v_sf[d]) -> bf16
-  if (m >= a.Nq) return;
   const float rl = 1.0f / l_run;
   const float *vsf = a.v_sf + bh * a.Dvp;
-  uint16_t *orow = a.O + b * a.o_b + head * a.o_h + m * a.o_n;
+  uint16_t ob[4][16];
 #pragma unroll
   for (int fd = 0; fd < 4; ++fd)
 #pragma unroll
     for (int q4 = 0; q4 < 4; ++q4) {
-      const int d = fd * 32 + q4 * 8 + h * 4;  // four consecutive head dims
-      if (d >= a.Dv) continue;
-      const float4 sv = *reinterpret_cast<const float4 *>(vsf + d);  // the scale row is padded to 16
+      const int d = fd * 32 + q4 * 8 + h * 4;  // four consecutive head dims; the scale row is padded to 16
+      const float4 sv = d < a.Dvp ? *reinterpret_cast<const float4 *>(vsf + d) : make_float4(0.f, 0.f, 0.f, 0.f);
       const float sc[4] = {rl * sv.x, rl * sv.y, rl * sv.z, rl * sv.w};
-      uint32_t o4[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o4[e] = __builtin_bit_cast(uint16_t, (__bf16)(OT[fd][4 * q4 + e] * sc[e]));
-      if (a.o_vec && d + 3 < a.Dv) {
-        *reinterpret_cast<uint2 *>(orow + d) = make_uint2(o4[0] | (o4[1] << 16), o4[2] | (o4[3] << 16));
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (d + e < a.Dv) orow[(d + e) * a.o_d] = (uint16_t)o4[e];
-      }
+      for (int e = 0; e < 4; ++e) ob[fd][4 * q4 + e] = __builtin_bit_cast(uint16_t, (__bf16)(OT[fd][4 * q4 + e] * sc[e]));
     }
+  mha_store_rows(a.O + b * a.o_b + head * a.o_h, a.o_n, a.o_d, a.o_vec, (int64_t)blockIdx.x * (32 * WAVES) + wave * 32, a.Nq,
+                 a.Dv, lane, mha_lds + wave * MHA_OUT_LDS, ob);
 }
 
 // Per-token-block int8 quantizer in front of it (python/ac4k_kernel/ops/attention.py:18-99, a Triton kernel in the
@@ -621,7 +643,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_mha_nvfp4_fwd(
             static_cast<const uint8_t *>(q_sf), static_cast<const uint8_t *>(k_sf), static_cast<const uint8_t *>(v_sf),
             q_gs, k_gs, v_gs, H, Nq, Nkv, align_up(Nq, 16), align_up(Nkv, 16), align_up(Nkv, 64), (int)(Dqk / 64), (int)Dv,
             (int)align_up(Dv, 16), sm_scale,
-            (o_d_stride == 1 && ((uintptr_t)O & 7) == 0 && o_b_stride % 4 == 0 && o_h_stride % 4 == 0 && o_n_stride % 4 == 0) ? 1 : 0};
+            (o_d_stride == 1 && Dv % 8 == 0 && ((uintptr_t)O & 15) == 0 && o_b_stride % 8 == 0 && o_h_stride % 8 == 0 && o_n_stride % 8 == 0) ? 1 : 0};
   // 256 query rows per workgroup unless that leaves most of the GPU's 256 CUs without one
   const bool wide = ceil_div(Nq, 256) * H * B >= 192 || ceil_div(Nq, 128) * H * B <= ceil_div(Nq, 256) * H * B;
   auto kern = wide ? mha_nvfp4_fwd_kernel<8> : mha_nvfp4_fwd_kernel<4>;
@@ -666,7 +688,7 @@ extern "C" __attribute__((visibility("default"))) int ac4k_mha_int8_x_fp8_fwd(
              static_cast<const int8_t *>(q), static_cast<const int8_t *>(k), static_cast<const uint8_t *>(v),
              q_sf, k_sf, v_sf, H, Nq, Nkv, align_up(Nkv, 16), ceil_div(Nq, q_quantize_block_size), ceil_div(Nkv, 128),
              (int)Dqk, (int)Dv, (int)align_up(Dv, 16), q_quantize_block_size, sm_scale,
-             (o_d_stride == 1 && ((uintptr_t)O & 7) == 0 && o_b_stride % 4 == 0 && o_h_stride % 4 == 0 && o_n_stride % 4 == 0) ? 1 : 0};
+             (o_d_stride == 1 && Dv % 8 == 0 && ((uintptr_t)O & 15) == 0 && o_b_stride % 8 == 0 && o_h_stride % 8 == 0 && o_n_stride % 8 == 0) ? 1 : 0};
   const bool wide = ceil_div(Nq, 256) * H * B >= 192 || ceil_div(Nq, 128) * H * B <= ceil_div(Nq, 256) * H * B;
   auto kern = wide ? mha_int8_x_fp8_fwd_kernel<8> : mha_int8_x_fp8_fwd_kernel<4>;
   {  // more than 64 KB of dynamic LDS has to be allowed once per device and kernel
