@@ -330,11 +330,11 @@ __global__ __launch_bounds__(64 * WAVES) void mha_nvfp4_fwd_kernel(MhaArgs a) {
 //   O * ((1 / l) * v_sf[d]) -> bf16                                                                   :886-905
 // The product Phat . Vhat^T is accumulated in fp32 here (the reference's MMA accumulates each tile in fp16).
 // Same structure as the NVFP4 kernel above: a lane owns one query row (S^T = K . Q^T with v_mfma_i32_32x32x32_i8,
-// O^T = Vhat . Phat^T with v_mfma_f32_32x32x16_fp8_fp8), but nothing has to be decoded: the int8 rows of K and the
+// O^T = Vhat . Phat^T with v_mfma_scale_f32_32x32x64_f8f6f4 on e4m3 operands, scales 2^0), but nothing has to be decoded: the int8 rows of K and the
 // e4m3 rows of V go from global memory into LDS as they are, and from there into the MFMAs.  V is stored with the
 // 16-group swizzle of quantize(v, 3, N_dim, swizzle=True, precision="fp8e4m3"): stored byte 8 h + 4 (j >> 1) + 2 q
 // + (j & 1) of a 16-group holds kv position 8 q + 4 h + j, so the eight positions that lane half h owns in a
-// 16-group are the contiguous stored bytes [8 h, 8 h + 8): one MFMA operand.
+// 16-group are the contiguous stored bytes [8 h, 8 h + 8): four such pieces are the lane's share of one MFMA operand.
 
 struct Mha8Args {
   uint16_t *O;
@@ -350,6 +350,7 @@ struct Mha8Args {
 };
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
 typedef int i32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int MHA8_PITCH = 144;                    // bytes per 128-byte row in LDS (bank spread)
@@ -505,25 +506,27 @@ __global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_kernel(Mha8Args
 #pragma unroll
         for (int e = 0; e < 16; ++e) OT[fd][e] *= alpha;
     }
-    // ---- P -> e4m3, O^T += Vhat . Phat^T: one MFMA per 16-group G of kv positions and 32 rows of d
+    // ---- P -> e4m3, O^T += Vhat . Phat^T: one MFMA (k = 64: v_mfma_scale_f32_32x32x64_f8f6f4 with unit scales; lane
+    // half h supplies 32 of the 64 k slots) per 64 kv positions and 32 rows of d
 #pragma unroll
-    for (int pj = 0; pj < 4; ++pj) {  // pairs of 16-groups = 32-row fragments of S^T
-      long PF[2];
+    for (int j2 = 0; j2 < 2; ++j2) {
+      i32x8 PF;
 #pragma unroll
-      for (int gh = 0; gh < 2; ++gh) {  // k slots in the stored order of V: e = 8 gh + {0, 1, 4, 5, 2, 3, 6, 7}
-        const float *pe = &ST[pj][8 * gh];
+      for (int g4 = 0; g4 < 4; ++g4) {  // the lane's four 16-group halves of these 64 positions, in the stored order of V:
+        const float *pe = &ST[2 * j2 + (g4 >> 1)][8 * (g4 & 1)];  // e = 8 (g4 & 1) + {0, 1, 4, 5, 2, 3, 6, 7}
         int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(pe[0], pe[1], 0, false);
         w0 = __builtin_amdgcn_cvt_pk_fp8_f32(pe[4], pe[5], w0, true);
         int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(pe[2], pe[3], 0, false);
         w1 = __builtin_amdgcn_cvt_pk_fp8_f32(pe[6], pe[7], w1, true);
-        PF[gh] = (long)(((unsigned long)(uint32_t)w1 << 32) | (uint32_t)w0);
+        PF[2 * g4] = w0;
+        PF[2 * g4 + 1] = w1;
       }
 #pragma unroll
       for (int fd = 0; fd < 4; ++fd) {
-        const uint4 vv = *reinterpret_cast<const uint4 *>(vb + fd * 32 * MHA8_PITCH + pj * 32);
-        const long v0 = (long)(((unsigned long)vv.y << 32) | vv.x), v1 = (long)(((unsigned long)vv.w << 32) | vv.z);
-        OT[fd] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(v0, PF[0], OT[fd], 0, 0, 0);
-        OT[fd] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(v1, PF[1], OT[fd], 0, 0, 0);
+        const uint4 va = *reinterpret_cast<const uint4 *>(vb + fd * 32 * MHA8_PITCH + (2 * j2) * 32);
+        const uint4 vc = *reinterpret_cast<const uint4 *>(vb + fd * 32 * MHA8_PITCH + (2 * j2 + 1) * 32);
+        const i32x8 VF = {(int)va.x, (int)va.y, (int)va.z, (int)va.w, (int)vc.x, (int)vc.y, (int)vc.z, (int)vc.w};
+        OT[fd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(VF, PF, OT[fd], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
       }
     }
     stage(buf ^ 1, nxt);
