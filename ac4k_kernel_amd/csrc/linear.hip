@@ -962,17 +962,32 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_ksplit_kernel(LinearArgs 
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)kwlds;
   // rows: transfer t = swave * NROW + q moves rows 8 t .. 8 t + 7 of the stage (weight rows first), lane l
   // the piece of row l / 8 that belongs at position l % 8
+  // On a weight image (a.prepacked) a stage is two blocks of the row's 128-row band, 64 bytes of the row in
+  // each, pieces at p ^ ((row >> 1) & 3), and the four chunk planes of scale dwords sit behind the blocks' data.
+  const int64_t img_band_bytes = (a.K / W_BLOCK_K) * (int64_t)W_BLOCK_BYTES;
   uint32_t offR[L::NROW], ldsR[L::NROW];
   const uint8_t *srcR[L::NROW];
+  int strR[L::NROW];  // bytes per stage along k
 #pragma unroll
   for (int q = 0; q < L::NROW; ++q) {
     const int t = swave * L::NROW + q;
     const bool isW = t < BN / 8;
     const int loc = (isW ? t : t - BN / 8) * 8 + (lane >> 3);
-    const int64_t rows = isW ? a.N : a.M, first = isW ? n0 : m0;
-    const int64_t row = first + loc < rows ? loc : rows - 1 - first;  // rows past the matrix read its last row
-    offR[q] = (uint32_t)(row * kb + ((lane & 7) ^ (loc & 7)) * 16);
-    srcR[q] = uniform_ptr((isW ? a.B + n0 * kb : a.A + m0 * kb) + (int64_t)s0 * KW_ROW);
+    const int pp = (lane & 7) ^ (loc & 7);  // the piece of the stage row that belongs at this lane's position
+    if (isW && a.prepacked) {
+      const int64_t wrow = n0 + loc;  // rows past N exist in the image (zeros)
+      const int64_t band = wrow / W_BLOCK_ROWS, within = wrow % W_BLOCK_ROWS;
+      offR[q] = (uint32_t)(band * img_band_bytes + (pp >> 2) * W_BLOCK_BYTES + within * 64 + (((pp & 3) ^ ((within >> 1) & 3)) * 16));
+      srcR[q] = uniform_ptr(a.B + (int64_t)s0 * (2 * W_BLOCK_BYTES));
+      strR[q] = 2 * W_BLOCK_BYTES;
+    } else {
+      const int64_t rows = isW ? a.N : a.M, first = isW ? n0 : m0;
+      const int64_t row = first + loc < rows ? loc : rows - 1 - first;  // rows past the matrix read its last row
+      offR[q] = (uint32_t)(row * kb + pp * 16);
+      srcR[q] = uniform_ptr((isW ? a.B + n0 * kb : a.A + m0 * kb) + (int64_t)s0 * KW_ROW);
+      strR[q] = KW_ROW;
+    }
+    strR[q] = __builtin_amdgcn_readfirstlane(strR[q]);
     ldsR[q] = (uint32_t)__builtin_amdgcn_readfirstlane(t * 1024);
   }
   // scales: one transfer is 256 dwords of the [chunk][row] picture, a lane the four dwords of rows
@@ -990,10 +1005,17 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_ksplit_kernel(LinearArgs 
     const int chunk = tt * cpt + lane / (bx / 4), grp = lane % (bx / 4);
     const int64_t rows_p = isW ? a.Np : a.Mp, first = isW ? n0 : m0;
     int64_t row = first + 4 * grp;
-    row = row + 4 <= rows_p ? row : rows_p - 4;           // groups past the padded rows read the last group
-    offS = (uint32_t)((chunk * rows_p + row) * 4);
-    strideS = 4 * rows_p * 4;                             // bytes per stage: four chunk planes
-    srcS = uniform_ptr(reinterpret_cast<const uint8_t *>(isW ? a.B_sf : a.A_sf) + s0 * strideS);
+    if (isW && a.prepacked) {
+      const int64_t band = row / W_BLOCK_ROWS, within = row % W_BLOCK_ROWS;
+      offS = (uint32_t)(band * img_band_bytes + (chunk >> 1) * W_BLOCK_BYTES + W_BLOCK_DATA + (chunk & 1) * (W_BLOCK_ROWS * 4) + within * 4);
+      strideS = 2 * W_BLOCK_BYTES;
+      srcS = uniform_ptr(a.B + s0 * strideS);
+    } else {
+      row = row + 4 <= rows_p ? row : rows_p - 4;         // groups past the padded rows read the last group
+      offS = (uint32_t)((chunk * rows_p + row) * 4);
+      strideS = 4 * rows_p * 4;                           // bytes per stage: four chunk planes
+      srcS = uniform_ptr(reinterpret_cast<const uint8_t *>(isW ? a.B_sf : a.A_sf) + s0 * strideS);
+    }
     ldsS = (uint32_t)__builtin_amdgcn_readfirstlane((isW ? L::OFF_SFW : L::OFF_SFA) + tt * 1024);
   }
   // Transfer q of this wave's NPIECES for stage `st` into the ring slot at `base`.  Past the end of the range
@@ -1001,7 +1023,7 @@ __global__ __launch_bounds__(256, 1) void linear_nvfp4_ksplit_kernel(LinearArgs 
   // read the last stage again (cache hits) into slots nobody reads any more.
   auto issue_piece = [&](uint32_t base, int st, int q) {
     if (q < L::NROW)
-      dma16(srcR[q] + (int64_t)st * KW_ROW, offR[q], base, ldsR[q]);
+      dma16(srcR[q] + (int64_t)st * strR[q], offR[q], base, ldsR[q]);
     else
       dma16(srcS + st * strideS, offS, base, ldsS);
   };
@@ -2457,11 +2479,13 @@ static int64_t weight_image_bytes(int64_t N, int64_t K) {
   return ceil_div(N, W_BLOCK_ROWS) * (K / W_BLOCK_K) * W_BLOCK_BYTES;
 }
 
-// How a linear on a weight image runs: the LDS-ring kernel for decode-sized M (K % 256 == 0), the tile
-// kernel otherwise, split along K when the workspace entry point of the plain layout would split too.
+// How a linear on a weight image runs: the LDS-ring kernel for decode-sized M (K % 256 == 0), the K-split-waves
+// kernel for 32 < M <= 128, the tile kernel otherwise, split along K when the workspace entry point of the plain
+// layout would split too.
 struct PrepackedPlan {
-  bool ring;
+  bool ring, mid;
   SkinnyPlan sp;
+  KsplitPlan kp;
   TilePlan tp;
   int64_t partial_bytes;
 };
@@ -2469,12 +2493,17 @@ static bool prepacked_plan(int64_t M, int64_t N, int64_t K, PrepackedPlan &p) {
   const int64_t bytes = weight_image_bytes(N, K);
   if (M < 1 || bytes == 0 || bytes >= (1ll << 32) || (K >> 1) * 256 >= (1ll << 31) || N >= (1ll << 27)) return false;
   p.ring = M <= 32 && K % ST_BK == 0;
+  p.mid = !p.ring && ksplit_shape(M, N, K);
   if (p.ring) {
     plan_lds_ring(M, N, K, p.sp);
     p.partial_bytes = p.sp.partial_bytes;
   } else {
     p.tp = tile_plan(M, N, K, true);
     p.partial_bytes = p.tp.partial_bytes;
+    if (p.mid) {
+      p.kp = ksplit_plan(M, N, K, true);
+      p.partial_bytes = p.kp.partial_bytes;
+    }
   }
   return true;
 }
@@ -2533,9 +2562,9 @@ extern "C" __attribute__((visibility("default"))) int ac4k_linear_nvfp4_prepacke
                 static_cast<const uint32_t *>(A_sf), nullptr, A_gs, B_gs, bias,
                 M, N, K, align_up(M, 16), align_up(N, 16), 1};
   int rc;
-  if (p.tp.splits > 1) {
-    rc = dispatch_mid(la, MidPlan{false, KsplitPlan{0, 0, 1, 0}, p.tp, p.tp.partial_bytes}, static_cast<float *>(workspace),
-                      workspace_bytes, d_dtype, bias_dtype, st);
+  if (p.mid || p.tp.splits > 1) {
+    rc = dispatch_mid(la, MidPlan{p.mid, p.mid ? p.kp : KsplitPlan{0, 0, 1, 0}, p.tp, p.partial_bytes},
+                      static_cast<float *>(workspace), workspace_bytes, d_dtype, bias_dtype, st);
   } else {
     switch (d_dtype) {
       case AC4K_DTYPE_BF16: rc = dispatch_prepacked_bias<AC4K_DTYPE_BF16>(la, p.tp, bias_dtype, st); break;

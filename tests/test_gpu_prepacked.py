@@ -71,9 +71,10 @@ def check_oracle(aq, wq, bias, d, o_dtype):
     torch.testing.assert_close(d.cpu(), ref, atol=ATOL, rtol=RTOL)
 
 
-# M > 32 and N >= 128: both entry points run the packed-operand tile kernel with the same plan
+# M > 32 and N >= 128: both entry points run the same kernel with the same plan (the K-split-waves kernel for
+# M <= 128 with K % 256 == 0, the packed-operand tile kernel otherwise)
 @pytest.mark.parametrize("m,n,k", [(33, 128, 128), (130, 257, 384), (64, 130, 1280), (300, 384, 256), (129, 1000, 512),
-                                   (100, 128, 4096)])
+                                   (100, 128, 4096), (128, 1000, 768), (96, 200, 2048)])
 def test_tile_kernel_bit_identical(m, n, k):
     aq, wq, bias, d_img, d_plain = both(m, n, k, seed=m, bias_dtype=torch.float32, o_dtype=torch.float32)
     assert torch.equal(d_img, d_plain)
