@@ -136,9 +136,12 @@ struct MhaFetch {
 };
 
 // WAVES = 8 (256 query rows per workgroup, two waves per SIMD: one wave's MFMAs run under the other's vector work)
-// or 4 (128 query rows, for problems with too few workgroups of 256 rows to fill the GPU)
+// or 4 (128 query rows, for problems with too few workgroups of 256 rows to fill the GPU).  Both are compiled for 256
+// registers per lane (the launch bounds ask for two 4-wave workgroups per CU, which the LDS tile buffers do not
+// allow anyway): with 512, the compiler keeps S^T and O^T in accumulation registers and copies all of them to
+// ordinary registers and back around the softmax of every tile.
 template <int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void mha_nvfp4_fwd_kernel(MhaArgs a) {
+__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mha_nvfp4_fwd_kernel(MhaArgs a) {
   constexpr int PARTS = 8 / WAVES;  // staging shares per thread: a tile is 512 quarter rows of K and of V
   extern __shared__ __attribute__((aligned(16))) uint8_t mha_lds[];
   __shared__ float lut[128];  // exact reciprocals of the e4m3 values, as in the quantizer
@@ -359,7 +362,7 @@ constexpr int MHA8_LDS_BYTES = 4 * MHA8_TILE_LDS;  // K tiles j & 1, then V tile
 constexpr float MHA8_EXP_OFFSET = 7.5f;
 
 template <int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void mha_int8_x_fp8_fwd_kernel(Mha8Args a) {
+__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mha_int8_x_fp8_fwd_kernel(Mha8Args a) {
   constexpr int PARTS = 8 / WAVES, PROWS = 128 / PARTS;
   extern __shared__ __attribute__((aligned(16))) uint8_t mha_lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
