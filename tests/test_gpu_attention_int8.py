@@ -136,3 +136,23 @@ def test_reference_long_sequence_shape(precision):
     rtol, stol = (1e-2, 0.99) if precision == "int8+fp8e4m3" else (1e-1, 0.98)
     assert cos > stol, cos
     torch.testing.assert_close(got, ref, atol=2e-1, rtol=rtol)
+
+
+@pytest.mark.parametrize("precision", ["int8+fp8e4m3", "nvfp4"])
+def test_random_shapes(precision):
+    """Seeded random batch sizes, head counts, lengths around the tile and block boundaries, head dims and layouts,
+    some with outliers: the whole `attention()` call against the oracle."""
+    import random
+    rnd = random.Random(2024 if precision == "nvfp4" else 4202)
+    for t in range(14):
+        B, H = rnd.choice([1, 1, 2, 3]), rnd.choice([1, 2, 3, 5, 40])
+        N = rnd.choice([1, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 256, 257, 300, 511, 777])
+        if H == 40:
+            N = min(N, 300)
+        D = rnd.choice([128, 128, 64, 100, 40, 88, 96, 16, 120])
+        layout = rnd.choice(["BNHD", "BHND"])
+        shape = (B, N, H, D) if layout == "BNHD" else (B, H, N, D)
+        q, k, v = (make_input(shape, seed=s * 1000 + t, outliers=rnd.random() < 0.3) for s in (1, 2, 3))
+        o = ops().attention(q.cuda(), k.cuda(), v.cuda(), layout=layout, precision=precision)
+        ref = A.attention_nvfp4(q, k, v, layout) if precision == "nvfp4" else A.attention_int8_x_fp8(q, k, v, layout)
+        torch.testing.assert_close(o.cpu().float(), ref.float(), atol=ATOL, rtol=RTOL, msg=lambda m: f"{shape} {layout}: {m}")
