@@ -402,7 +402,10 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
   if (wave == 0) {
     const uint32_t own = group_umax<16>(red[lane & 15]);
     const uint32_t i0 = lane * 4;
-    if (timeout_ticks) __builtin_amdgcn_s_sleep(40);
+    // (bounds of up to 1 us - 100 ticks - are there to force the slow path from the host: no delay in front of the
+    // first poll, the clock looked at on every poll, so that the first workgroup to arrive finds peers missing)
+    const bool forced = timeout_ticks <= 100;
+    if (!forced) __builtin_amdgcn_s_sleep(40);
     bool ok, r0, r1, r2, r3, lane_ready = false;
     uint4 a = make_uint4(0, 0, 0, 0);
     for (uint32_t it = 0;; ++it) {  // at least one poll, whatever the timeout
@@ -417,8 +420,8 @@ __global__ __launch_bounds__(OP_THREADS) void quantize_nvfp4_onepass_kernel(
       lane_ready = (i0 + 0 >= nwg || r0) && (i0 + 1 >= nwg || r1) && (i0 + 2 >= nwg || r2) && (i0 + 3 >= nwg || r3);
       ok = __all(lane_ready);
       if (ok) break;
-      // the clock is looked at on every fourth poll only (and at once when the bound is zero)
-      if ((timeout_ticks == 0 || (it & 3) == 3) && wall_clock64() >= t_end) break;
+      // the clock is looked at on every fourth poll only (and at once when the bound is zero or forced)
+      if ((forced || (it & 3) == 3) && wall_clock64() >= t_end) break;
       __builtin_amdgcn_s_sleep(2);
     }
     // maxima that were published under this launch's tag; the others are marked for recomputation
@@ -1424,10 +1427,14 @@ extern "C" __attribute__((visibility("default"))) int ac4k_quantize_int8(void *o
 
 extern "C" __attribute__((visibility("default"))) void ac4k_set_quantize_sync_timeout_us(int64_t us) {
   ac4k::g_sync_timeout_ticks.store(us < 0 ? -1 : us * 100);
-  // a new bound starts with a clean slate: no stream keeps backing off because of waits under the old one
+  // a new bound starts with a clean slate: no stream keeps backing off because of waits under the old one,
+  // reported and acted on or reported and not yet looked at
   std::lock_guard<std::mutex> lock(ac4k::g_slot_mutex);
-  for (auto &dev : ac4k::g_slots)
-    for (auto &slot : dev) slot.backoff = 0;
+  for (int d = 0; d < ac4k::OP_MAX_DEVICES; ++d)
+    for (int i = 0; i < ac4k::OP_SLOTS; ++i) {
+      ac4k::g_slots[d][i].backoff = 0;
+      if (ac4k::g_reports[d].host) ac4k::g_slots[d][i].seen = *reinterpret_cast<volatile uint32_t *>(ac4k::g_reports[d].host + i);
+    }
 }
 
 #ifdef AC4K_ONEPASS_TIMELINE

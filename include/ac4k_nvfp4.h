@@ -83,7 +83,8 @@ int ac4k_quantize_nvfp4_bf16(void *out, void *sf, float *global_scale, const voi
  * single-launch kernel wait for each other's maxima for at most this many microseconds (default
  * 200).  A workgroup whose wait runs out - its peers were not all resident because other kernels
  * hold the GPU - recomputes the missing maxima from memory itself and finishes: slower, same bits.
- * 0 = look once, then recompute (used by the tests; not reported as a timeout); a negative value
+ * 0 = look once, then recompute (used by the tests; not reported as a timeout); 1 = the same, but
+ * reported (a wait that runs out for certain, forced from the host by the tests); a negative value
  * switches the single-launch kernel off (three launches, as under graph capture).  A wait that runs
  * out costs the bound plus a second read of the missing workgroups' shares, so a stream on which it
  * happened takes the three-launch path for its next 64 calls (see ac4k_debug_quantize_timeouts_seen);

@@ -512,8 +512,9 @@ def test_reference_bandwidth_shape_at_full_size():
 def test_single_launch_timeout_is_reported_and_backs_off():
     """A grid wait that runs out is reported to the host through mapped memory; the next calls on that stream
     take the three-launch path (64 of them), then the single launch is tried again.  The condition is forced
-    from the host with a bound of 1 us, which the launch stagger alone exceeds: every kernel still exits
-    normally, and every output equals the oracle's."""
+    from the host with a bound of 1 us: with it a workgroup looks at the clock on its first poll, more than 1 us
+    after its entry, and the first workgroup to get there finds peers missing (the launch stagger alone is longer
+    than a poll).  Every kernel still exits normally, and every output equals the oracle's."""
     from ac4k_kernel_amd import _lib
     L = _lib.load()
     x = make_input((4096, 2048), seed=77, outliers=True)
