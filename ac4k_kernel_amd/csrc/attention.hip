@@ -180,6 +180,18 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mha_nvfp4_fwd_kernel(Mh
       }
     }
   };
+  // the same for a tile that lies inside Nkv as a whole, head dims of 128: nothing to test, nothing to zero
+  auto fetch_whole = [&](int64_t n0, MhaFetch (&fs)[PARTS]) {
+#pragma unroll
+    for (int p = 0; p < PARTS; ++p) {
+      MhaFetch &f = fs[p];
+      const int64_t n = n0 + srow + p * PROWS;
+      f.k = *reinterpret_cast<const uint4 *>(k_src + n * qk_row);
+      f.ksc = *reinterpret_cast<const uint16_t *>(ksf_src + n * 4);
+      f.v = *reinterpret_cast<const uint4 *>(v_src + p * PROWS * v_row_bytes + n0 / 2);
+      f.vsc = *reinterpret_cast<const uint16_t *>(vsf_src + p * PROWS * 4 + (n0 / 64) * (a.Dvp * 4));
+    }
+  };
   // decode once per workgroup, into LDS tile buffers `buf`.  V: the thread's 32-group holds 16 stored bytes; operand
   // piece (t, hh) takes the t-th 16-bit halves of its dwords 2 hh and 2 hh + 1, and the scale of stored block hh.
   auto stage = [&](int buf, const MhaFetch (&fs)[PARTS]) {
@@ -235,8 +247,10 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mha_nvfp4_fwd_kernel(Mh
   stage(0, nxt);
   __syncthreads();
   int buf = 0;
-  for (int64_t n0 = 0; n0 < a.Nkv; n0 += 128, buf ^= 1) {
-    fetch(n0 + 128, nxt);  // the next tile's packed bytes travel while this one is multiplied (zeros past the end)
+  auto tile_step = [&](auto whole_next_tag, int64_t n0) {
+    // the next tile's packed bytes travel while this one is multiplied (zeros past the end)
+    if constexpr (decltype(whole_next_tag)::value) fetch_whole(n0 + 128, nxt);
+    else fetch(n0 + 128, nxt);
     const uint8_t *kb = mha_lds + buf * MHA_TILE_LDS + r * MHA_PITCH + h * 64;
     const uint8_t *vb = mha_lds + (2 + buf) * MHA_TILE_LDS + r * MHA_PITCH + h * 16;
     // ---- S^T = Khat . Qhat^T for the 128 kv positions of the tile (four 32-row fragments)
@@ -308,7 +322,12 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mha_nvfp4_fwd_kernel(Mh
     }
     stage(buf ^ 1, nxt);
     __syncthreads();
-  }
+  };
+  int64_t n0 = 0;
+  // tiles followed by a whole tile: the fetch without tests (worth 2 % with eight waves; with four it loses 5 %)
+  if (WAVES == 8 && a.chunks == 2 && a.Dv == 128)
+    for (; n0 + 256 <= a.Nkv; n0 += 128, buf ^= 1) tile_step(std::true_type{}, n0);
+  for (; n0 < a.Nkv; n0 += 128, buf ^= 1) tile_step(std::false_type{}, n0);
 
   // the zero-filled kv positions of the last tile each added exp(0 - m) to the row sum
   if (a.Nkv % 128 != 0) l_run -= (float)(128 - a.Nkv % 128) / __builtin_amdgcn_exp2f(ml_run);
@@ -396,6 +415,19 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mha_int8_x_fp8_fwd_kern
       if (vrow && n0 + sq * 32 + 16 < a.Nkv16) f.v1 = *reinterpret_cast<const uint4 *>(vs + 16);
     }
   };
+  // the same for a tile that lies inside Nkv as a whole, head dims of 128: nothing to test, nothing to zero
+  auto fetch_whole = [&](int64_t n0, Fetch (&fs)[PARTS]) {
+#pragma unroll
+    for (int p = 0; p < PARTS; ++p) {
+      Fetch &f = fs[p];
+      const uint4 *src = reinterpret_cast<const uint4 *>(k_src + (n0 + srow + p * PROWS) * a.Dp);
+      f.k0 = src[0];
+      f.k1 = src[1];
+      const uint8_t *vs = v_src + p * PROWS * a.Nkv16 + n0;
+      f.v0 = *reinterpret_cast<const uint4 *>(vs);
+      f.v1 = *reinterpret_cast<const uint4 *>(vs + 16);
+    }
+  };
   // K rows as they are; V: the thread's two 16-groups (2 sq, 2 sq + 1) regrouped so that the 8-byte pieces of lane
   // half hh of both are one 16-byte run at 32 sq + 16 hh
   auto stage = [&](int buf, const Fetch (&fs)[PARTS]) {
@@ -433,12 +465,24 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mha_int8_x_fp8_fwd_kern
   __syncthreads();
   // one kv tile; TAIL: the last, partial one, whose positions past Nkv are masked (a copy of the code of its own:
   // as a branch inside one body the masks were turned into selects that every tile paid for)
-  auto tile_step = [&](auto tail_tag, int64_t n0, int buf) {
+  // The scale of a K tile is asked for in front of the loads of the next tile: behind them, its wait would be a wait
+  // for all of them in the middle of the tile.  With eight waves it is loaded a whole tile ahead (the four-wave
+  // kernel has no register left for that).
+  constexpr bool KSF_AHEAD = WAVES == 8;
+  const float *ksf_src = a.k_sf + bh * a.nkb;
+  float ksf_cur = KSF_AHEAD ? ksf_src[0] : 0.0f;
+  auto tile_step = [&](auto tail_tag, auto whole_next_tag, int64_t n0, int buf) {
     constexpr bool tail = decltype(tail_tag)::value;
-    fetch(n0 + 128, nxt);  // the next tile travels while this one is multiplied (zeros past the end)
+    const int64_t t_next = n0 / 128 + 1 < a.nkb ? n0 / 128 + 1 : a.nkb - 1;
+    const float ksf_load = ksf_src[KSF_AHEAD ? t_next : n0 / 128];
+    asm volatile("" ::: "memory");  // keeps this load in front of the ones below
+    // the next tile travels while this one is multiplied (zeros past the end)
+    if constexpr (decltype(whole_next_tag)::value) fetch_whole(n0 + 128, nxt);
+    else fetch(n0 + 128, nxt);
     const uint8_t *kb = mha_lds + buf * MHA8_TILE_LDS + r * MHA8_PITCH + h * 16;
     const uint8_t *vb = mha_lds + (2 + buf) * MHA8_TILE_LDS + r * MHA8_PITCH + h * 16;
-    const float qk = qs * a.k_sf[bh * a.nkb + n0 / 128];
+    const float qk = qs * (KSF_AHEAD ? ksf_cur : ksf_load);
+    if (KSF_AHEAD) ksf_cur = ksf_load;
     // ---- S^T = K . Q^T for the 128 kv positions of the tile (four 32-row fragments)
     i32x16 SI[4];
 #pragma unroll
@@ -537,8 +581,10 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mha_int8_x_fp8_fwd_kern
   };
   int buf = 0;
   int64_t n0 = 0;
-  for (; n0 + 128 <= a.Nkv; n0 += 128, buf ^= 1) tile_step(std::false_type{}, n0, buf);
-  if (n0 < a.Nkv) tile_step(std::true_type{}, n0, buf);
+  if (a.Dp == 128 && a.Dv == 128)  // tiles followed by a whole tile: the fetch without tests
+    for (; n0 + 256 <= a.Nkv; n0 += 128, buf ^= 1) tile_step(std::false_type{}, std::true_type{}, n0, buf);
+  for (; n0 + 128 <= a.Nkv; n0 += 128, buf ^= 1) tile_step(std::false_type{}, std::false_type{}, n0, buf);
+  if (n0 < a.Nkv) tile_step(std::true_type{}, std::false_type{}, n0, buf);
 
   // ---- O = O * ((1 / l) * v_sf[d]) -> bf16
   const float rl = 1.0f / l_run;
