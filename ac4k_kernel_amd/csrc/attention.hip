@@ -428,6 +428,26 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mha_int8_x_fp8_fwd_kern
       f.v1 = *reinterpret_cast<const uint4 *>(vs + 16);
     }
   };
+  // a whole tile with smaller head dims: columns of K and rows of V that do not exist are read from a place that does
+  // (column 0, row 0) and zeroed by a mask; places and masks do not change from tile to tile
+  const int8_t *k_src0 = kc0 ? k_src : k_src - sq * 32, *k_src1 = kc1 ? k_src + 16 : k_src - sq * 32;
+  const uint32_t km0 = kc0 ? ~0u : 0u, km1 = kc1 ? ~0u : 0u;
+  auto fetch_whole_masked = [&](int64_t n0, Fetch (&fs)[PARTS]) {
+#pragma unroll
+    for (int p = 0; p < PARTS; ++p) {
+      Fetch &f = fs[p];
+      const int64_t n = n0 + srow + p * PROWS;
+      const bool vrow = srow + p * PROWS < a.Dv;
+      const uint32_t vm = vrow ? ~0u : 0u;
+      const uint8_t *vs = (vrow ? v_src + p * PROWS * a.Nkv16 : a.v + bh * a.Dv * a.Nkv16 + sq * 32) + n0;
+      const uint4 k0 = *reinterpret_cast<const uint4 *>(k_src0 + n * a.Dp), k1 = *reinterpret_cast<const uint4 *>(k_src1 + n * a.Dp);
+      const uint4 v0 = *reinterpret_cast<const uint4 *>(vs), v1 = *reinterpret_cast<const uint4 *>(vs + 16);
+      f.k0 = make_uint4(k0.x & km0, k0.y & km0, k0.z & km0, k0.w & km0);
+      f.k1 = make_uint4(k1.x & km1, k1.y & km1, k1.z & km1, k1.w & km1);
+      f.v0 = make_uint4(v0.x & vm, v0.y & vm, v0.z & vm, v0.w & vm);
+      f.v1 = make_uint4(v1.x & vm, v1.y & vm, v1.z & vm, v1.w & vm);
+    }
+  };
   // K rows as they are; V: the thread's two 16-groups (2 sq, 2 sq + 1) regrouped so that the 8-byte pieces of lane
   // half hh of both are one 16-byte run at 32 sq + 16 hh
   auto stage = [&](int buf, const Fetch (&fs)[PARTS]) {
@@ -477,7 +497,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mha_int8_x_fp8_fwd_kern
     const float ksf_load = ksf_src[KSF_AHEAD ? t_next : n0 / 128];
     asm volatile("" ::: "memory");  // keeps this load in front of the ones below
     // the next tile travels while this one is multiplied (zeros past the end)
-    if constexpr (decltype(whole_next_tag)::value) fetch_whole(n0 + 128, nxt);
+    if constexpr (decltype(whole_next_tag)::value == 1) fetch_whole(n0 + 128, nxt);
+    else if constexpr (decltype(whole_next_tag)::value == 2) fetch_whole_masked(n0 + 128, nxt);
     else fetch(n0 + 128, nxt);
     const uint8_t *kb = mha_lds + buf * MHA8_TILE_LDS + r * MHA8_PITCH + h * 16;
     const uint8_t *vb = mha_lds + (2 + buf) * MHA8_TILE_LDS + r * MHA8_PITCH + h * 16;
@@ -581,10 +602,15 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mha_int8_x_fp8_fwd_kern
   };
   int buf = 0;
   int64_t n0 = 0;
+  using FetchTested = std::integral_constant<int, 0>;
+  using FetchWhole = std::integral_constant<int, 1>;
+  using FetchWholeMasked = std::integral_constant<int, 2>;
   if (a.Dp == 128 && a.Dv == 128)  // tiles followed by a whole tile: the fetch without tests
-    for (; n0 + 256 <= a.Nkv; n0 += 128, buf ^= 1) tile_step(std::false_type{}, std::true_type{}, n0, buf);
-  for (; n0 + 128 <= a.Nkv; n0 += 128, buf ^= 1) tile_step(std::false_type{}, std::false_type{}, n0, buf);
-  if (n0 < a.Nkv) tile_step(std::true_type{}, std::false_type{}, n0, buf);
+    for (; n0 + 256 <= a.Nkv; n0 += 128, buf ^= 1) tile_step(std::false_type{}, FetchWhole{}, n0, buf);
+  else if constexpr (WAVES == 8)  // (the four-wave kernel has no registers to spare for a third copy of the loop)
+    for (; n0 + 256 <= a.Nkv; n0 += 128, buf ^= 1) tile_step(std::false_type{}, FetchWholeMasked{}, n0, buf);
+  for (; n0 + 128 <= a.Nkv; n0 += 128, buf ^= 1) tile_step(std::false_type{}, FetchTested{}, n0, buf);
+  if (n0 < a.Nkv) tile_step(std::true_type{}, FetchTested{}, n0, buf);
 
   // ---- O = O * ((1 / l) * v_sf[d]) -> bf16
   const float rl = 1.0f / l_run;
